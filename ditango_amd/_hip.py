@@ -1,0 +1,343 @@
+"""ctypes binding of ``libditango_hip.so`` (the C ABI declared in ``include/ditango_hip.h``).
+
+There is no fallback: if the library has not been built, or an entry point
+returns an error code, the call raises.  PyTorch only supplies device memory
+(``tensor.data_ptr()``) and the stream (``torch.cuda.current_stream()``).
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from pathlib import Path
+from typing import List, Optional, Sequence
+
+import torch
+
+LIB_PATH = Path(__file__).resolve().parent / "lib" / "libditango_hip.so"
+
+DT_BF16, DT_FP32 = 0, 1
+DT_LSE_BHS, DT_LSE_BSH = 0, 1
+DT_MAX_CHUNKS = 40
+DT_MAX_JOBS = 40
+DT_MAX_JOB_ENTRIES = 64
+DT_MAX_MERGE = 40
+
+c_i32, c_i64, c_f32, c_vp = ctypes.c_int32, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
+_P = ctypes.POINTER
+
+_SIGNATURES = {
+    "dt_version": (ctypes.c_int, []),
+    "dt_last_error": (ctypes.c_char_p, []),
+    "dt_attn_chunk_fwd": (ctypes.c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_i32,
+                                         c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_f32, c_vp]),
+    "dt_attn_jobs_fwd": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i64, c_i64, c_i64,
+                                        c_i32, _P(c_vp), _P(c_vp), _P(c_i32), _P(c_i64), c_i64, c_i64,
+                                        c_i32, _P(c_i32), _P(c_i32), _P(c_vp), _P(c_vp), c_f32, c_vp]),
+    "dt_attn_sched_fwd": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i64, c_i64, c_i64,
+                                         c_i32, _P(c_vp), _P(c_vp), _P(c_i32), _P(c_i64), c_i64, c_i64,
+                                         c_vp, c_vp, c_i32, c_vp, c_i64, c_vp, c_i64, c_i32, c_vp, c_vp,
+                                         c_f32, c_vp]),
+    "dt_merge_states": (ctypes.c_int, [c_i32, _P(c_vp), _P(c_vp), _P(c_i32), _P(c_i32), c_vp, c_i32, c_vp, c_i32,
+                                       c_i32, c_i32, c_i32, c_i32, c_vp]),
+    "dt_cache_store": (ctypes.c_int, [c_vp, c_i32, c_vp, c_i32, c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_vp]),
+    "dt_cache_load": (ctypes.c_int, [c_vp, c_vp, c_vp, c_i32, c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp]),
+    "dt_build_schedule": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp, c_vp]),
+    "dt_build_schedule_table": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp, c_vp]),
+    "dt_rel_l1_sums": (ctypes.c_int, [c_vp, c_vp, c_i64, c_vp, c_vp]),
+}
+
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+_lib: Optional[ctypes.CDLL] = None
+
+
+class DitangoHipError(RuntimeError):
+    pass
+
+
+def load_library(path: Optional[os.PathLike] = None) -> ctypes.CDLL:
+    """Load the built library (once) and declare the signatures.  Raises if it is absent."""
+    global _lib
+    if _lib is not None and path is None:
+        return _lib
+    p = Path(path) if path is not None else LIB_PATH
+    if not p.exists():
+        raise DitangoHipError(
+            f"{p} is missing: build it with `python -m ditango_amd.build` "
+            "(there is no non-HIP fallback for this path)")
+    lib = ctypes.CDLL(str(p))
+    for name, (res, args) in _SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    if path is None:
+        _lib = lib
+    return lib
+
+
+def _check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = load_library().dt_last_error().decode("utf-8", "replace")
+        raise DitangoHipError(f"{what} failed with code {rc}: {msg}")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.bfloat16:
+        return DT_BF16
+    if t.dtype == torch.float32:
+        return DT_FP32
+    raise DitangoHipError(f"unsupported state dtype {t.dtype} (bf16 or fp32)")
+
+
+def _require(cond: bool, msg: str) -> None:
+    if not cond:
+        raise DitangoHipError(msg)
+
+
+def _check_qkv(q: torch.Tensor, name: str = "q") -> None:
+    _require(q.is_cuda, f"{name} must live on the GPU")
+    _require(q.dtype == torch.bfloat16, f"{name} must be bf16 (got {q.dtype})")
+    _require(q.dim() == 4 and q.stride(-1) == 1, f"{name} must be [B,S,H,D] with contiguous D")
+
+
+def lse_layout_of(lse: torch.Tensor, B: int, S: int, H: int) -> int:
+    """Classify an lse tensor as [B,H,S] or [B,S,H(,1)] storage; it must be dense in that order."""
+    if lse.dim() == 4 and lse.shape[-1] == 1:
+        lse = lse.squeeze(-1)
+    _require(lse.dim() == 3 and lse.dtype == torch.float32, "lse must be fp32 with 3 (or 4, last=1) dims")
+    if tuple(lse.shape) == (B, H, S):
+        if lse.is_contiguous():
+            return DT_LSE_BHS
+        if lse.transpose(1, 2).is_contiguous():
+            return DT_LSE_BSH
+    if tuple(lse.shape) == (B, S, H):
+        if lse.is_contiguous():
+            return DT_LSE_BSH
+        if lse.transpose(1, 2).is_contiguous():
+            return DT_LSE_BHS
+    raise DitangoHipError(f"lse of shape {tuple(lse.shape)} / strides {lse.stride()} is not a dense [B,H,S] or [B,S,H]")
+
+
+# ---------------------------------------------------------------------------------------------
+# K1: chunk attention
+# ---------------------------------------------------------------------------------------------
+
+def attn_chunk_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_scale: float = 0.0,
+                   out: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None):
+    """(out bf16 [B,Sq,H,D], lse fp32 [B,H,Sq]) of q against one KV chunk."""
+    lib = load_library()
+    _check_qkv(q, "q"); _check_qkv(k, "k"); _check_qkv(v, "v")
+    B, Sq, H, D = q.shape
+    Sk = k.shape[1]
+    _require(k.shape == v.shape and k.shape[0] == B and k.shape[2] == H and k.shape[3] == D, "k/v shape mismatch")
+    _require(k.stride() == v.stride(), "k and v must share strides")
+    if out is None:
+        out = torch.empty((B, Sq, H, D), dtype=torch.bfloat16, device=q.device)
+    if lse is None:
+        lse = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device)
+    _require(out.is_contiguous() and lse.is_contiguous(), "out/lse must be contiguous")
+    rc = lib.dt_attn_chunk_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
+                               B, Sq, Sk, H, D, q.stride(0), q.stride(1), q.stride(2),
+                               k.stride(0), k.stride(1), k.stride(2), float(softmax_scale), _stream())
+    _check(rc, "dt_attn_chunk_fwd")
+    return out, lse
+
+
+class ChunkTable:
+    """Host-side table of the KV chunks one layer call can touch (pointers, lengths, strides)."""
+
+    def __init__(self, k_chunks: Sequence[torch.Tensor], v_chunks: Sequence[torch.Tensor]):
+        n = len(k_chunks)
+        _require(0 < n <= DT_MAX_CHUNKS and n == len(v_chunks), f"need 1..{DT_MAX_CHUNKS} KV chunks")
+        self.n = n
+        self.keep = (list(k_chunks), list(v_chunks))  # keep the tensors alive while pointers are in use
+        self.k_ptrs = (c_vp * n)()
+        self.v_ptrs = (c_vp * n)()
+        self.lens = (c_i32 * n)()
+        self.sb = (c_i64 * n)()
+        ss = sh = None
+        for i, (k, v) in enumerate(zip(k_chunks, v_chunks)):
+            _check_qkv(k, f"k[{i}]"); _check_qkv(v, f"v[{i}]")
+            _require(k.shape == v.shape and k.stride() == v.stride(), f"k[{i}] / v[{i}] mismatch")
+            if k.shape[1] > 0:
+                if ss is None:
+                    ss, sh = k.stride(1), k.stride(2)
+                    self.B, self.H, self.D = k.shape[0], k.shape[2], k.shape[3]
+                _require((k.stride(1), k.stride(2)) == (ss, sh), "all chunks must share token/head strides")
+                _require((k.shape[0], k.shape[2], k.shape[3]) == (self.B, self.H, self.D), "chunk B/H/D mismatch")
+            self.k_ptrs[i] = k.data_ptr()
+            self.v_ptrs[i] = v.data_ptr()
+            self.lens[i] = k.shape[1]
+            self.sb[i] = k.stride(0)
+        _require(ss is not None, "all KV chunks are empty")
+        self.ss, self.sh = ss, sh
+
+
+def attn_jobs_fwd(q: torch.Tensor, table: ChunkTable, jobs: Sequence[Sequence[int]],
+                  outs: Sequence[torch.Tensor], lses: Sequence[torch.Tensor], softmax_scale: float = 0.0) -> None:
+    """One launch; job j attends q to the concatenation of chunks ``jobs[j]`` and writes (outs[j], lses[j])."""
+    lib = load_library()
+    _check_qkv(q, "q")
+    B, Sq, H, D = q.shape
+    _require((B, H, D) == (table.B, table.H, table.D), "q and KV chunks disagree on B/H/D")
+    nj = len(jobs)
+    _require(nj == len(outs) == len(lses) and nj <= DT_MAX_JOBS, f"need at most {DT_MAX_JOBS} jobs with one destination each")
+    if nj == 0:
+        return
+    begin = (c_i32 * (nj + 1))()
+    flat: List[int] = []
+    for j, ids in enumerate(jobs):
+        begin[j] = len(flat)
+        flat.extend(int(c) for c in ids)
+    begin[nj] = len(flat)
+    _require(len(flat) <= DT_MAX_JOB_ENTRIES, f"more than {DT_MAX_JOB_ENTRIES} chunk references in one launch")
+    chunks = (c_i32 * max(1, len(flat)))(*flat)
+    out_ptrs = (c_vp * nj)()
+    lse_ptrs = (c_vp * nj)()
+    for j in range(nj):
+        o, l = outs[j], lses[j]
+        _require(o.dtype == torch.bfloat16 and o.is_contiguous() and tuple(o.shape) == (B, Sq, H, D), f"outs[{j}] must be contiguous bf16 [B,Sq,H,D]")
+        _require(l.dtype == torch.float32 and l.is_contiguous() and tuple(l.shape) == (B, H, Sq), f"lses[{j}] must be contiguous fp32 [B,H,Sq]")
+        out_ptrs[j] = o.data_ptr()
+        lse_ptrs[j] = l.data_ptr()
+    rc = lib.dt_attn_jobs_fwd(q.data_ptr(), B, Sq, H, D, q.stride(0), q.stride(1), q.stride(2),
+                              table.n, table.k_ptrs, table.v_ptrs, table.lens, table.sb, table.ss, table.sh,
+                              nj, begin, chunks, out_ptrs, lse_ptrs, float(softmax_scale), _stream())
+    _check(rc, "dt_attn_jobs_fwd")
+
+
+def attn_sched_fwd(q: torch.Tensor, table: ChunkTable, dev_compute_ids: torch.Tensor, dev_count: torch.Tensor,
+                   max_jobs: int, slot_out: torch.Tensor, slot_lse: torch.Tensor, diag: int,
+                   diag_out: Optional[torch.Tensor], diag_lse: Optional[torch.Tensor],
+                   softmax_scale: float = 0.0) -> None:
+    """Device-scheduled launch: chunk ids come from ``dev_compute_ids[:dev_count]`` in device memory and
+    each state lands in its slot of the arena (``slot_out [C,B,Sq,H,D]`` bf16, ``slot_lse [C,B,H,Sq]`` fp32)."""
+    lib = load_library()
+    _check_qkv(q, "q")
+    B, Sq, H, D = q.shape
+    _require((B, H, D) == (table.B, table.H, table.D), "q and KV chunks disagree on B/H/D")
+    _require(dev_compute_ids.dtype == torch.int32 and dev_count.dtype == torch.int32 and dev_compute_ids.is_cuda and dev_count.is_cuda,
+             "schedule tensors must be int32 on the GPU")
+    _require(dev_compute_ids.is_contiguous() and dev_compute_ids.numel() >= max_jobs, "compute id list shorter than max_jobs")
+    _require(slot_out.dtype == torch.bfloat16 and slot_out.is_contiguous() and tuple(slot_out.shape[1:]) == (B, Sq, H, D)
+             and slot_out.shape[0] >= table.n, "slot_out must be contiguous bf16 [C,B,Sq,H,D]")
+    _require(slot_lse.dtype == torch.float32 and slot_lse.is_contiguous() and tuple(slot_lse.shape[1:]) == (B, H, Sq)
+             and slot_lse.shape[0] >= table.n, "slot_lse must be contiguous fp32 [C,B,H,Sq]")
+    if 0 <= diag < table.n:
+        _require(diag_out is not None and diag_lse is not None, "a diag chunk needs (diag_out, diag_lse)")
+        _require(diag_out.dtype == torch.bfloat16 and diag_out.is_contiguous() and tuple(diag_out.shape) == (B, Sq, H, D), "diag_out must be contiguous bf16 [B,Sq,H,D]")
+        _require(diag_lse.dtype == torch.float32 and diag_lse.is_contiguous() and tuple(diag_lse.shape) == (B, H, Sq), "diag_lse must be contiguous fp32 [B,H,Sq]")
+    rc = lib.dt_attn_sched_fwd(q.data_ptr(), B, Sq, H, D, q.stride(0), q.stride(1), q.stride(2),
+                               table.n, table.k_ptrs, table.v_ptrs, table.lens, table.sb, table.ss, table.sh,
+                               dev_compute_ids.data_ptr(), dev_count.data_ptr(), int(max_jobs),
+                               slot_out.data_ptr(), slot_out.stride(0), slot_lse.data_ptr(), slot_lse.stride(0),
+                               int(diag), diag_out.data_ptr() if diag_out is not None else None,
+                               diag_lse.data_ptr() if diag_lse is not None else None,
+                               float(softmax_scale), _stream())
+    _check(rc, "dt_attn_sched_fwd")
+
+
+# ---------------------------------------------------------------------------------------------
+# K2: merge, K3: cache store/load
+# ---------------------------------------------------------------------------------------------
+
+def merge_states(outs: Sequence[torch.Tensor], lses: Sequence[torch.Tensor],
+                 dst_out: Optional[torch.Tensor] = None, dst_lse: Optional[torch.Tensor] = None,
+                 dst_dtype: torch.dtype = torch.float32, dst_lse_bsh: bool = False):
+    """N-way LSE merge in one pass.  outs[i] contiguous [B,Sq,H,D] (bf16 or fp32), lses[i] fp32 in
+    [B,H,Sq] or [B,Sq,H(,1)] storage.  Returns (dst_out, dst_lse)."""
+    lib = load_library()
+    n = len(outs)
+    _require(0 < n <= DT_MAX_MERGE and n == len(lses), f"need 1..{DT_MAX_MERGE} states")
+    B, Sq, H, D = outs[0].shape
+    dev = outs[0].device
+    out_ptrs = (c_vp * n)()
+    lse_ptrs = (c_vp * n)()
+    dts = (c_i32 * n)()
+    lays = (c_i32 * n)()
+    for i, (o, l) in enumerate(zip(outs, lses)):
+        _require(o.is_cuda and o.is_contiguous() and tuple(o.shape) == (B, Sq, H, D), f"outs[{i}] must be contiguous [B,Sq,H,D] on the GPU")
+        out_ptrs[i] = o.data_ptr()
+        lse_ptrs[i] = l.data_ptr()
+        dts[i] = _dtype_code(o)
+        lays[i] = lse_layout_of(l, B, Sq, H)
+    if dst_out is None:
+        dst_out = torch.empty((B, Sq, H, D), dtype=dst_dtype, device=dev)
+    if dst_lse is None:
+        dst_lse = torch.empty((B, Sq, H, 1) if dst_lse_bsh else (B, H, Sq), dtype=torch.float32, device=dev)
+    _require(dst_out.is_contiguous() and tuple(dst_out.shape) == (B, Sq, H, D), "dst_out must be contiguous [B,Sq,H,D]")
+    dlay = lse_layout_of(dst_lse, B, Sq, H)
+    rc = lib.dt_merge_states(n, out_ptrs, lse_ptrs, dts, lays, dst_out.data_ptr(), _dtype_code(dst_out),
+                             dst_lse.data_ptr(), dlay, B, Sq, H, D, _stream())
+    _check(rc, "dt_merge_states")
+    return dst_out, dst_lse
+
+
+def cache_store(src_out: torch.Tensor, src_lse: torch.Tensor, slot_out: torch.Tensor, slot_lse: torch.Tensor) -> None:
+    lib = load_library()
+    B, Sq, H, D = src_out.shape
+    _require(src_out.is_cuda and src_out.is_contiguous(), "src_out must be contiguous on the GPU")
+    _require(slot_out.dtype == torch.bfloat16 and slot_out.is_contiguous() and tuple(slot_out.shape) == (B, Sq, H, D), "slot_out must be contiguous bf16 [B,Sq,H,D]")
+    _require(slot_lse.dtype == torch.float32 and slot_lse.is_contiguous() and tuple(slot_lse.shape) == (B, H, Sq), "slot_lse must be contiguous fp32 [B,H,Sq]")
+    rc = lib.dt_cache_store(src_out.data_ptr(), _dtype_code(src_out), src_lse.data_ptr(), lse_layout_of(src_lse, B, Sq, H),
+                            slot_out.data_ptr(), slot_lse.data_ptr(), B, Sq, H, D, _stream())
+    _check(rc, "dt_cache_store")
+
+
+def cache_load(slot_out: torch.Tensor, slot_lse: torch.Tensor, dst_dtype: torch.dtype = torch.float32,
+               dst_lse_bsh: bool = False):
+    lib = load_library()
+    B, Sq, H, D = slot_out.shape
+    _require(slot_out.dtype == torch.bfloat16 and slot_out.is_contiguous(), "slot_out must be contiguous bf16")
+    _require(slot_lse.dtype == torch.float32 and slot_lse.is_contiguous() and tuple(slot_lse.shape) == (B, H, Sq), "slot_lse must be contiguous fp32 [B,H,Sq]")
+    dst_out = torch.empty((B, Sq, H, D), dtype=dst_dtype, device=slot_out.device)
+    dst_lse = torch.empty((B, Sq, H, 1) if dst_lse_bsh else (B, H, Sq), dtype=torch.float32, device=slot_out.device)
+    rc = lib.dt_cache_load(slot_out.data_ptr(), slot_lse.data_ptr(), dst_out.data_ptr(), _dtype_code(dst_out),
+                           dst_lse.data_ptr(), DT_LSE_BSH if dst_lse_bsh else DT_LSE_BHS, B, Sq, H, D, _stream())
+    _check(rc, "dt_cache_load")
+    return dst_out, dst_lse
+
+
+# ---------------------------------------------------------------------------------------------
+# K4: schedule builder, rel-L1 sums
+# ---------------------------------------------------------------------------------------------
+
+def build_schedule(mask: torch.Tensor, t: int, l: int, diag: int = -1):
+    """(compute_ids [C], reuse_ids [C], counts [2]) int32 device tensors for row (t, l) of mask uint8 [T,L,C]."""
+    lib = load_library()
+    _require(mask.is_cuda and mask.dtype == torch.uint8 and mask.dim() == 3 and mask.is_contiguous(), "mask must be contiguous uint8 [T,L,C] on the GPU")
+    T, L, C = mask.shape
+    comp = torch.empty(C, dtype=torch.int32, device=mask.device)
+    reu = torch.empty(C, dtype=torch.int32, device=mask.device)
+    cnt = torch.empty(2, dtype=torch.int32, device=mask.device)
+    rc = lib.dt_build_schedule(mask.data_ptr(), T, L, C, int(t), int(l), int(diag), comp.data_ptr(), reu.data_ptr(), cnt.data_ptr(), _stream())
+    _check(rc, "dt_build_schedule")
+    return comp, reu, cnt
+
+
+def build_schedule_table(mask: torch.Tensor, diag: int = -1):
+    lib = load_library()
+    _require(mask.is_cuda and mask.dtype == torch.uint8 and mask.dim() == 3 and mask.is_contiguous(), "mask must be contiguous uint8 [T,L,C] on the GPU")
+    T, L, C = mask.shape
+    comp = torch.empty((T, L, C), dtype=torch.int32, device=mask.device)
+    reu = torch.empty((T, L, C), dtype=torch.int32, device=mask.device)
+    cnt = torch.empty((T, L, 2), dtype=torch.int32, device=mask.device)
+    rc = lib.dt_build_schedule_table(mask.data_ptr(), T, L, C, int(diag), comp.data_ptr(), reu.data_ptr(), cnt.data_ptr(), _stream())
+    _check(rc, "dt_build_schedule_table")
+    return comp, reu, cnt
+
+
+def rel_l1_sums(a: torch.Tensor, b: torch.Tensor, sums: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp64 [4] device tensor: sum|a-b|, sum|a|, sum|b|, count over entries where neither is NaN (no host sync)."""
+    lib = load_library()
+    _require(a.is_cuda and b.is_cuda and a.dtype == torch.float32 and b.dtype == torch.float32, "inputs must be fp32 on the GPU")
+    _require(a.is_contiguous() and b.is_contiguous() and a.numel() == b.numel(), "inputs must be contiguous and equally sized")
+    if sums is None:
+        sums = torch.zeros(4, dtype=torch.float64, device=a.device)
+    rc = lib.dt_rel_l1_sums(a.data_ptr(), b.data_ptr(), a.numel(), sums.data_ptr(), _stream())
+    _check(rc, "dt_rel_l1_sums")
+    return sums

@@ -1,0 +1,64 @@
+"""Build libditango_hip.so (gfx950) in-tree with hipcc.
+
+``python -m ditango_amd.build`` compiles every translation unit under
+``ditango_amd/csrc`` and links ``ditango_amd/lib/libditango_hip.so``.  hipcc
+cross-compiles for gfx950 without a GPU.  Packed-FP32 instruction selection is
+switched off for all device code (``-target-feature -packed-fp32-ops``).
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+PKG = Path(__file__).resolve().parent
+ROOT = PKG.parent
+CSRC = PKG / "csrc"
+LIB_DIR = PKG / "lib"
+LIB_PATH = LIB_DIR / "libditango_hip.so"
+SOURCES = ["attn_fwd.hip", "state_ops.hip", "capi.hip"]
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+COMMON = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+    f"-I{ROOT / 'include'}", f"-I{CSRC}",
+]
+
+
+def _run(cmd):
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("command failed: " + " ".join(map(str, cmd)) + "\n" + res.stdout + res.stderr)
+    return res
+
+
+def build_lib(verbose: bool = False, extra_flags=()) -> Path:
+    """Compile and link the library unconditionally; returns its path."""
+    LIB_DIR.mkdir(exist_ok=True)
+    objs = []
+
+    def compile_one(src):
+        obj = LIB_DIR / (Path(src).stem + ".o")
+        cmd = [HIPCC, *COMMON, *extra_flags, "-c", str(CSRC / src), "-o", str(obj)]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        _run(cmd)
+        return obj
+
+    with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as ex:
+        objs = list(ex.map(compile_one, SOURCES))
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objs), "-o", str(LIB_PATH)]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    _run(cmd)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    path = build_lib(verbose=True)
+    print(f"built {path}")
+    sys.exit(0)

@@ -1,0 +1,368 @@
+// Chunk attention forward for gfx950 (MI355X): out = softmax(q k^T * scale) v and
+// the natural-log lse of one query shard against one or several KV chunks.
+//
+// Stands in for flash_attn_func as called at core/attention.py:137-143,185-191
+// of the reference.
+//
+// Shape of the computation
+//   * One workgroup = 4 wavefronts = 128 queries of one (batch, head); each
+//     wavefront owns 32 queries.  Two workgroups per CU (8 waves/CU, 256 VGPRs
+//     each) so one wave's softmax VALU work overlaps another's MFMA work.
+//   * KV is consumed in tiles of 64 keys.  K is staged in LDS as [key][d],
+//     V is transposed on the way in and staged as [d][key]; both are
+//     double-buffered and XOR-swizzled in 16-byte units so that the MFMA
+//     operand reads (ds_read_b128) are bank-conflict free.
+//   * Scores are computed TRANSPOSED, S^T = K Q^T, with v_mfma_f32_32x32x16_bf16:
+//     in the accumulator layout a lane then owns ONE query (column lane%32) and
+//     16 of the 32 keys of the tile, so the online-softmax max/sum are
+//     in-register reductions plus a single exchange with lane^32.
+//   * The rows of the K operand are permuted (bits 2 and 3 of the row index
+//     swapped) so that the 8 accumulator registers a lane holds for a half tile
+//     are 8 CONSECUTIVE keys.  Rounded to bf16 they are directly the B operand
+//     of the second MFMA, O^T += V^T P^T, whose A operand is one 16-byte read of
+//     8 consecutive keys of one d-row of the transposed V tile.
+//   * O^T stays in registers as [d][query]: the per-tile rescale is a multiply by
+//     a per-lane scalar.  The epilogue transposes through LDS so that the global
+//     stores are 16 bytes per lane, 16 lanes per 256-byte row.
+//   * Workgroups are mapped to (head, query tile) so that the 8 XCDs each work
+//     through a contiguous range of heads: the workgroups that share an XCD's
+//     L2 stream the same K/V.
+#include "dt_common.h"
+
+namespace dt {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kWaves = 4;
+constexpr int kThreads = kWaves * 64;
+constexpr int kBQ = 128;  // queries per workgroup
+constexpr int kBK = 64;   // keys per tile
+constexpr int kXcds = 8;
+
+template <int N> struct VecOf;
+template <> struct VecOf<4> { typedef u32x4 type; };
+template <> struct VecOf<2> { typedef u32x2 type; };
+
+// Row permutation of the K operand: MFMA row i -> key (within a 32-key half tile).
+__device__ __forceinline__ int key_of_row(int i) {
+  return (i & 19) | ((i & 4) << 1) | ((i & 8) >> 1);
+}
+
+template <int D>
+struct Tile {
+  static constexpr int kRowBytesK = D * 2;            // one key, all d
+  static constexpr int kChunksK = D / 8;              // 16-byte chunks per K row
+  static constexpr int kBytesK = kBK * kRowBytesK;
+  static constexpr int kBytesV = D * kBK * 2;         // [d][64 keys]
+  static constexpr int kBytesBuf = kBytesK + kBytesV;
+  static constexpr int kLoadsK = kBK * kChunksK / kThreads;  // 16-byte loads per thread
+  static constexpr int kDV = D / 16;                  // d values per thread in the V transpose
+  static constexpr int kVW = kDV / 2;                 // dwords per V load
+  static constexpr int kPitchO = D * 2 + 16;          // epilogue row pitch
+
+  // byte offset of 16-byte chunk c of K row `key`
+  __device__ static __forceinline__ int k_off(int key, int c) {
+    if (kChunksK == 16) return key * kRowBytesK + ((c ^ (key & 15)) << 4);
+    return key * kRowBytesK + ((c ^ ((key >> 1) & 7)) << 4);
+  }
+  // byte offset of 16-byte chunk c (8 keys) of V^T row d
+  __device__ static __forceinline__ int v_off(int d, int c) {
+    return d * (kBK * 2) + ((c ^ (((d >> 1) ^ (d >> 4)) & 7)) << 4);
+  }
+};
+
+template <int D>
+__global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a) {
+  using T = Tile<D>;
+  using VLoad = typename VecOf<T::kVW>::type;
+  __shared__ __attribute__((aligned(16))) uint8_t lds[2 * T::kBytesBuf];
+
+  // ---- which (job, batch, head, query tile) ------------------------------------------
+  const int job = blockIdx.y;
+  const int xcd = blockIdx.x & (kXcds - 1);
+  const int idx = blockIdx.x >> 3;
+  const int item = xcd * a.per_xcd + idx;
+  if (idx >= a.per_xcd || item >= a.total) return;
+  const int bh = item / a.nqt;
+  const int qt = item - bh * a.nqt;
+  const int b = bh / a.H;
+  const int h = bh - b * a.H;
+
+  int seg_begin, seg_end, single = -1;
+  __bf16* out_ptr;
+  float* lse_ptr;
+  if (a.dev_ids != nullptr) {
+    if (job >= *a.dev_count) return;
+    single = a.dev_ids[job];
+    if (single < 0 || single >= a.n_chunks) return;  // never index the tables with a bad id
+    seg_begin = 0;
+    seg_end = 1;
+    if (single == a.diag) {
+      out_ptr = a.diag_out;
+      lse_ptr = a.diag_lse;
+    } else {
+      out_ptr = a.slot_out + (int64_t)single * a.slot_out_stride;
+      lse_ptr = a.slot_lse + (int64_t)single * a.slot_lse_stride;
+    }
+  } else {
+    seg_begin = a.job_begin[job];
+    seg_end = a.job_begin[job + 1];
+    out_ptr = a.job_out[job];
+    lse_ptr = a.job_lse[job];
+  }
+  auto chunk_of = [&](int seg) -> int { return single >= 0 ? single : (int)a.job_chunks[seg]; };
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int col = lane & 31;   // query column (B operand) / operand row (A operand)
+  const int hh = lane >> 5;    // which half of the contraction dimension this lane feeds
+  const int q0 = qt * kBQ + wave * 32;
+
+  // ---- Q fragments: B operand of S^T = K Q^T, kept in registers ----------------------
+  bf16x8 qf[D / 16];
+  {
+    int qrow = q0 + col;
+    if (qrow > a.Sq - 1) qrow = a.Sq - 1;
+    const __bf16* qp = a.q + (int64_t)b * a.q_sb + (int64_t)qrow * a.q_ss + (int64_t)h * a.q_sh + 8 * hh;
+#pragma unroll
+    for (int s = 0; s < D / 16; ++s) qf[s] = *reinterpret_cast<const bf16x8*>(qp + 16 * s);
+  }
+
+  // ---- tile bookkeeping -----------------------------------------------------------------
+  int n_tiles = 0;
+  for (int s = seg_begin; s < seg_end; ++s) n_tiles += (a.kv_len[chunk_of(s)] + kBK - 1) / kBK;
+
+  // load cursor (one tile ahead of the compute cursor)
+  int ld_seg = seg_begin, ld_k0 = 0;
+  int cp_seg = seg_begin, cp_k0 = 0;
+  while (ld_seg < seg_end && a.kv_len[chunk_of(ld_seg)] == 0) ++ld_seg;
+  cp_seg = ld_seg;
+
+  // thread -> K tile elements
+  const int kc = tid % T::kChunksK;            // 16-byte chunk within the row
+  const int kr0 = tid / T::kChunksK;           // first key row
+  constexpr int kRowStep = kThreads / T::kChunksK;
+  // thread -> V tile elements: 4 keys x kDV d
+  const int vdg = tid & 15;
+  const int vkg = tid >> 4;
+
+  u32x4 kreg[T::kLoadsK];
+  VLoad vreg[4];
+
+  auto load_tile = [&](int seg, int k0) {
+    const int cid = chunk_of(seg);
+    const int len = a.kv_len[cid];
+    const __bf16* kb = a.k[cid] + (int64_t)b * a.kv_sb[cid] + (int64_t)h * a.kv_sh;
+    const __bf16* vb = a.v[cid] + (int64_t)b * a.kv_sb[cid] + (int64_t)h * a.kv_sh;
+#pragma unroll
+    for (int i = 0; i < T::kLoadsK; ++i) {
+      int key = k0 + kr0 + i * kRowStep;
+      if (key > len - 1) key = len - 1;  // clamped rows are masked out of the softmax
+      kreg[i] = *reinterpret_cast<const u32x4*>(kb + (int64_t)key * a.kv_ss + 8 * kc);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      int key = k0 + 4 * vkg + r;
+      if (key > len - 1) key = len - 1;  // weight of a clamped row is exactly 0
+      vreg[r] = *reinterpret_cast<const VLoad*>(vb + (int64_t)key * a.kv_ss + T::kDV * vdg);
+    }
+  };
+
+  auto store_tile = [&](int buf) {
+    uint8_t* kl = lds + buf * T::kBytesBuf;
+    uint8_t* vl = kl + T::kBytesK;
+#pragma unroll
+    for (int i = 0; i < T::kLoadsK; ++i) {
+      const int key = kr0 + i * kRowStep;
+      *reinterpret_cast<u32x4*>(kl + T::k_off(key, kc)) = kreg[i];
+    }
+    // transpose 4 keys x kDV d -> kDV rows of 4 keys
+#pragma unroll
+    for (int jj = 0; jj < T::kDV; ++jj) {
+      const int w = jj >> 1;
+      const uint32_t sel = (jj & 1) ? 0x07060302u : 0x05040100u;
+      u32x2 o;
+      o.x = __builtin_amdgcn_perm(vreg[1][w], vreg[0][w], sel);
+      o.y = __builtin_amdgcn_perm(vreg[3][w], vreg[2][w], sel);
+      const int d = T::kDV * vdg + jj;
+      *reinterpret_cast<u32x2*>(vl + T::v_off(d, vkg >> 1) + ((vkg & 1) << 3)) = o;
+    }
+  };
+
+  auto advance = [&](int& seg, int& k0) {
+    k0 += kBK;
+    if (k0 >= a.kv_len[chunk_of(seg)]) {
+      k0 = 0;
+      ++seg;
+      while (seg < seg_end && a.kv_len[chunk_of(seg)] == 0) ++seg;
+    }
+  };
+
+  // ---- accumulators ---------------------------------------------------------------------
+  f32x16 o_acc[D / 32];
+#pragma unroll
+  for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o_acc[i][r] = 0.f;
+  float m_run = -INFINITY;  // running max of the raw scores of this lane's query
+  float l_run = 0.f;        // running sum over THIS lane's keys (halves combined at the end)
+  const float c = a.scale_log2;
+
+  if (n_tiles > 0) {
+    load_tile(ld_seg, ld_k0);
+    store_tile(0);
+    advance(ld_seg, ld_k0);
+  }
+  __syncthreads();
+
+  const int krow = key_of_row(col);
+
+  for (int t = 0; t < n_tiles; ++t) {
+    const bool has_next = (t + 1 < n_tiles);
+    if (has_next) load_tile(ld_seg, ld_k0);
+
+    const uint8_t* kl = lds + (t & 1) * T::kBytesBuf;
+    const uint8_t* vl = kl + T::kBytesK;
+    const int kvalid = a.kv_len[chunk_of(cp_seg)] - cp_k0;  // >= 1
+
+    // ---- S^T = K Q^T : two 32-key halves ------------------------------------------------
+    f32x16 s_acc[2];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s_acc[kb][r] = 0.f;
+      const int row = 32 * kb + krow;
+#pragma unroll
+      for (int s = 0; s < D / 16; ++s) {
+        const bf16x8 ka = *reinterpret_cast<const bf16x8*>(kl + T::k_off(row, 2 * s + hh));
+        s_acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[s], s_acc[kb], 0, 0, 0);
+      }
+    }
+    if (kvalid < kBK) {
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = 32 * kb + 16 * (r >> 3) + 8 * hh + (r & 7);
+          if (key >= kvalid) s_acc[kb][r] = -INFINITY;
+        }
+    }
+
+    // ---- online softmax -----------------------------------------------------------------
+    float mx = s_acc[0][0];
+#pragma unroll
+    for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s_acc[0][r]);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s_acc[1][r]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float m_new = fmaxf(m_run, mx);
+    const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c);
+    const float mc = m_new * c;
+    m_run = m_new;
+    float rs = 0.f;
+    bf16x8 pf[2][2];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int r = 0; r < 16; r += 2) {
+        f32x2 p;
+        p.x = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[kb][r], c, -mc));
+        p.y = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[kb][r + 1], c, -mc));
+        rs += p.x + p.y;
+        const bf16x2 pb = __builtin_convertvector(p, bf16x2);
+        pf[kb][r >> 3][r & 7] = pb.x;
+        pf[kb][r >> 3][(r & 7) + 1] = pb.y;
+      }
+    l_run = l_run * alpha + rs;
+#pragma unroll
+    for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o_acc[i][r] *= alpha;
+
+    // ---- O^T += V^T P^T -----------------------------------------------------------------
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db) {
+      const int d = 32 * db + col;
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          const bf16x8 va = *reinterpret_cast<const bf16x8*>(vl + T::v_off(d, 4 * kb + 2 * half + hh));
+          o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pf[kb][half], o_acc[db], 0, 0, 0);
+        }
+    }
+
+    advance(cp_seg, cp_k0);
+    if (has_next) {
+      store_tile((t + 1) & 1);
+      advance(ld_seg, ld_k0);
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue -------------------------------------------------------------------------
+  const float l_tot = l_run + __shfl_xor(l_run, 32);
+  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+  const float lse = l_tot > 0.f ? (m_run * c + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f : -INFINITY;
+  const int qrow = q0 + col;
+  if (hh == 0 && qrow < a.Sq) lse_ptr[((int64_t)b * a.H + h) * a.Sq + qrow] = lse;
+
+  // O^T (registers, [d][query]) -> LDS [query][d] bf16 -> coalesced 16-byte stores.
+  // The loop ended with a barrier, so the tile buffers are free.
+  uint8_t* ol = lds + wave * (32 * T::kPitchO);
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      f32x2 lo, hi;
+      lo.x = o_acc[db][4 * g + 0] * inv;
+      lo.y = o_acc[db][4 * g + 1] * inv;
+      hi.x = o_acc[db][4 * g + 2] * inv;
+      hi.y = o_acc[db][4 * g + 3] * inv;
+      const bf16x2 l2 = __builtin_convertvector(lo, bf16x2);
+      const bf16x2 h2 = __builtin_convertvector(hi, bf16x2);
+      bf16x4 pk;
+      pk.x = l2.x; pk.y = l2.y; pk.z = h2.x; pk.w = h2.y;
+      const int d = 32 * db + 8 * g + 4 * hh;
+      *reinterpret_cast<bf16x4*>(ol + col * T::kPitchO + d * 2) = pk;
+    }
+  __syncthreads();
+  constexpr int kLanesPerRow = D / 8;
+  constexpr int kRowsPerPass = 64 / kLanesPerRow;
+  const int rr = lane / kLanesPerRow;
+  const int cc = lane % kLanesPerRow;
+#pragma unroll
+  for (int p = 0; p < 32 / kRowsPerPass; ++p) {
+    const int row = p * kRowsPerPass + rr;
+    const int qg = q0 + row;
+    const u32x4 val = *reinterpret_cast<const u32x4*>(ol + row * T::kPitchO + cc * 16);
+    if (qg < a.Sq) {
+      __bf16* dst = out_ptr + (((int64_t)b * a.Sq + qg) * a.H + h) * D + cc * 8;
+      *reinterpret_cast<u32x4*>(dst) = val;
+    }
+  }
+}
+
+int launch_attn(const AttnArgs& a, int D, int n_jobs, hipStream_t stream) {
+  if (n_jobs <= 0 || a.total <= 0) return DT_OK;
+  dim3 grid((unsigned)(a.per_xcd * kXcds), (unsigned)n_jobs, 1);
+  dim3 block(kThreads, 1, 1);
+  if (D == 128) {
+    hipLaunchKernelGGL(attn_fwd_kernel<128>, grid, block, 0, stream, a);
+  } else if (D == 64) {
+    hipLaunchKernelGGL(attn_fwd_kernel<64>, grid, block, 0, stream, a);
+  } else {
+    set_error("head dim %d not built (64 and 128 are)", D);
+    return DT_ERR_UNSUPPORTED;
+  }
+  return hip_fail(hipGetLastError(), "attn_fwd launch");
+}
+
+}  // namespace dt

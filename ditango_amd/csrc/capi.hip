@@ -1,0 +1,193 @@
+// C ABI entry points of the chunk-attention kernel plus the error plumbing.
+// Argument checks happen here, on the host, before any launch: the kernels
+// assume the shapes, strides and alignments validated below.
+#include <cstdarg>
+#include <cstdio>
+#include <cmath>
+
+#include "dt_common.h"
+
+namespace dt {
+
+static thread_local char g_error[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+
+int hip_fail(hipError_t e, const char* what) {
+  if (e == hipSuccess) return DT_OK;
+  set_error("%s: %s", what, hipGetErrorString(e));
+  return DT_ERR_HIP;
+}
+
+}  // namespace dt
+
+using namespace dt;
+
+extern "C" int dt_version(void) { return 100; }
+extern "C" const char* dt_last_error(void) { return g_error; }
+
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+static int fill_common(AttnArgs& a, const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D, int64_t q_sb,
+                       int64_t q_ss, int64_t q_sh, int32_t n_chunks, const void* const* k_ptrs,
+                       const void* const* v_ptrs, const int32_t* kv_lens, const int64_t* kv_sb, int64_t kv_ss,
+                       int64_t kv_sh, float softmax_scale) {
+  if (B <= 0 || Sq <= 0 || H <= 0) {
+    set_error("B, Sq, H must be positive (got %d, %d, %d)", B, Sq, H);
+    return DT_ERR_INVALID;
+  }
+  if (D != 64 && D != 128) {
+    set_error("head dim %d not built (64 and 128 are)", D);
+    return DT_ERR_UNSUPPORTED;
+  }
+  if (!q || !aligned16(q) || (q_sb % 8) || (q_ss % 8) || (q_sh % 8)) {
+    set_error("q must be non-null, 16-byte aligned, with strides that are multiples of 8 elements");
+    return DT_ERR_INVALID;
+  }
+  if (n_chunks <= 0 || n_chunks > DT_MAX_CHUNKS) {
+    set_error("%d KV chunks: need 1..%d", n_chunks, DT_MAX_CHUNKS);
+    return DT_ERR_INVALID;
+  }
+  if (!k_ptrs || !v_ptrs || !kv_lens || !kv_sb) {
+    set_error("null chunk table");
+    return DT_ERR_INVALID;
+  }
+  if ((kv_ss % 8) || (kv_sh % 8) || kv_ss <= 0) {
+    set_error("k/v token and head strides must be multiples of 8 elements");
+    return DT_ERR_INVALID;
+  }
+  a.q = static_cast<const __bf16*>(q);
+  a.q_sb = q_sb; a.q_ss = q_ss; a.q_sh = q_sh;
+  a.B = B; a.H = H; a.Sq = Sq;
+  a.nqt = (Sq + 127) / 128;
+  const int64_t total = (int64_t)B * H * a.nqt;
+  if (total > (1 << 28)) {
+    set_error("too many query tiles (%lld)", (long long)total);
+    return DT_ERR_INVALID;
+  }
+  a.total = (int32_t)total;
+  a.per_xcd = (a.total + 7) / 8;
+  const float scale = softmax_scale > 0.f ? softmax_scale : 1.0f / std::sqrt((float)D);
+  a.scale_log2 = scale * 1.4426950408889634f;
+  for (int i = 0; i < n_chunks; ++i) {
+    if (kv_lens[i] < 0) {
+      set_error("chunk %d has negative length", i);
+      return DT_ERR_INVALID;
+    }
+    if (kv_lens[i] > 0 && (!k_ptrs[i] || !v_ptrs[i] || !aligned16(k_ptrs[i]) || !aligned16(v_ptrs[i]) || (kv_sb[i] % 8))) {
+      set_error("chunk %d: null or misaligned k/v", i);
+      return DT_ERR_INVALID;
+    }
+    a.k[i] = static_cast<const __bf16*>(k_ptrs[i]);
+    a.v[i] = static_cast<const __bf16*>(v_ptrs[i]);
+    a.kv_len[i] = kv_lens[i];
+    a.kv_sb[i] = kv_sb[i];
+  }
+  a.n_chunks = n_chunks;
+  a.kv_ss = kv_ss;
+  a.kv_sh = kv_sh;
+  return DT_OK;
+}
+
+extern "C" int dt_attn_jobs_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D, int64_t q_sb, int64_t q_ss,
+                                int64_t q_sh, int32_t n_chunks, const void* const* k_ptrs, const void* const* v_ptrs,
+                                const int32_t* kv_lens, const int64_t* kv_sb, int64_t kv_ss, int64_t kv_sh,
+                                int32_t n_jobs, const int32_t* job_begin, const int32_t* job_chunks,
+                                void* const* out_ptrs, float* const* lse_ptrs, float softmax_scale, void* stream) {
+  AttnArgs a{};
+  if (int rc = fill_common(a, q, B, Sq, H, D, q_sb, q_ss, q_sh, n_chunks, k_ptrs, v_ptrs, kv_lens, kv_sb, kv_ss, kv_sh,
+                           softmax_scale))
+    return rc;
+  if (n_jobs == 0) return DT_OK;
+  if (n_jobs < 0 || n_jobs > DT_MAX_JOBS || !job_begin || !job_chunks || !out_ptrs || !lse_ptrs) {
+    set_error("%d jobs: need 0..%d and non-null job tables", n_jobs, DT_MAX_JOBS);
+    return DT_ERR_INVALID;
+  }
+  if (job_begin[0] != 0 || job_begin[n_jobs] > DT_MAX_JOB_ENTRIES) {
+    set_error("job_begin must start at 0 and end at most at %d", DT_MAX_JOB_ENTRIES);
+    return DT_ERR_INVALID;
+  }
+  for (int j = 0; j < n_jobs; ++j) {
+    if (job_begin[j + 1] < job_begin[j]) {
+      set_error("job_begin is not monotone at job %d", j);
+      return DT_ERR_INVALID;
+    }
+    if (!out_ptrs[j] || !lse_ptrs[j] || !aligned16(out_ptrs[j])) {
+      set_error("job %d: null or misaligned destination", j);
+      return DT_ERR_INVALID;
+    }
+    a.job_out[j] = static_cast<__bf16*>(out_ptrs[j]);
+    a.job_lse[j] = lse_ptrs[j];
+    a.job_begin[j] = job_begin[j];
+  }
+  a.job_begin[n_jobs] = job_begin[n_jobs];
+  for (int e = 0; e < job_begin[n_jobs]; ++e) {
+    if (job_chunks[e] < 0 || job_chunks[e] >= n_chunks) {
+      set_error("job chunk reference %d is outside the chunk table", job_chunks[e]);
+      return DT_ERR_INVALID;
+    }
+    a.job_chunks[e] = (uint8_t)job_chunks[e];
+  }
+  return launch_attn(a, D, n_jobs, (hipStream_t)stream);
+}
+
+extern "C" int dt_attn_chunk_fwd(const void* q, const void* k, const void* v, void* out, float* lse, int32_t B,
+                                 int32_t Sq, int32_t Sk, int32_t H, int32_t D, int64_t q_sb, int64_t q_ss, int64_t q_sh,
+                                 int64_t kv_sb, int64_t kv_ss, int64_t kv_sh, float softmax_scale, void* stream) {
+  const void* kp[1] = {k};
+  const void* vp[1] = {v};
+  const int32_t lens[1] = {Sk};
+  const int64_t sbs[1] = {kv_sb};
+  const int32_t begin[2] = {0, 1};
+  const int32_t chunks[1] = {0};
+  void* outs[1] = {out};
+  float* lses[1] = {lse};
+  return dt_attn_jobs_fwd(q, B, Sq, H, D, q_sb, q_ss, q_sh, 1, kp, vp, lens, sbs, kv_ss, kv_sh, 1, begin, chunks, outs,
+                          lses, softmax_scale, stream);
+}
+
+extern "C" int dt_attn_sched_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D, int64_t q_sb, int64_t q_ss,
+                                 int64_t q_sh, int32_t n_chunks, const void* const* k_ptrs, const void* const* v_ptrs,
+                                 const int32_t* kv_lens, const int64_t* kv_sb, int64_t kv_ss, int64_t kv_sh,
+                                 const int32_t* dev_compute_ids, const int32_t* dev_count, int32_t max_jobs,
+                                 void* slot_out, int64_t slot_out_stride, float* slot_lse, int64_t slot_lse_stride,
+                                 int32_t diag, void* diag_out, float* diag_lse, float softmax_scale, void* stream) {
+  AttnArgs a{};
+  if (int rc = fill_common(a, q, B, Sq, H, D, q_sb, q_ss, q_sh, n_chunks, k_ptrs, v_ptrs, kv_lens, kv_sb, kv_ss, kv_sh,
+                           softmax_scale))
+    return rc;
+  if (max_jobs == 0) return DT_OK;
+  if (max_jobs < 0 || max_jobs > n_chunks) {
+    set_error("max_jobs %d must be in 0..n_chunks (%d)", max_jobs, n_chunks);
+    return DT_ERR_INVALID;
+  }
+  if (!dev_compute_ids || !dev_count || !slot_out || !slot_lse || !aligned16(slot_out) || (slot_out_stride % 8)) {
+    set_error("null or misaligned schedule/arena pointer");
+    return DT_ERR_INVALID;
+  }
+  for (int i = 0; i < n_chunks; ++i) {
+    if (kv_lens[i] > 0 && (!k_ptrs[i] || !v_ptrs[i])) {
+      set_error("chunk %d: null k/v", i);
+      return DT_ERR_INVALID;
+    }
+  }
+  if (diag >= 0 && diag < n_chunks && (!diag_out || !diag_lse || !aligned16(diag_out))) {
+    set_error("diag chunk %d needs a destination outside the cache", diag);
+    return DT_ERR_INVALID;
+  }
+  a.dev_ids = dev_compute_ids;
+  a.dev_count = dev_count;
+  a.slot_out = static_cast<__bf16*>(slot_out);
+  a.slot_lse = slot_lse;
+  a.slot_out_stride = slot_out_stride;
+  a.slot_lse_stride = slot_lse_stride;
+  a.diag = diag;
+  a.diag_out = static_cast<__bf16*>(diag_out);
+  a.diag_lse = diag_lse;
+  return launch_attn(a, D, max_jobs, (hipStream_t)stream);
+}

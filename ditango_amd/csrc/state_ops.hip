@@ -1,0 +1,430 @@
+// HBM-bound kernels around the attention-state cache (gfx950):
+//   * N-way LSE merge       (utils.py:24-84 of the reference, fused to one pass)
+//   * state copy / convert  (cache store and load, core/cache.py:75-84)
+//   * schedule builder      (per-chunk generalisation of core/attention.py:90-116)
+//   * relative-L1 sums      (utils.py:214-241)
+//
+// Work decomposition of the row kernels: one workgroup handles kRowsPerWg
+// consecutive queries of ONE (batch, head).  A group of D/8 lanes owns one row
+// (query, head) and moves 16 bytes of bf16 (8 elements) per lane per state, so a
+// row is one contiguous 128/256-byte access, and the lse values of consecutive
+// rows are consecutive floats in the [B,H,Sq] layout.
+#include "dt_common.h"
+
+namespace dt {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kThreads = 256;
+constexpr int kQPerWg = 64;  // queries per workgroup (several passes)
+
+struct MergeArgs {
+  int32_t n;
+  int32_t B, Sq, H;
+  const void* out[DT_MAX_MERGE];
+  const float* lse[DT_MAX_MERGE];
+  uint64_t fp32_mask;   // bit i: out[i] is fp32 (else bf16)
+  uint64_t bsh_mask;    // bit i: lse[i] is [B,Sq,H] (else [B,H,Sq])
+  void* dst_out;
+  float* dst_lse;
+  int32_t dst_fp32;
+  int32_t dst_bsh;
+};
+
+__device__ __forceinline__ int64_t lse_index(bool bsh, int b, int h, int s, int H, int Sq) {
+  return bsh ? ((int64_t)b * Sq + s) * H + h : ((int64_t)b * H + h) * Sq + s;
+}
+
+__device__ __forceinline__ void load8(const void* base, bool fp32, int64_t elem, float (&x)[8]) {
+  if (fp32) {
+    const f32x4* p = reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(base) + elem);
+    const f32x4 a = p[0], b = p[1];
+    x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w;
+    x[4] = b.x; x[5] = b.y; x[6] = b.z; x[7] = b.w;
+  } else {
+    const u32x4 v = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(base) + elem);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      x[2 * i] = __uint_as_float(v[i] << 16);
+      x[2 * i + 1] = __uint_as_float(v[i] & 0xffff0000u);
+    }
+  }
+}
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  f32x2 f;
+  f.x = lo;
+  f.y = hi;
+  const bf16x2 b = __builtin_convertvector(f, bf16x2);  // round to nearest even
+  return __builtin_bit_cast(uint32_t, b);
+}
+
+__device__ __forceinline__ void store8(void* base, bool fp32, int64_t elem, const float (&x)[8]) {
+  if (fp32) {
+    f32x4* p = reinterpret_cast<f32x4*>(reinterpret_cast<float*>(base) + elem);
+    f32x4 a, b;
+    a.x = x[0]; a.y = x[1]; a.z = x[2]; a.w = x[3];
+    b.x = x[4]; b.y = x[5]; b.z = x[6]; b.w = x[7];
+    p[0] = a;
+    p[1] = b;
+  } else {
+    u32x4 v;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = pack_bf16x2(x[2 * i], x[2 * i + 1]);
+    *reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(base) + elem) = v;
+  }
+}
+
+template <int D>
+__global__ __launch_bounds__(kThreads) void merge_states_kernel(const MergeArgs a) {
+  constexpr int kLanesPerRow = D / 8;
+  constexpr int kRowsPerPass = kThreads / kLanesPerRow;
+  const int n_st = (a.Sq + kQPerWg - 1) / kQPerWg;
+  const int wg = blockIdx.x;
+  const int st = wg % n_st;
+  const int bh = wg / n_st;
+  const int b = bh / a.H;
+  const int h = bh - b * a.H;
+  const int rr = threadIdx.x / kLanesPerRow;
+  const int cc = threadIdx.x % kLanesPerRow;
+#pragma unroll 1
+  for (int p = 0; p < kQPerWg / kRowsPerPass; ++p) {
+    const int s = st * kQPerWg + p * kRowsPerPass + rr;
+    if (s >= a.Sq) break;
+    const int64_t elem = (((int64_t)b * a.Sq + s) * a.H + h) * D + cc * 8;
+    // pass 1: the maximum lse
+    float m = -INFINITY;
+    for (int i = 0; i < a.n; ++i) {
+      const float l = a.lse[i][lse_index((a.bsh_mask >> i) & 1, b, h, s, a.H, a.Sq)];
+      m = fmaxf(m, l);
+    }
+    float acc[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) acc[k] = 0.f;
+    float den = 0.f;
+    if (m > -INFINITY) {
+#pragma unroll 4
+      for (int i = 0; i < a.n; ++i) {
+        const float l = a.lse[i][lse_index((a.bsh_mask >> i) & 1, b, h, s, a.H, a.Sq)];
+        const float w = __expf(l - m);
+        float x[8];
+        load8(a.out[i], (a.fp32_mask >> i) & 1, elem, x);
+        den += w;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) acc[k] = __builtin_fmaf(w, x[k], acc[k]);
+      }
+    }
+    const float inv = den > 0.f ? 1.f / den : 0.f;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) acc[k] *= inv;
+    store8(a.dst_out, a.dst_fp32 != 0, elem, acc);
+    if (cc == 0 && a.dst_lse != nullptr)
+      a.dst_lse[lse_index(a.dst_bsh != 0, b, h, s, a.H, a.Sq)] = den > 0.f ? m + __logf(den) : -INFINITY;
+  }
+}
+
+struct CopyArgs {
+  const void* src_out;
+  const float* src_lse;
+  void* dst_out;
+  float* dst_lse;
+  int32_t B, Sq, H;
+  int32_t src_fp32, src_bsh, dst_fp32, dst_bsh;
+};
+
+template <int D>
+__global__ __launch_bounds__(kThreads) void state_copy_kernel(const CopyArgs a) {
+  constexpr int kLanesPerRow = D / 8;
+  constexpr int kRowsPerPass = kThreads / kLanesPerRow;
+  const int n_st = (a.Sq + kQPerWg - 1) / kQPerWg;
+  const int wg = blockIdx.x;
+  const int st = wg % n_st;
+  const int bh = wg / n_st;
+  const int b = bh / a.H;
+  const int h = bh - b * a.H;
+  const int rr = threadIdx.x / kLanesPerRow;
+  const int cc = threadIdx.x % kLanesPerRow;
+#pragma unroll
+  for (int p = 0; p < kQPerWg / kRowsPerPass; ++p) {
+    const int s = st * kQPerWg + p * kRowsPerPass + rr;
+    if (s < a.Sq) {
+      const int64_t elem = (((int64_t)b * a.Sq + s) * a.H + h) * D + cc * 8;
+      float x[8];
+      load8(a.src_out, a.src_fp32 != 0, elem, x);
+      store8(a.dst_out, a.dst_fp32 != 0, elem, x);
+      if (cc == 0 && a.dst_lse != nullptr && a.src_lse != nullptr)
+        a.dst_lse[lse_index(a.dst_bsh != 0, b, h, s, a.H, a.Sq)] =
+            a.src_lse[lse_index(a.src_bsh != 0, b, h, s, a.H, a.Sq)];
+    }
+  }
+}
+
+// One wavefront per (t, l) row: ballot + prefix popcount compaction.
+__global__ __launch_bounds__(64) void build_schedule_kernel(const uint8_t* mask, int T, int L, int C, int row0,
+                                                            int diag, int32_t* compute_ids, int32_t* reuse_ids,
+                                                            int32_t* counts) {
+  const int row = row0 + blockIdx.x;          // t*L + l
+  const int orow = blockIdx.x;                // output row (0 for the single-row entry point)
+  const uint8_t* m = mask + (int64_t)row * C;
+  int32_t* comp = compute_ids + (int64_t)orow * C;
+  int32_t* reu = reuse_ids + (int64_t)orow * C;
+  const int lane = threadIdx.x;
+  const bool has_diag = (diag >= 0 && diag < C);
+  int n_comp = has_diag ? 1 : 0;
+  int n_reu = 0;
+  if (has_diag && lane == 0) comp[0] = diag;
+  for (int c0 = 0; c0 < C; c0 += 64) {
+    const int c = c0 + lane;
+    const bool in = c < C && c != diag;
+    const bool is_comp = in && m[c] == 0;
+    const bool is_reu = in && m[c] != 0;
+    const unsigned long long bc = __ballot(is_comp);
+    const unsigned long long br = __ballot(is_reu);
+    const unsigned long long lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+    if (is_comp) comp[n_comp + __popcll(bc & lt)] = c;
+    if (is_reu) reu[n_reu + __popcll(br & lt)] = c;
+    n_comp += __popcll(bc);
+    n_reu += __popcll(br);
+  }
+  for (int i = lane; i < C; i += 64) {
+    if (i >= n_comp) comp[i] = -1;
+    if (i >= n_reu) reu[i] = -1;
+  }
+  if (lane == 0) {
+    counts[2 * orow] = n_comp;
+    counts[2 * orow + 1] = n_reu;
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void rel_l1_sums_kernel(const float* a, const float* b, int64_t n,
+                                                               double* sums) {
+  float d = 0.f, sa = 0.f, sb = 0.f, cnt = 0.f;
+  const int64_t stride = (int64_t)gridDim.x * kThreads * 4;
+  for (int64_t i = ((int64_t)blockIdx.x * kThreads + threadIdx.x) * 4; i < n; i += stride) {
+    float xa[4], xb[4];
+    if (i + 4 <= n) {
+      const f32x4 va = *reinterpret_cast<const f32x4*>(a + i);
+      const f32x4 vb = *reinterpret_cast<const f32x4*>(b + i);
+      xa[0] = va.x; xa[1] = va.y; xa[2] = va.z; xa[3] = va.w;
+      xb[0] = vb.x; xb[1] = vb.y; xb[2] = vb.z; xb[3] = vb.w;
+    } else {
+      for (int k = 0; k < 4; ++k) {
+        const bool ok = i + k < n;
+        xa[k] = ok ? a[i + k] : NAN;
+        xb[k] = ok ? b[i + k] : NAN;
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const bool ok = !(xa[k] != xa[k]) && !(xb[k] != xb[k]);
+      if (ok) {
+        d += fabsf(xa[k] - xb[k]);
+        sa += fabsf(xa[k]);
+        sb += fabsf(xb[k]);
+        cnt += 1.f;
+      }
+    }
+  }
+  // wavefront reduction, then one fp64 atomic per wavefront
+  double v[4] = {(double)d, (double)sa, (double)sb, (double)cnt};
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v[k] += __shfl_xor(v[k], off);
+  }
+  if ((threadIdx.x & 63) == 0) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) atomicAdd(&sums[k], v[k]);
+  }
+}
+
+// ---- host-side launchers ---------------------------------------------------------------
+
+int launch_merge(const MergeArgs& a, int D, hipStream_t stream) {
+  const int n_st = (a.Sq + kQPerWg - 1) / kQPerWg;
+  const int64_t wgs = (int64_t)a.B * a.H * n_st;
+  if (wgs <= 0) return DT_OK;
+  if (wgs > 0x7fffffffLL) {
+    set_error("merge grid too large");
+    return DT_ERR_INVALID;
+  }
+  if (D == 128) {
+    hipLaunchKernelGGL(merge_states_kernel<128>, dim3((unsigned)wgs), dim3(kThreads), 0, stream, a);
+  } else if (D == 64) {
+    hipLaunchKernelGGL(merge_states_kernel<64>, dim3((unsigned)wgs), dim3(kThreads), 0, stream, a);
+  } else {
+    set_error("head dim %d not built (64 and 128 are)", D);
+    return DT_ERR_UNSUPPORTED;
+  }
+  return hip_fail(hipGetLastError(), "merge_states launch");
+}
+
+int launch_copy(const CopyArgs& a, int D, hipStream_t stream) {
+  const int n_st = (a.Sq + kQPerWg - 1) / kQPerWg;
+  const int64_t wgs = (int64_t)a.B * a.H * n_st;
+  if (wgs <= 0) return DT_OK;
+  if (wgs > 0x7fffffffLL) {
+    set_error("copy grid too large");
+    return DT_ERR_INVALID;
+  }
+  if (D == 128) {
+    hipLaunchKernelGGL(state_copy_kernel<128>, dim3((unsigned)wgs), dim3(kThreads), 0, stream, a);
+  } else if (D == 64) {
+    hipLaunchKernelGGL(state_copy_kernel<64>, dim3((unsigned)wgs), dim3(kThreads), 0, stream, a);
+  } else {
+    set_error("head dim %d not built (64 and 128 are)", D);
+    return DT_ERR_UNSUPPORTED;
+  }
+  return hip_fail(hipGetLastError(), "state_copy launch");
+}
+
+}  // namespace dt
+
+using namespace dt;
+
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+static int check_dims(int32_t B, int32_t Sq, int32_t H, int32_t D) {
+  if (B <= 0 || Sq <= 0 || H <= 0) {
+    set_error("B, Sq, H must be positive (got %d, %d, %d)", B, Sq, H);
+    return DT_ERR_INVALID;
+  }
+  if (D != 64 && D != 128) {
+    set_error("head dim %d not built (64 and 128 are)", D);
+    return DT_ERR_UNSUPPORTED;
+  }
+  return DT_OK;
+}
+
+extern "C" int dt_merge_states(int32_t n, const void* const* outs, const float* const* lses,
+                               const int32_t* src_dtype, const int32_t* src_lse_layout, void* dst_out,
+                               int32_t dst_dtype, float* dst_lse, int32_t dst_lse_layout, int32_t B, int32_t Sq,
+                               int32_t H, int32_t D, void* stream) {
+  if (int rc = check_dims(B, Sq, H, D)) return rc;
+  if (n <= 0 || n > DT_MAX_MERGE) {
+    set_error("merge of %d states: need 1..%d", n, DT_MAX_MERGE);
+    return DT_ERR_INVALID;
+  }
+  if (!outs || !lses || !dst_out) {
+    set_error("null pointer argument");
+    return DT_ERR_INVALID;
+  }
+  MergeArgs a{};
+  a.n = n;
+  a.B = B; a.Sq = Sq; a.H = H;
+  for (int i = 0; i < n; ++i) {
+    if (!outs[i] || !lses[i] || !aligned16(outs[i])) {
+      set_error("state %d: null or misaligned pointer", i);
+      return DT_ERR_INVALID;
+    }
+    a.out[i] = outs[i];
+    a.lse[i] = lses[i];
+    const int dtp = src_dtype ? src_dtype[i] : DT_BF16;
+    const int lay = src_lse_layout ? src_lse_layout[i] : DT_LSE_BHS;
+    if ((dtp != DT_BF16 && dtp != DT_FP32) || (lay != DT_LSE_BHS && lay != DT_LSE_BSH)) {
+      set_error("state %d: bad dtype/layout code", i);
+      return DT_ERR_INVALID;
+    }
+    if (dtp == DT_FP32) a.fp32_mask |= (1ull << i);
+    if (lay == DT_LSE_BSH) a.bsh_mask |= (1ull << i);
+  }
+  if (!aligned16(dst_out) || (dst_dtype != DT_BF16 && dst_dtype != DT_FP32) ||
+      (dst_lse_layout != DT_LSE_BHS && dst_lse_layout != DT_LSE_BSH)) {
+    set_error("bad destination pointer/dtype/layout");
+    return DT_ERR_INVALID;
+  }
+  a.dst_out = dst_out;
+  a.dst_lse = dst_lse;
+  a.dst_fp32 = dst_dtype == DT_FP32;
+  a.dst_bsh = dst_lse_layout == DT_LSE_BSH;
+  return launch_merge(a, D, (hipStream_t)stream);
+}
+
+static int state_copy(const void* src_out, int32_t src_dtype, const float* src_lse, int32_t src_layout, void* dst_out,
+                      int32_t dst_dtype, float* dst_lse, int32_t dst_layout, int32_t B, int32_t Sq, int32_t H,
+                      int32_t D, void* stream) {
+  if (int rc = check_dims(B, Sq, H, D)) return rc;
+  if (!src_out || !dst_out || !aligned16(src_out) || !aligned16(dst_out)) {
+    set_error("null or misaligned state pointer");
+    return DT_ERR_INVALID;
+  }
+  if ((src_dtype != DT_BF16 && src_dtype != DT_FP32) || (dst_dtype != DT_BF16 && dst_dtype != DT_FP32) ||
+      (src_layout != DT_LSE_BHS && src_layout != DT_LSE_BSH) || (dst_layout != DT_LSE_BHS && dst_layout != DT_LSE_BSH)) {
+    set_error("bad dtype/layout code");
+    return DT_ERR_INVALID;
+  }
+  CopyArgs a{};
+  a.src_out = src_out; a.src_lse = src_lse; a.dst_out = dst_out; a.dst_lse = dst_lse;
+  a.B = B; a.Sq = Sq; a.H = H;
+  a.src_fp32 = src_dtype == DT_FP32; a.src_bsh = src_layout == DT_LSE_BSH;
+  a.dst_fp32 = dst_dtype == DT_FP32; a.dst_bsh = dst_layout == DT_LSE_BSH;
+  return launch_copy(a, D, (hipStream_t)stream);
+}
+
+extern "C" int dt_cache_store(const void* src_out, int32_t src_dtype, const float* src_lse, int32_t src_lse_layout,
+                              void* slot_out, float* slot_lse, int32_t B, int32_t Sq, int32_t H, int32_t D,
+                              void* stream) {
+  return state_copy(src_out, src_dtype, src_lse, src_lse_layout, slot_out, DT_BF16, slot_lse, DT_LSE_BHS, B, Sq, H, D,
+                    stream);
+}
+
+extern "C" int dt_cache_load(const void* slot_out, const float* slot_lse, void* dst_out, int32_t dst_dtype,
+                             float* dst_lse, int32_t dst_lse_layout, int32_t B, int32_t Sq, int32_t H, int32_t D,
+                             void* stream) {
+  return state_copy(slot_out, DT_BF16, slot_lse, DT_LSE_BHS, dst_out, dst_dtype, dst_lse, dst_lse_layout, B, Sq, H, D,
+                    stream);
+}
+
+static int check_sched(const uint8_t* mask, int32_t T, int32_t L, int32_t C, const void* a, const void* b,
+                       const void* c) {
+  if (!mask || !a || !b || !c) {
+    set_error("null pointer argument");
+    return DT_ERR_INVALID;
+  }
+  if (T <= 0 || L <= 0 || C <= 0 || C > 1024) {
+    set_error("schedule dims T=%d L=%d C=%d out of range (C <= 1024)", T, L, C);
+    return DT_ERR_INVALID;
+  }
+  return DT_OK;
+}
+
+extern "C" int dt_build_schedule(const uint8_t* mask, int32_t T, int32_t L, int32_t C, int32_t t, int32_t l,
+                                 int32_t diag, int32_t* compute_ids, int32_t* reuse_ids, int32_t* counts,
+                                 void* stream) {
+  if (int rc = check_sched(mask, T, L, C, compute_ids, reuse_ids, counts)) return rc;
+  if (t < 0 || t >= T || l < 0 || l >= L) {
+    set_error("(t,l)=(%d,%d) outside [0,%d)x[0,%d)", t, l, T, L);
+    return DT_ERR_INVALID;
+  }
+  hipLaunchKernelGGL(build_schedule_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, mask, T, L, C, t * L + l, diag,
+                     compute_ids, reuse_ids, counts);
+  return hip_fail(hipGetLastError(), "build_schedule launch");
+}
+
+extern "C" int dt_build_schedule_table(const uint8_t* mask, int32_t T, int32_t L, int32_t C, int32_t diag,
+                                       int32_t* compute_ids, int32_t* reuse_ids, int32_t* counts, void* stream) {
+  if (int rc = check_sched(mask, T, L, C, compute_ids, reuse_ids, counts)) return rc;
+  hipLaunchKernelGGL(build_schedule_kernel, dim3((unsigned)(T * L)), dim3(64), 0, (hipStream_t)stream, mask, T, L, C,
+                     0, diag, compute_ids, reuse_ids, counts);
+  return hip_fail(hipGetLastError(), "build_schedule_table launch");
+}
+
+extern "C" int dt_rel_l1_sums(const float* a, const float* b, int64_t n, double* sums, void* stream) {
+  if (!a || !b || !sums || n < 0) {
+    set_error("null pointer or negative length");
+    return DT_ERR_INVALID;
+  }
+  if (!aligned16(a) || !aligned16(b)) {
+    set_error("inputs must be 16-byte aligned");
+    return DT_ERR_INVALID;
+  }
+  if (n == 0) return DT_OK;
+  int64_t wgs = (n / 4 + kThreads - 1) / kThreads;
+  if (wgs > 2048) wgs = 2048;
+  if (wgs < 1) wgs = 1;
+  hipLaunchKernelGGL(rel_l1_sums_kernel, dim3((unsigned)wgs), dim3(kThreads), 0, (hipStream_t)stream, a, b, n, sums);
+  return hip_fail(hipGetLastError(), "rel_l1_sums launch");
+}

@@ -1,0 +1,167 @@
+/*
+ * libditango_hip.so -- C ABI of the MI355X (gfx950) kernels behind DiTango's
+ * cached block attention.
+ *
+ * The reference (chen-yy20/ditango) is pure Python; the GPU arithmetic of this
+ * path lives in the third-party flash_attn wheel and in eager torch ops.  Each
+ * entry point below replaces one of those call sites; the citation names the
+ * reference interface it stands in for.  All pointers are device pointers
+ * unless the comment says "host".  Every function enqueues work on `stream`
+ * (a hipStream_t passed as void*), never synchronises, never allocates, and
+ * returns DT_OK or a negative error code; dt_last_error() then holds a
+ * message for the calling thread.
+ *
+ * Tensor layouts (element strides, innermost dimension contiguous):
+ *   q / out state   bf16  [B, Sq, H, D]
+ *   k, v chunk      bf16  [B, Sk, H, D]
+ *   lse state       fp32  [B, H, Sq]     (DT_LSE_BHS, flash-attn's layout)
+ *                   fp32  [B, Sq, H]     (DT_LSE_BSH, the running layout
+ *                                         [B,S,H,1] of utils.py:49)
+ * D is 64 or 128.  Base pointers and the q/k/v token, head and batch strides
+ * must keep every row 16-byte aligned.
+ */
+#ifndef DITANGO_HIP_H
+#define DITANGO_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DT_OK 0
+#define DT_ERR_INVALID (-1)     /* bad argument (shape, alignment, null pointer, limit) */
+#define DT_ERR_UNSUPPORTED (-2) /* valid request this build does not cover (e.g. head dim) */
+#define DT_ERR_HIP (-3)         /* a HIP runtime call failed */
+
+#define DT_BF16 0
+#define DT_FP32 1
+
+#define DT_LSE_BHS 0
+#define DT_LSE_BSH 1
+
+#define DT_MAX_CHUNKS 40       /* KV chunks one launch can address */
+#define DT_MAX_JOBS 40         /* attention states one launch can produce */
+#define DT_MAX_JOB_ENTRIES 64  /* total chunk references over all jobs of a launch */
+#define DT_MAX_MERGE 40        /* states one merge launch can combine */
+
+int dt_version(void);
+const char* dt_last_error(void);
+
+/*
+ * One KV chunk of non-causal attention: out = softmax(q k^T * scale) v and the
+ * natural-log lse.  Replaces
+ *   flash_attn_func(q, k, v, dropout_p=0.0, return_attn_probs=True)
+ * as called at core/attention.py:137-143 and :185-191 (first two results).
+ * out is bf16 [B,Sq,H,D] contiguous, lse fp32 [B,H,Sq] contiguous.
+ * softmax_scale <= 0 selects D^-0.5 (flash_attn's default).
+ */
+int dt_attn_chunk_fwd(const void* q, const void* k, const void* v, void* out, float* lse,
+                      int32_t B, int32_t Sq, int32_t Sk, int32_t H, int32_t D,
+                      int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
+                      int64_t kv_stride_b, int64_t kv_stride_s, int64_t kv_stride_h,
+                      float softmax_scale, void* stream);
+
+/*
+ * Several attention states in one launch.  Job j attends q to the
+ * concatenation of the chunks job_chunks[job_begin[j] .. job_begin[j+1]) and
+ * writes ONE state (out_ptrs[j], lse_ptrs[j]).  A job of one chunk is the call
+ * above; a job of several chunks equals computing each chunk separately and
+ * folding the results with update_out_and_lse (core/attention.py:185-196,
+ * utils.py:42-84), i.e. the "fresh" state of a target block.
+ * k_ptrs/v_ptrs/kv_lens/kv_stride_b, job_begin, job_chunks, out_ptrs,
+ * lse_ptrs are HOST arrays; they are copied into the kernel arguments.
+ * All chunks share kv_stride_s / kv_stride_h.
+ */
+int dt_attn_jobs_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D,
+                     int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
+                     int32_t n_chunks, const void* const* k_ptrs, const void* const* v_ptrs,
+                     const int32_t* kv_lens, const int64_t* kv_stride_b,
+                     int64_t kv_stride_s, int64_t kv_stride_h,
+                     int32_t n_jobs, const int32_t* job_begin, const int32_t* job_chunks,
+                     void* const* out_ptrs, float* const* lse_ptrs,
+                     float softmax_scale, void* stream);
+
+/*
+ * Same, driven by a schedule that lives in device memory (dt_build_schedule*):
+ * job j (0 <= j < max_jobs) is active iff j < *dev_count and computes the
+ * single chunk id dev_compute_ids[j], writing its state into cache slot
+ * `id` of the state arena (slot_out + id*slot_out_stride elements,
+ * slot_lse + id*slot_lse_stride elements), or into (diag_out, diag_lse) when
+ * id == diag -- the local chunk is recomputed on every call and never cached
+ * (core/attention.py:137-144,193-194).  max_jobs sizes the grid; the host
+ * never reads the schedule.
+ */
+int dt_attn_sched_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D,
+                      int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
+                      int32_t n_chunks, const void* const* k_ptrs, const void* const* v_ptrs,
+                      const int32_t* kv_lens, const int64_t* kv_stride_b,
+                      int64_t kv_stride_s, int64_t kv_stride_h,
+                      const int32_t* dev_compute_ids, const int32_t* dev_count, int32_t max_jobs,
+                      void* slot_out, int64_t slot_out_stride, float* slot_lse, int64_t slot_lse_stride,
+                      int32_t diag, void* diag_out, float* diag_lse,
+                      float softmax_scale, void* stream);
+
+/*
+ * N-way LSE merge: lse = logsumexp_i lse_i, out = sum_i exp(lse_i - lse) out_i.
+ * Replaces the chain of update_out_and_lse / _update_out_and_lse calls
+ * (utils.py:24-84; called at core/attention.py:116,144,194,196,213 and
+ * core/cache.py:42) with one pass over HBM.  outs[i] is [B,Sq,H,D] contiguous
+ * in src_dtype[i]; lses[i] is fp32 in src_lse_layout[i].  A state whose lse is
+ * -inf contributes nothing.  dst may alias one of the inputs of the same dtype
+ * and layout (in-place cache coarsening, core/cache.py:28-46).  A pointer may
+ * appear more than once (the reference can merge the local chunk twice,
+ * core/attention.py:120-145 followed by :193-194).
+ * outs, lses, src_dtype, src_lse_layout are HOST arrays of length n.
+ */
+int dt_merge_states(int32_t n, const void* const* outs, const float* const* lses,
+                    const int32_t* src_dtype, const int32_t* src_lse_layout,
+                    void* dst_out, int32_t dst_dtype, float* dst_lse, int32_t dst_lse_layout,
+                    int32_t B, int32_t Sq, int32_t H, int32_t D, void* stream);
+
+/*
+ * State cache store / load: one streaming copy of (out, lse) between a caller
+ * tensor and a cache slot (out bf16 [B,Sq,H,D], lse fp32 [B,H,Sq]).  Replaces
+ * proCache.store_block / get_block (core/cache.py:75-84), which in the
+ * reference keep Python references to fp32 tensors.
+ */
+int dt_cache_store(const void* src_out, int32_t src_dtype, const float* src_lse, int32_t src_lse_layout,
+                   void* slot_out, float* slot_lse,
+                   int32_t B, int32_t Sq, int32_t H, int32_t D, void* stream);
+int dt_cache_load(const void* slot_out, const float* slot_lse,
+                  void* dst_out, int32_t dst_dtype, float* dst_lse, int32_t dst_lse_layout,
+                  int32_t B, int32_t Sq, int32_t H, int32_t D, void* stream);
+
+/*
+ * Device-side schedule builder.  mask is uint8 [T,L,C] (1 = reuse the cached
+ * state of chunk c at step t, layer l; 0 = recompute).  For row (t,l):
+ *   compute_ids = [diag (if 0 <= diag < C)] + ascending {c != diag : mask == 0}
+ *   reuse_ids   = ascending {c != diag : mask != 0}
+ *   counts      = {len(compute_ids), len(reuse_ids)}
+ * Unused tail entries are set to -1.  The reference derives the equivalent
+ * decision on the host from the stride table (core/attention.py:90-116,
+ * core/redundancy_map.py:49-87); this kernel is the per-chunk generalisation.
+ * dt_build_schedule handles one row (outputs int32 [C], [C], [2]);
+ * dt_build_schedule_table all rows (outputs int32 [T,L,C], [T,L,C], [T,L,2]).
+ * C <= 1024.
+ */
+int dt_build_schedule(const uint8_t* mask, int32_t T, int32_t L, int32_t C, int32_t t, int32_t l,
+                      int32_t diag, int32_t* compute_ids, int32_t* reuse_ids, int32_t* counts,
+                      void* stream);
+int dt_build_schedule_table(const uint8_t* mask, int32_t T, int32_t L, int32_t C, int32_t diag,
+                            int32_t* compute_ids, int32_t* reuse_ids, int32_t* counts, void* stream);
+
+/*
+ * Relative-L1 partial sums for the profiling mode: accumulates, over entries
+ * where neither input is NaN, sums[0] += |a-b|, sums[1] += |a|, sums[2] += |b|,
+ * sums[3] += count (all fp64, device memory, caller zeroes them).  Replaces the
+ * mask-select / abs / mean chain with its three host syncs in rel_l1
+ * (utils.py:214-241), used by record_out_redundancy
+ * (core/redundancy_map.py:174-197).  a, b are fp32, n elements.
+ */
+int dt_rel_l1_sums(const float* a, const float* b, int64_t n, double* sums, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DITANGO_HIP_H */

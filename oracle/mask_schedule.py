@@ -1,0 +1,99 @@
+"""Explicit per-chunk mask mode (CPU oracle; test infrastructure only).
+
+The reference can only say "recompute one aligned block of ``stride`` chunks
+plus the local chunk" (core/attention.py:100-216).  The benchmark
+configurations instead give a seeded mask ``M[t, l, c]`` (1 = reuse the cached
+state of chunk ``c``, 0 = recompute it).  This mode has no counterpart in the
+reference; its semantics are fixed here and the HIP schedule builder has to
+reproduce them bit-exactly:
+
+* ``compute(t,l) = {c : M[t,l,c] == 0} U {diag}``; ``reuse(t,l)`` is the rest.
+  ``diag`` is the local ("diagonal") chunk, which the reference always
+  recomputes and never caches (core/attention.py:137-144,193-194);
+  ``diag = -1`` means there is none.
+* compute list order: ``diag`` first (if any), then ascending chunk id.
+  reuse list order: ascending chunk id.
+* every computed chunk other than ``diag`` overwrites the cached state of that
+  chunk; a reused chunk reads the most recently stored state (the lifetime rule
+  of ``store_block``, core/cache.py:82-84).  Reusing a chunk that was never
+  stored is an error.
+* merge order: reused (ascending), then ``diag``, then the other fresh chunks.
+"""
+from __future__ import annotations
+
+from typing import Callable, Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+
+
+def build_schedule(mask_row: Sequence[int], diag: int = -1) -> Tuple[List[int], List[int]]:
+    """(compute_ids, reuse_ids) for one ``(t, l)`` row of the mask."""
+    C = len(mask_row)
+    compute: List[int] = []
+    reuse: List[int] = []
+    if 0 <= diag < C:
+        compute.append(diag)
+    for c in range(C):
+        if c == diag:
+            continue
+        if int(mask_row[c]) == 0:
+            compute.append(c)
+        else:
+            reuse.append(c)
+    return compute, reuse
+
+
+def build_schedule_table(mask: np.ndarray, diag: int = -1) -> Tuple[np.ndarray, np.ndarray, np.ndarray]:
+    """All rows at once: mask ``[T,L,C]`` -> (compute_ids ``[T,L,C]`` int32,
+    reuse_ids ``[T,L,C]`` int32, counts ``[T,L,2]`` int32); unused tail entries are -1."""
+    T, L, C = mask.shape
+    comp = -np.ones((T, L, C), dtype=np.int32)
+    reu = -np.ones((T, L, C), dtype=np.int32)
+    cnt = np.zeros((T, L, 2), dtype=np.int32)
+    for t in range(T):
+        for l in range(L):
+            c_ids, r_ids = build_schedule(mask[t, l], diag)
+            comp[t, l, :len(c_ids)] = c_ids
+            reu[t, l, :len(r_ids)] = r_ids
+            cnt[t, l] = (len(c_ids), len(r_ids))
+    return comp, reu, cnt
+
+
+def seeded_mask(T: int, L: int, C: int, reuse_prob: float, seed: int, diag: int = -1,
+                cold_first_step: bool = True) -> np.ndarray:
+    """The benchmark masks: Bernoulli(``reuse_prob``) per entry from
+    ``numpy.random.default_rng(seed)``; the diagonal chunk is never reused and
+    nothing is reused at step 0 (cold cache)."""
+    rng = np.random.default_rng(seed)
+    m = (rng.random((T, L, C)) < reuse_prob).astype(np.uint8)
+    if 0 <= diag < C:
+        m[:, :, diag] = 0
+    if cold_first_step:
+        m[0] = 0
+    return m
+
+
+class MaskCacheOracle:
+    """One layer's cache in mask mode, with opaque payloads (see state_machine)."""
+
+    def __init__(self, n_chunks: int, diag: int = -1):
+        self.C = n_chunks
+        self.diag = diag
+        self.slots: List[Optional[object]] = [None] * n_chunks
+
+    def call(self, mask_row: Sequence[int], attn_fn: Callable[[int], object],
+             merge_all_fn: Callable[[List[object]], object],
+             store_fn: Callable[[object], object] = lambda s: s):
+        compute, reuse = build_schedule(mask_row, self.diag)
+        states: List[object] = []
+        for c in reuse:
+            if self.slots[c] is None:
+                raise RuntimeError(f"mask asks to reuse chunk {c} but no state was ever stored for it")
+            states.append(self.slots[c])
+        for c in compute:
+            st = attn_fn(c)
+            if c != self.diag:
+                st = store_fn(st)
+                self.slots[c] = st
+            states.append(st)
+        return merge_all_fn(states), compute, reuse

@@ -1,0 +1,202 @@
+"""Parity of the HIP kernels (through the C ABI) against the CPU oracle.
+
+Tolerances (the stated bar): out max-abs <= 2e-2 (bf16), lse <= 1e-3 (fp32).
+The tests additionally bound the error relative to the magnitude of the exact
+result, because attention outputs over thousands of keys are far smaller than 1.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import attention_math as om
+from oracle import mask_schedule as ms
+
+pytestmark = pytest.mark.gpu
+
+OUT_TOL = 2e-2
+LSE_TOL = 1e-3
+
+
+def _qkv(B, Sq, Sk, H, D, seed, norm=None):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, Sq, H, D, generator=g)
+    k = torch.randn(B, Sk, H, D, generator=g)
+    v = torch.randn(B, Sk, H, D, generator=g)
+    if norm == "rms":
+        q = q / q.pow(2).mean(-1, keepdim=True).sqrt()
+        k = k / k.pow(2).mean(-1, keepdim=True).sqrt()
+    elif norm == "layer":
+        q = torch.nn.functional.layer_norm(q, (D,))
+        k = torch.nn.functional.layer_norm(k, (D,))
+    return q.bfloat16(), k.bfloat16(), v.bfloat16()
+
+
+def _check_state(out, lse, ref_out, ref_lse, what=""):
+    out = out.float().cpu()
+    lse = lse.float().cpu()
+    err = (out - ref_out).abs().max().item()
+    lerr = (lse - ref_lse).abs().max().item()
+    rel = (out - ref_out).norm().item() / max(ref_out.norm().item(), 1e-30)
+    print(f"{what} out max-abs {err:.3e} rel-l2 {rel:.3e} lse max-abs {lerr:.3e}", flush=True)
+    assert err <= OUT_TOL, f"{what}: out max-abs {err}"
+    assert lerr <= LSE_TOL, f"{what}: lse max-abs {lerr}"
+    assert rel <= 1e-2, f"{what}: out relative l2 {rel}"
+
+
+@pytest.mark.parametrize("B,Sq,Sk,H,D", [
+    (1, 128, 64, 1, 128),
+    (1, 128, 128, 2, 128),
+    (1, 100, 77, 3, 128),      # ragged Sq and Sk
+    (2, 257, 333, 2, 128),     # batch > 1, several tiles, ragged
+    (1, 1, 1, 1, 128),         # smallest
+    (1, 128, 64, 1, 64),
+    (2, 190, 201, 3, 64),
+    (1, 33, 1000, 2, 64),
+])
+def test_chunk_attention_matches_oracle(hip, B, Sq, Sk, H, D):
+    print(f"case chunk B={B} Sq={Sq} Sk={Sk} H={H} D={D}", flush=True)
+    q, k, v = _qkv(B, Sq, Sk, H, D, seed=B * 1000 + Sq + Sk + D)
+    ref_out, ref_lse = om.chunk_attention(q, k, v)
+    out, lse = hip.attn_chunk_fwd(q.cuda(), k.cuda(), v.cuda())
+    torch.cuda.synchronize()
+    _check_state(out, lse, ref_out, ref_lse, "chunk")
+
+
+def test_chunk_attention_strided_inputs(hip):
+    """q/k/v as slices of a fused [B,S,3,H,D] projection (non-contiguous token stride)."""
+    B, S, H, D = 1, 300, 2, 128
+    g = torch.Generator().manual_seed(5)
+    qkv = torch.randn(B, S, 3, H, D, generator=g).bfloat16()
+    q, k, v = qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
+    ref_out, ref_lse = om.chunk_attention(q, k, v)
+    dq = qkv.cuda()
+    out, lse = hip.attn_chunk_fwd(dq[:, :, 0], dq[:, :, 1], dq[:, :, 2])
+    torch.cuda.synchronize()
+    _check_state(out, lse, ref_out, ref_lse, "strided")
+
+
+def test_multi_chunk_job_equals_merge_of_chunks(hip):
+    """One job over several chunks == folding per-chunk states with update_out_and_lse."""
+    B, Sq, H, D = 1, 200, 2, 128
+    lens = [64, 130, 0, 77, 1]
+    g = torch.Generator().manual_seed(11)
+    q = torch.randn(B, Sq, H, D, generator=g).bfloat16()
+    ks = [torch.randn(B, n, H, D, generator=g).bfloat16() for n in lens]
+    vs = [torch.randn(B, n, H, D, generator=g).bfloat16() for n in lens]
+    # oracle: literal fold
+    o = l = None
+    for k, v in zip(ks, vs):
+        if k.shape[1] == 0:
+            continue
+        bo, bl = om.chunk_attention(q, k, v)
+        o, l = om.update_out_and_lse(o, l, bo.bfloat16(), bl)
+    ref_out, ref_lse = o, l.squeeze(-1).transpose(1, 2)
+    full_out, full_lse = om.full_attention(q, ks, vs)
+    assert (full_out - ref_out).abs().max() < 5e-3  # the fold itself is pinned by full attention
+
+    dq = q.cuda()
+    table = hip.ChunkTable([k.cuda() for k in ks], [v.cuda() for v in vs])
+    outs = [torch.empty(B, Sq, H, D, dtype=torch.bfloat16, device="cuda") for _ in range(3)]
+    lses = [torch.empty(B, H, Sq, dtype=torch.float32, device="cuda") for _ in range(3)]
+    hip.attn_jobs_fwd(dq, table, [[0, 1, 2, 3, 4], [3], [2]], outs, lses)
+    torch.cuda.synchronize()
+    _check_state(outs[0], lses[0], full_out, full_lse, "job all chunks")
+    r3o, r3l = om.chunk_attention(q, ks[3], vs[3])
+    _check_state(outs[1], lses[1], r3o, r3l, "job chunk 3")
+    # a job whose only chunk is empty yields the neutral state
+    assert torch.isinf(lses[2]).all() and (lses[2] < 0).all()
+    assert (outs[2].float() == 0).all()
+
+
+@pytest.mark.parametrize("D,n,src_fp32", [(128, 1, False), (128, 5, False), (64, 8, False), (128, 3, True), (64, 33, False)])
+def test_merge_states_matches_closed_form(hip, D, n, src_fp32):
+    B, Sq, H = 2, 150, 3
+    g = torch.Generator().manual_seed(n * 7 + D)
+    outs = [torch.randn(B, Sq, H, D, generator=g) for _ in range(n)]
+    lses = [torch.randn(B, H, Sq, generator=g) * 3 for _ in range(n)]
+    if n >= 3:
+        lses[1][:, :, ::5] = -math.inf   # partially empty state
+    if not src_fp32:
+        outs = [o.bfloat16() for o in outs]
+    ref_out, ref_lse = om.merge_states_closed_form(outs, lses)
+    d_out, d_lse = hip.merge_states([o.cuda() for o in outs], [l.cuda() for l in lses])
+    torch.cuda.synchronize()
+    assert (d_out.cpu() - ref_out).abs().max() < 1e-5 * max(1, n)
+    assert (d_lse.cpu() - ref_lse).abs().max() < 1e-5
+    # literal sigmoid/logsigmoid fold of the reference agrees with the fused kernel
+    o = l = None
+    for bo, bl in zip(outs, lses):
+        o, l = om.update_out_and_lse(o, l, bo, bl)
+    finite = torch.isfinite(l.squeeze(-1).transpose(1, 2))
+    assert (d_lse.cpu()[finite] - l.squeeze(-1).transpose(1, 2)[finite]).abs().max() < 1e-4
+
+
+def test_merge_all_empty_and_layouts(hip):
+    B, Sq, H, D = 1, 70, 2, 128
+    g = torch.Generator().manual_seed(3)
+    outs = [torch.randn(B, Sq, H, D, generator=g).bfloat16() for _ in range(2)]
+    lses = [torch.full((B, H, Sq), -math.inf) for _ in range(2)]
+    d_out, d_lse = hip.merge_states([o.cuda() for o in outs], [l.cuda() for l in lses])
+    torch.cuda.synchronize()
+    assert (d_out == 0).all() and torch.isinf(d_lse).all()
+    # running layout [B,S,H,1] in, [B,S,H,1] out, bf16 destination, in place
+    lses = [torch.randn(B, H, Sq, generator=g) for _ in range(2)]
+    ref_out, ref_lse = om.merge_states_closed_form(outs, lses)
+    a_out = outs[0].cuda()
+    a_lse = lses[0].transpose(1, 2).contiguous().unsqueeze(-1).cuda()   # [B,S,H,1]
+    b_out, b_lse = outs[1].cuda(), lses[1].cuda()
+    r_out, r_lse = hip.merge_states([a_out, b_out], [a_lse, b_lse], dst_out=a_out, dst_lse=a_lse)
+    torch.cuda.synchronize()
+    assert r_out.data_ptr() == a_out.data_ptr()
+    assert (a_out.float().cpu() - ref_out).abs().max() < 2e-2
+    assert (a_lse.cpu().squeeze(-1).transpose(1, 2) - ref_lse).abs().max() < 1e-5
+
+
+def test_cache_store_load_roundtrip(hip):
+    B, Sq, H, D = 2, 131, 3, 64
+    g = torch.Generator().manual_seed(9)
+    src = torch.randn(B, Sq, H, D, generator=g)
+    lse = torch.randn(B, Sq, H, 1, generator=g)
+    slot_out = torch.empty(B, Sq, H, D, dtype=torch.bfloat16, device="cuda")
+    slot_lse = torch.empty(B, H, Sq, dtype=torch.float32, device="cuda")
+    hip.cache_store(src.cuda(), lse.cuda(), slot_out, slot_lse)
+    torch.cuda.synchronize()
+    assert torch.equal(slot_out.cpu(), src.bfloat16())            # round-to-nearest-even, bit exact
+    assert torch.equal(slot_lse.cpu(), lse.squeeze(-1).transpose(1, 2))
+    o, l = hip.cache_load(slot_out, slot_lse, torch.float32, dst_lse_bsh=True)
+    torch.cuda.synchronize()
+    assert torch.equal(o.cpu(), src.bfloat16().float())
+    assert torch.equal(l.cpu(), lse)
+
+
+@pytest.mark.parametrize("T,L,C,p,diag", [(3, 4, 8, 0.5, 0), (2, 3, 32, 0.9, -1), (2, 2, 1, 0.5, 0), (1, 2, 100, 0.3, 77), (2, 2, 64, 0.0, 3), (1, 1, 65, 1.0, 64)])
+def test_schedule_builder_bit_exact(hip, T, L, C, p, diag):
+    mask = ms.seeded_mask(T, L, C, p, seed=C + T, diag=diag, cold_first_step=False)
+    comp, reu, cnt = ms.build_schedule_table(mask, diag)
+    dmask = torch.from_numpy(mask).cuda()
+    dcomp, dreu, dcnt = hip.build_schedule_table(dmask, diag)
+    torch.cuda.synchronize()
+    assert np.array_equal(dcomp.cpu().numpy(), comp)
+    assert np.array_equal(dreu.cpu().numpy(), reu)
+    assert np.array_equal(dcnt.cpu().numpy(), cnt)
+    t, l = T - 1, L - 1
+    c1, r1, n1 = hip.build_schedule(dmask, t, l, diag)
+    torch.cuda.synchronize()
+    assert np.array_equal(c1.cpu().numpy(), comp[t, l])
+    assert np.array_equal(r1.cpu().numpy(), reu[t, l])
+    assert np.array_equal(n1.cpu().numpy(), cnt[t, l])
+
+
+def test_rel_l1_sums(hip):
+    g = torch.Generator().manual_seed(2)
+    a = torch.randn(1, 77, 3, 64, generator=g)
+    b = a + 0.05 * torch.randn(1, 77, 3, 64, generator=g)
+    a[0, 3, 1, 5] = float("nan")
+    b[0, 9, 2, 7] = float("nan")
+    ref = om.rel_l1(a, b)
+    s = hip.rel_l1_sums(a.cuda(), b.cuda()).cpu()
+    val = (s[0] / s[3]).item() / ((s[2] / s[3]).item() + 1e-8)
+    assert s[3].item() == a.numel() - 2
+    assert abs(val - ref) < 1e-5 * max(1.0, abs(ref))
