@@ -1,0 +1,357 @@
+"""Cached block attention: the per-layer driver.
+
+API of the reference's ``proAttention`` (core/attention.py:20-419):
+``proAttention(layer_id, isp_group).attn(query, key, value)`` with inputs
+``[B, S, H, D]`` bf16 and an fp32 result of the same shape.
+
+One GPU plays one sequence-parallel rank.  Where the reference interleaves ring
+hops, one ``flash_attn_func`` call per chunk and one eager merge chain per state,
+this driver first derives the whole call's schedule on the host from the same
+integer state (stride table, rotating target pointer, cache occupancy), then
+issues
+
+1. ONE attention launch that produces every state of the call (``dt_attn_jobs_fwd``:
+   the local chunk, and the fresh state of the target block as a single multi-chunk
+   job written straight into its cache tensors), and
+2. ONE fused N-way merge (``dt_merge_states``) over the cached states, the local
+   state and the fresh states.
+
+Which chunk the ring would have delivered at each hop follows from tracking, as
+integers, the chunk id every ring position holds (``plan_call``); the chunk order, the reuse set, the cache writes and the pointer
+movement match the reference step for step, including the case in which it
+merges the local chunk twice (core/attention.py:120-145 followed by :193-194).
+
+Mask mode (an addition, see ``RedundancyMap.set_chunk_mask``): the chunks to
+compute come from a device-resident schedule and every state lives in a
+contiguous per-layer arena.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import List, Optional, Tuple
+
+import torch
+
+from .. import _hip
+from ..logger import init_logger
+from ..timer import get_timer
+from ..utils import get_timestep
+from .cache import proCache
+from .config import get_config
+from .redundancy_map import get_redundancy_map
+
+logger = init_logger(__name__)
+
+
+@dataclass
+class Job:
+    chunks: Tuple[int, ...]   # KV chunk ids attended to as one concatenated sequence
+    kind: str                 # 'local' (computed while the first fetch is in flight), 'own', 'fresh'
+    store_slot: Optional[int] = None  # cache block the state is stored in, if any
+
+
+@dataclass
+class CallPlan:
+    """The schedule of one ``attn`` call (what has to match the reference bit for bit)."""
+    timestep: int
+    layer_id: int
+    rank: int
+    curr_stride: int
+    next_stride: int
+    reuse_probed: List[int] = field(default_factory=list)
+    reuse_merged: List[int] = field(default_factory=list)
+    computed: List[Tuple[int, str]] = field(default_factory=list)
+    jobs: List[Job] = field(default_factory=list)
+    stores: List[Tuple[int, Tuple[int, ...]]] = field(default_factory=list)
+    flushes: List[Tuple[int, ...]] = field(default_factory=list)
+    target_after: int = 0
+    nblk_after: int = 0
+    occupancy_after: List[bool] = field(default_factory=list)
+
+
+def plan_call(N: int, r: int, curr: int, nxt: int, targets: List[int], use_ditango: bool = True,
+              small_ring_stride: int = 8) -> Tuple[CallPlan, List[int]]:
+    """Schedule of one call from the integer state alone (core/attention.py:100-216).
+
+    ``targets[x]`` is the rotating target pointer of ring position ``x``; all positions
+    are tracked because which chunk a hop delivers depends on what the NEIGHBOUR fetched:
+    after a stride-1 step the pointers of one block's ranks can point into different
+    target blocks, and the reference then hands chunks of other blocks round the ring.
+    ``held[x]`` is the chunk id position ``x`` has in hand; an exchange replaces it by
+    the id held by the position it receives from (ring sends to ``x-1``, receives from
+    ``x+1`` inside a small ring of ``ss`` positions, :160-161; an inter-ring hop receives
+    from ``x+ss`` inside the block, :162-163).
+
+    Returns (plan of position ``r`` without the cache-dependent fields, new pointers).
+    """
+    assert N % curr == 0, f"Does not support this ISP stride {curr} for SP size {N}"
+    plan = CallPlan(0, 0, r, curr, nxt)
+    nblk = N // curr
+    targets = list(targets)
+    tb_of = [targets[x] // curr for x in range(N)]  # read before the pointer reset (:104)
+    lb, tb = r // curr, tb_of[r]
+    if curr == N:
+        targets = list(range(N))  # :107-108
+    else:
+        plan.reuse_probed = [(tb + 1 + i) % nblk for i in range(nblk - 1)]
+    # first fetch (:120-145): position x takes the chunk of the same inner offset in its target block
+    held = list(range(N))
+    fetching = [targets[x] != x for x in range(N)]
+    if any(fetching):
+        if not all(fetching):
+            raise RuntimeError("ring positions disagree on whether to fetch first: the reference's exchange would hang "
+                               "(the first step of a run has to be a full-stride step)")
+        src = [tb_of[x] * curr + x % curr for x in range(N)]
+        dst = [((x // curr - (tb_of[x] - x // curr)) % nblk) * curr + x % curr for x in range(N)]
+        for x in range(N):
+            if dst[src[x]] != x:
+                raise RuntimeError(f"unpaired first fetch at ring position {x}: the reference's exchange would hang")
+        held = [held[src[x]] for x in range(N)]
+        plan.computed.append((r, "local"))
+        plan.jobs.append(Job((r,), "local"))
+    upd = 1 if curr == N else curr
+    ss = curr
+    if curr > small_ring_stride and use_ditango:
+        assert curr % small_ring_stride == 0, f"Does not support this ISP stride {curr} for overlap ring strategy"
+        ss = small_ring_stride
+    nlarge = curr // ss
+    fresh: List[int] = []
+    cnt = 0
+    for i in range(nlarge):
+        for j in range(ss):
+            c = held[r]
+            if lb == tb and i == 0 and j == 0:
+                plan.computed.append((c, "own"))
+                plan.jobs.append(Job((c,), "own"))
+            else:
+                plan.computed.append((c, "fresh"))
+                fresh.append(c)
+            cnt += 1
+            if j + 1 != ss:
+                held = [held[(x + 1) % ss + x // ss * ss] for x in range(N)]
+            elif i + 1 != nlarge:
+                held = [held[(x + ss) % curr + x // curr * curr] for x in range(N)]
+            if cnt == upd:
+                if fresh:
+                    slot = None
+                    if nxt != N:
+                        slot = targets[r] if curr == N else tb
+                        plan.stores.append((slot, tuple(fresh)))
+                    plan.flushes.append(tuple(fresh))
+                    plan.jobs.append(Job(tuple(fresh), "fresh", slot))
+                targets = [(tg + cnt) % N for tg in targets]  # every position flushes in the same iteration
+                fresh = []
+                cnt = 0
+    plan.target_after = targets[r]
+    return plan, targets
+
+
+def _as4d(t: torch.Tensor, B: int) -> torch.Tensor:
+    """Packed ``[B*S, H, D]`` (the varlen entry's layout) viewed as ``[B, S, H, D]``."""
+    return t if t.dim() == 4 else t.view(B, t.shape[0] // B, t.shape[1], t.shape[2])
+
+
+class proAttention:
+    def __init__(self, layer_id: int, isp_group, dry_run: bool = False):
+        self.group = isp_group
+        self.isp_size = self.group.world_size
+        self.global_rank = getattr(get_config(), "rank", 0) if get_config() is not None else 0
+        self.local_chunk_id = self.group.rank_in_group
+        self.layer_id = layer_id
+        self.target_chunk_id = self.local_chunk_id // self.isp_size  # core/attention.py:27
+        # pointers of all ring positions (each starts at position // isp_size = 0); see plan_call
+        self._ring_targets = [x // self.isp_size for x in range(self.isp_size)]
+        self.cache = proCache(isp_size=self.isp_size, layer_id=layer_id)
+        cfg = get_config()
+        self.use_ditango = cfg.use_ditango if cfg is not None else True
+        self.small_ring_stride = 8
+        self.measure_memory = False
+        self.dry_run = dry_run  # plan and book-keep only (host tests of the schedule); computes nothing
+        self.last_plan: Optional[CallPlan] = None
+        self.last_lse: Optional[torch.Tensor] = None  # merged lse of the last call, fp32 [B,S,H,1]
+        if self.layer_id == 0:
+            logger.info(f"R{self.global_rank}L{layer_id} | cached block attention on HIP kernels (gfx950)")
+
+    # ---- stride mode ------------------------------------------------------------------------------
+    def _strides(self, timestep: int) -> Tuple[int, int]:
+        rm = get_redundancy_map()
+        return rm.get_curr_isp_stride(timestep, self.layer_id), rm.get_next_isp_stride(timestep, self.layer_id)
+
+    @get_timer("oAttn")
+    def attn(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor) -> Optional[torch.Tensor]:
+        """query ``[B,Sq,H,D]``, key/value ``[B,Sk,H,D]`` = this rank's shard (bf16).
+        Returns fp32 ``[B,Sq,H,D]`` (core/attention.py:74-237)."""
+        rm = get_redundancy_map()
+        if rm is not None and rm.chunk_mask is not None and not self.dry_run:
+            return self._attn_masked(query, key, value)
+        timestep = get_timestep()
+        N, r = self.isp_size, self.local_chunk_id
+        curr, nxt = self._strides(timestep)
+        if timestep == 0 and value is not None:
+            self.cache.set_block_size_mb(value)  # :93-94
+        if not self.dry_run and not self.cache.pass_memory_check(nxt, self.layer_id):  # :97-98
+            nxt = N
+        if self._ring_targets[r] != self.target_chunk_id:  # the pointer was set from outside: same offset everywhere
+            shift = (self.target_chunk_id - self._ring_targets[r]) % N
+            self._ring_targets = [(tg + shift) % N for tg in self._ring_targets]
+        plan, new_targets = plan_call(N, r, curr, nxt, self._ring_targets, self.use_ditango, self.small_ring_stride)
+        new_target = new_targets[r]
+        plan.timestep, plan.layer_id = timestep, self.layer_id
+
+        # 1. cached states of the blocks that are not recomputed (:107-116)
+        merge_outs, merge_lses = [], []
+        for b in plan.reuse_probed:
+            c_out, c_lse = self.cache.get_block(b)
+            if c_lse is not None:
+                plan.reuse_merged.append(b)
+                merge_outs.append(c_out)
+                merge_lses.append(c_lse)
+
+        out = None
+        if self.dry_run:
+            for job in plan.jobs:
+                if job.store_slot is not None:
+                    self.cache.out_block_cache[job.store_slot] = job.chunks
+                    self.cache.lse_block_cache[job.store_slot] = job.chunks
+        else:
+            out = self._execute(plan, query, key, value, merge_outs, merge_lses)
+
+        # 4./5. pointer and cache management (:214, :219-220)
+        self.target_chunk_id = new_target
+        self._ring_targets = new_targets
+        if self.dry_run:
+            self._dry_update_cache(nxt, new_target // nxt)
+        else:
+            self.cache.update_cache_blocks(nxt, new_target // nxt)
+        plan.nblk_after = self.cache.curr_block_num
+        plan.occupancy_after = [o is not None for o in self.cache.out_block_cache]
+        self.last_plan = plan
+        if out is not None:
+            rm.record_out_redundancy(timestep=timestep, layer_id=self.layer_id, curr_out=out)  # :233-236
+        return out
+
+    def _dry_update_cache(self, nxt: int, next_target_block: int) -> None:
+        """``update_cache_blocks`` on occupancy tokens (tuples of chunk ids) instead of tensors."""
+        cache = self.cache
+        if nxt != self.isp_size and nxt != 0:
+            new_n = self.isp_size // nxt
+            assert new_n <= cache.curr_block_num, "Invalid ISP stride."
+            if new_n != cache.curr_block_num:
+                group = cache.curr_block_num // new_n
+                merged = []
+                for i in range(new_n):
+                    parts = [cache.out_block_cache[i * group + j] for j in range(group)
+                             if cache.out_block_cache[i * group + j] is not None]
+                    merged.append(tuple(c for p in parts for c in p) if parts else None)
+                cache.out_block_cache = merged
+                cache.lse_block_cache = list(merged)
+                cache.curr_block_num = new_n
+            cache.curr_isp_stride = nxt
+            cache.out_block_cache[next_target_block] = None
+            cache.lse_block_cache[next_target_block] = None
+        else:
+            cache.update_cache_blocks(nxt, next_target_block)
+
+    def _execute(self, plan: CallPlan, query, key, value, merge_outs, merge_lses) -> torch.Tensor:
+        B, Sq, H, D = query.shape
+        N, r = self.isp_size, self.local_chunk_id
+        dev = query.device
+        # chunk table: the local chunk is (key, value); the others come from the ring stand-in
+        needed = sorted({c for job in plan.jobs for c in job.chunks})
+        ks: List[torch.Tensor] = []
+        vs: List[torch.Tensor] = []
+        index = {}
+        for c in needed:
+            index[c] = len(ks)
+            k_c, v_c = (key, value) if c == r else self.group.kv_chunk(c)
+            ks.append(_as4d(k_c, B))
+            vs.append(_as4d(v_c, B))
+        # one launch for all distinct states; a chunk computed twice by the reference
+        # (local + own) is computed once and merged twice
+        job_lists, dests, seen = [], [], {}
+        states = []
+        for job in plan.jobs:
+            if job.chunks in seen and job.store_slot is None:
+                states.append(seen[job.chunks])
+                continue
+            o = torch.empty((B, Sq, H, D), dtype=torch.bfloat16, device=dev)
+            l = torch.empty((B, H, Sq), dtype=torch.float32, device=dev)
+            job_lists.append([index[c] for c in job.chunks])
+            dests.append((o, l))
+            seen[job.chunks] = (o, l)
+            states.append((o, l))
+        if job_lists:
+            table = _hip.ChunkTable(ks, vs)
+            _hip.attn_jobs_fwd(query, table, job_lists, [d[0] for d in dests], [d[1] for d in dests])
+        for job, (o, l) in zip(plan.jobs, states):
+            if job.store_slot is not None:
+                self.cache.store_block(job.store_slot, o, l)  # :207-211
+            merge_outs.append(o)
+            merge_lses.append(l)
+        out, lse = _hip.merge_states(merge_outs, merge_lses, dst_dtype=torch.float32, dst_lse_bsh=True)
+        self.last_lse = lse
+        return out
+
+    # ---- mask mode ----------------------------------------------------------------------------------
+    def _attn_masked(self, query, key, value) -> torch.Tensor:
+        rm = get_redundancy_map()
+        t, l = get_timestep(), self.layer_id
+        C = rm.chunk_mask.shape[2]
+        diag = rm.mask_diag
+        B, Sq, H, D = query.shape
+        cache = self.cache
+        cache.ensure_arena(C, B, Sq, H, D, query.device)
+        row = rm.chunk_mask[t, l]
+        ks, vs = [], []
+        for c in range(C):
+            use_local = (c == self.local_chunk_id and c == diag and key is not None)
+            k_c, v_c = (key, value) if use_local else self.group.kv_chunk(c)
+            ks.append(_as4d(k_c, B))
+            vs.append(_as4d(v_c, B))
+        for c in range(C):
+            if c != diag and row[c] != 0 and not cache.arena_valid[c]:
+                raise RuntimeError(f"T{t}L{l}: mask asks to reuse chunk {c} but no state was ever stored for it")
+        n_comp = int(rm.sched_counts_host[t, l, 0])
+        table = _hip.ChunkTable(ks, vs)
+        _hip.attn_sched_fwd(query, table, rm.sched_compute_ids[t, l], rm.sched_counts[t, l, 0:1], n_comp,
+                            cache.arena_out, cache.arena_lse, diag, cache.diag_out, cache.diag_lse)
+        outs, lses = [], []
+        for c in range(C):
+            if c == diag:
+                outs.append(cache.diag_out)
+                lses.append(cache.diag_lse)
+            else:
+                if row[c] == 0:
+                    cache.arena_valid[c] = True
+                outs.append(cache.arena_out[c])
+                lses.append(cache.arena_lse[c])
+        out, lse = _hip.merge_states(outs, lses, dst_dtype=torch.float32, dst_lse_bsh=True)
+        self.last_lse = lse
+        rm.record_out_redundancy(timestep=t, layer_id=l, curr_out=out)
+        return out
+
+    # ---- varlen entry (HunyuanVideo) ---------------------------------------------------------------
+    @get_timer("varlen oAttn")
+    def varlen_attn(self, query, key, value, cu_seqlens_q=None, cu_seqlens_kv=None, max_seqlen_q=None,
+                    max_seqlen_kv=None, batch_size=1):
+        """core/attention.py:239-419.  Without sequence lengths it is ``attn`` (:252-254).
+        With them, inputs are ``[B*S, H, D]``; the single-segment-per-sample case (every
+        sample one full-length segment) is the dense path on a reshaped view.  Several
+        segments per sample are not built yet and raise."""
+        if cu_seqlens_q is None and cu_seqlens_kv is None and max_seqlen_q is None and max_seqlen_kv is None:
+            logger.warning("cu_seqlens_q not provided, using normal attention instead.")
+            return self.attn(query, key, value)
+        total_q, H, D = query.shape
+        total_k = key.shape[0]
+        cq = [int(x) for x in cu_seqlens_q.tolist()]
+        ck = [int(x) for x in cu_seqlens_kv.tolist()]
+        nb = len(cq) - 1
+        uniform = (len(ck) == len(cq) and total_q % nb == 0 and total_k % nb == 0
+                   and cq == [i * (total_q // nb) for i in range(nb + 1)]
+                   and ck == [i * (total_k // nb) for i in range(nb + 1)])
+        if not uniform:
+            raise NotImplementedError("varlen_attn with several (or ragged) segments per sample is not built yet; "
+                                      "only one full-length segment per sample is")
+        out = self.attn(query.view(nb, total_q // nb, H, D), key.view(nb, total_k // nb, H, D),
+                        value.view(nb, total_k // nb, H, D))
+        return out.view(total_q, H, D)

@@ -1,0 +1,54 @@
+"""The built library loads and exports every function include/ditango_hip.h declares
+(no compute calls: this runs without a GPU)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "ditango_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(dt_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    names = _declared()
+    for must in ("dt_attn_chunk_fwd", "dt_attn_jobs_fwd", "dt_attn_sched_fwd", "dt_merge_states", "dt_cache_store",
+                 "dt_cache_load", "dt_build_schedule", "dt_build_schedule_table", "dt_rel_l1_sums", "dt_version",
+                 "dt_last_error"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol():
+    from ditango_amd import _hip
+    if not _hip.LIB_PATH.exists():
+        from ditango_amd.build import build_lib
+        build_lib()
+    lib = _hip.load_library()
+    for name in _declared():
+        assert hasattr(lib, name), f"{name} declared in the header but not exported"
+    assert set(_declared()) == set(_hip.EXPORTED_SYMBOLS)
+    assert lib.dt_version() >= 100
+    assert isinstance(lib.dt_last_error(), bytes)
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    from ditango_amd import _hip
+    with pytest.raises(_hip.DitangoHipError):
+        _hip.load_library(tmp_path / "nope.so")
+
+
+def test_argument_errors_are_reported_without_a_gpu():
+    """Validation happens on the host before any launch."""
+    from ditango_amd import _hip
+    lib = _hip.load_library()
+    rc = lib.dt_merge_states(0, None, None, None, None, None, 0, None, 0, 1, 1, 1, 128, None)
+    assert rc == -1 and b"need 1.." in lib.dt_last_error()
+    rc = lib.dt_attn_chunk_fwd(None, None, None, None, None, 1, 1, 1, 1, 96, 0, 0, 0, 0, 0, 0, 0.0, None)
+    assert rc == -2 and b"head dim" in lib.dt_last_error()
+    rc = lib.dt_build_schedule(None, 1, 1, 1, 0, 0, -1, None, None, None, None)
+    assert rc == -1

@@ -1,0 +1,116 @@
+"""The product's host-side schedule (closed-form ring delivery, pointer, cache
+bookkeeping) must equal the lock-step ring simulation of the oracle bit for bit."""
+import random
+import types
+
+import numpy as np
+import pytest
+import torch
+
+from oracle.state_machine import RingOracle, legal_divider_column, strides_from_dividers
+
+
+@pytest.fixture
+def ditango_env():
+    from ditango_amd.core import config, parallel_state, redundancy_map
+    from ditango_amd import utils
+
+    def make(N, rank, T, L, use_ditango=True):
+        parallel_state.init_local_groups(N, rank)
+        config.init_config(None, num_inference_steps=T, num_layers=L, use_ditango=use_ditango)
+        redundancy_map.destroy_redundancy_map()
+        redundancy_map._redundancy_map = redundancy_map.RedundancyMap(config.get_config())
+        return redundancy_map.get_redundancy_map()
+
+    yield make
+    from ditango_amd.core import parallel_state as ps, redundancy_map as rmod
+    rmod.destroy_redundancy_map()
+    ps.destroy_local_groups()
+    utils.update_timestep(0)
+
+
+def _random_column(T, N, rng):
+    mid, prev = [], 1
+    for _ in range(T - 5):
+        prev = rng.choice([d for d in (1, 2, 4, 8) if d <= N and (prev == 1 or d <= prev)])
+        mid.append(prev)
+    col = (1, 1, 1) + tuple(mid) + (1, 1)
+    assert legal_divider_column(col)
+    return col
+
+
+@pytest.mark.parametrize("N,use_ditango", [(2, True), (4, True), (8, True), (16, True), (16, False)])
+def test_plan_matches_ring_oracle(ditango_env, N, use_ditango):
+    from ditango_amd.core.attention import proAttention
+    from ditango_amd.core.parallel_state import get_usp_group
+    from ditango_amd.utils import update_timestep
+
+    T = 14
+    rng = random.Random(N)
+    for trial in range(6):
+        col = _random_column(T, N, rng)
+        curr, nxt = strides_from_dividers(N, col)
+        ring = RingOracle(N, use_ditango=use_ditango)
+        oracle_traces = [ring.call(t, curr[t], nxt[t]) for t in range(T)]
+        for rank in range(N):
+            rm = ditango_env(N, rank, T, 1, use_ditango)
+            rm.divider_map[:, 0] = torch.tensor(col)
+            attn = proAttention(0, get_usp_group(), dry_run=True)
+            for t in range(T):
+                update_timestep(t)
+                attn.attn(None, None, None)
+                p, o = attn.last_plan, oracle_traces[t][rank]
+                ctx = (col, rank, t)
+                assert (p.curr_stride, p.next_stride) == (o.curr_stride, o.next_stride), ctx
+                assert p.reuse_probed == o.reuse_probed, ctx
+                assert p.reuse_merged == o.reuse_merged, ctx
+                assert p.computed == o.computed, ctx
+                assert p.stores == o.stores, ctx
+                assert p.flushes == o.flushes, ctx
+                assert p.target_after == o.target_after, ctx
+                assert p.nblk_after == o.nblk_after, ctx
+                assert p.occupancy_after == o.occupancy_after, ctx
+
+
+def test_strides_follow_divider_map(ditango_env):
+    from oracle import divider_map as od
+    rm = ditango_env(8, 0, 6, 3)
+    rm.divider_map = torch.tensor([[1, 1, 1], [8, 4, 2], [8, 2, 1], [4, 2, 1], [1, 1, 1], [2, 2, 2]])
+    div = rm.divider_map.numpy()
+    for t in range(6):
+        for l in range(3):
+            assert rm.get_curr_isp_stride(t, l) == od.curr_stride(div, 8, t, l)
+            assert rm.get_next_isp_stride(t, l) == od.next_stride(div, 8, t, l)
+    assert rm.get_next_isp_stride(5, 0) == 8  # last step announces a full refresh
+    rm.auto_setting = True
+    assert rm.get_curr_isp_stride(1, 0) == 8 and rm.get_next_isp_stride(1, 0) == 8
+    rm.auto_setting = False
+    # base weight smaller than the divider -> stride 1 (redundancy_map.py:63-64)
+    rm.base_weight = 4
+    assert rm.get_curr_isp_stride(1, 0) == 1
+
+
+def test_set_pattern_rows(ditango_env):
+    rm = ditango_env(8, 0, 5, 6)
+    rm.set_pattern_for_rows(range(1, 3), [2, 4], [8, 4, 2])
+    assert rm.divider_map[1].tolist() == [8, 8, 4, 4, 2, 2] and rm.divider_map[0].tolist() == [1] * 6
+    rm.set_full_stride_for_rows([3])
+    assert rm.divider_map[3].tolist() == [8] * 6
+    with pytest.raises(ValueError):
+        rm.set_pattern_for_row(9, [], [1])
+    rm.reset_map()
+    assert int(rm.divider_map.sum()) == 30
+
+
+def test_memory_guard_falls_back_to_full_refresh(ditango_env):
+    """An over-budget prediction turns the announced stride into N (core/attention.py:97-98)."""
+    from ditango_amd.core.cache import proCache
+    c = proCache(8, 0)
+    c.block_size_mb = 100.0
+    c.memory_constraint = 1000.0
+    c.memory_probe = lambda: 500.0
+    assert c.pass_memory_check(8, 0) is True          # full refresh is always fine
+    assert c.pass_memory_check(2, 0) is True           # 4 blocks * 100 MB + 500 <= 1000
+    assert c.pass_memory_check(1, 0) is False          # 8 blocks * 100 MB + 500 > 1000
+    c.out_block_cache = [object()] * 8                 # already holding as many blocks as predicted
+    assert c.pass_memory_check(1, 0) is True
