@@ -1,0 +1,244 @@
+#!/usr/bin/env python3
+"""Benchmark of the cached block attention hot path on ONE MI355X.
+
+A "step" is one ``proAttention.attn`` call (one transformer layer's attention at one
+diffusion step) at the HunyuanVideo per-rank shape: local query shard of 14882 tokens,
+KV = 8 chunks of 14882 tokens, H=24, D=128, bf16, under the seeded Bernoulli(0.6) reuse mask
+over 50 steps x 60 layers.  Inputs are resident in HBM before the timed region.
+
+Prints ONE JSON line: ms per layer call plus
+  * ``roofline``        the fresh-chunk attention kernel against the bf16 dense MFMA peak,
+  * ``roofline_merge``  the fused LSE-merge kernel against the HBM peak,
+  * ``cache_gbs``       cache store / load copies against the HBM peak,
+  * ``cpu_baseline``    the torch-math oracle timed on this box's host cores on a bounded sample.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+WORKLOADS = {
+    # name: (label, B, H, D, Sq, chunk lengths, T, L, reuse probability, diag, qk norm)
+    "hunyuanvideo": ("HunyuanVideo per-rank share (configs[2])", 1, 24, 128, 14882, [14882] * 8, 50, 60, 0.6, 0, "rms"),
+    "cogvideox": ("CogVideoX-5B per-rank share (configs[1])", 1, 48, 64, 2222, [2222] * 8, 50, 42, 0.5, 0, "layer"),
+    "stepvideo": ("Step-Video-T2V per-rank share (configs[3])", 1, 48, 128, 6851, [6851] * 8, 50, 48, 0.75, 0, None),
+    "sweep": ("reuse sweep at HunyuanVideo scale (configs[4])", 1, 24, 128, 119056, [3721] * 16 + [3720] * 16, 1, 60, 0.5, -1, "rms"),
+}
+
+
+def make_inputs(B, H, D, Sq, lens, norm, device, seed=0):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+
+    def draw(n, normalise):
+        x = torch.randn(B, n, H, D, generator=g)
+        if normalise == "rms":
+            x = x / x.pow(2).mean(-1, keepdim=True).sqrt()
+        elif normalise == "layer":
+            x = torch.nn.functional.layer_norm(x, (D,))
+        return x.bfloat16()
+
+    q = draw(Sq, norm).to(device)
+    ks = [draw(n, norm).to(device) for n in lens]
+    vs = [draw(n, None).to(device) for n in lens]
+    return q, ks, vs
+
+
+def time_kernel(fn, reps, warm=3):
+    """Average duration in ms of ``fn`` over ``reps`` launches (HIP events on the launch stream)."""
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / reps
+
+
+def cpu_baseline(B, H, D, Sq, lens, mean_computed, n_chunks, norm, budget_s=20.0):
+    """The oracle's torch math on the host cores, on a bounded sample scaled to one layer call."""
+    from oracle import attention_math as om
+    cores = len(os.sched_getaffinity(0))
+    torch.set_num_threads(cores)
+    Sk = lens[0]
+    g = torch.Generator().manual_seed(1)
+    heads = 1
+    q = torch.randn(B, Sq, heads, D, generator=g).bfloat16()
+    k = torch.randn(B, Sk, heads, D, generator=g).bfloat16()
+    v = torch.randn(B, Sk, heads, D, generator=g).bfloat16()
+    t0 = time.perf_counter()
+    n_done = 0
+    while True:
+        om.chunk_attention(q, k, v)
+        n_done += 1
+        el = time.perf_counter() - t0
+        if el > budget_s * 0.7 or n_done >= 8:
+            break
+    per_head_chunk = el / n_done
+    # merge of n_chunks states on 1/8 of the rows, literal reference fold
+    rows_s = max(1, Sq // 8)
+    outs = [torch.randn(B, rows_s, H, D, generator=g).bfloat16() for _ in range(n_chunks)]
+    lses = [torch.randn(B, H, rows_s, generator=g) for _ in range(n_chunks)]
+    t1 = time.perf_counter()
+    o = l = None
+    for bo, bl in zip(outs, lses):
+        o, l = om.update_out_and_lse(o, l, bo, bl)
+    merge_s = (time.perf_counter() - t1) * (Sq / rows_s)
+    layer_ms = 1e3 * (per_head_chunk * H * mean_computed + merge_s)
+    flops = 4.0 * B * H * Sq * Sk * D * mean_computed
+    return {
+        "value": round(layer_ms, 1), "unit": "ms", "cores": cores, "kind": "port",
+        "attn_tflops": round(flops / (per_head_chunk * H * mean_computed) / 1e12, 3),
+        "sample": (f"{n_done}x one head of one KV chunk (Sq={Sq}, Sk={Sk}, D={D}) in {el:.1f}s, scaled x{H} heads x "
+                   f"{mean_computed:.2f} computed chunks/call; literal update_out_and_lse fold of {n_chunks} states on "
+                   f"1/8 of the rows scaled x8"),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=120)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="hunyuanvideo", choices=list(WORKLOADS))
+    ap.add_argument("--layers", type=int, default=None, help="layers to instantiate (default: all of the model)")
+    ap.add_argument("--reuse", type=float, default=None, help="override the mask's reuse probability")
+    ap.add_argument("--kernel-reps", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one sequence-parallel rank's share on ONE GPU; --gpus > 1 is not part of this build",
+              file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+
+    from ditango_amd import _hip
+    from ditango_amd.core import config, parallel_state, redundancy_map as rmod
+    from ditango_amd.core.attention import proAttention
+    from ditango_amd.utils import update_timestep
+    _hip.load_library()
+
+    label, B, H, D, Sq, lens, T, L, p, diag, norm = WORKLOADS[args.workload]
+    if args.reuse is not None:
+        p = args.reuse
+    C = len(lens)
+    L_run = min(L, args.layers) if args.layers else L
+    if args.workload == "sweep":
+        L_run = min(L_run, 2)   # 32 cached states of 743 MB per layer
+        T = 2                   # step 0 fills the cache, step 1 is measured
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    rank = max(diag, 0)
+    parallel_state.init_local_groups(C, rank)
+    cfg = config.init_config(None, num_inference_steps=T, num_layers=L)
+    rmod.destroy_redundancy_map()
+    rmod._redundancy_map = rmod.RedundancyMap(cfg)
+    rm = rmod.get_redundancy_map()
+    mask = rmod.make_bernoulli_mask(T, L, C, p, seed=0, diag=diag)
+    rm.set_chunk_mask(mask, diag=diag)
+
+    q, ks, vs = make_inputs(B, H, D, Sq, lens, norm, dev)
+    group = parallel_state.get_usp_group()
+    group.set_kv_chunks(ks, vs)
+    layers = [proAttention(l, group) for l in range(L_run)]
+
+    # fill the caches: step 0 recomputes everything (not timed, not a warm-up step)
+    update_timestep(0)
+    for l in range(L_run):
+        layers[l].attn(q, ks[rank], vs[rank])
+    torch.cuda.synchronize()
+
+    calls = [(t, l) for t in range(1, T) for l in range(L_run)]
+    need = args.warmup + args.steps
+    seq = [calls[i % len(calls)] for i in range(need)]
+
+    def run(t, l):
+        update_timestep(t)
+        return layers[l].attn(q, ks[rank], vs[rank])
+
+    for t, l in seq[:args.warmup]:
+        run(t, l)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for t, l in seq[args.warmup:]:
+        run(t, l)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = 1e3 * elapsed / args.steps
+    timed = seq[args.warmup:]
+    n_comp = [int(rm.sched_counts_host[t, l, 0]) for t, l in timed]
+    mean_computed = float(np.mean(n_comp))
+    Sk_mean = float(np.mean(lens))
+    flops_per_chunk = 4.0 * B * H * Sq * Sk_mean * D
+    rows = B * Sq * H
+
+    # ---- per-kernel rooflines, measured live with HIP events on the launch stream ----------
+    reps = args.kernel_reps
+    out_s = torch.empty(B, Sq, H, D, dtype=torch.bfloat16, device=dev)
+    lse_s = torch.empty(B, H, Sq, dtype=torch.float32, device=dev)
+    k1_ms = time_kernel(lambda: _hip.attn_chunk_fwd(q, ks[0], vs[0], out=out_s, lse=lse_s), reps)
+    k1_flops = 4.0 * B * H * Sq * lens[0] * D
+    k1_tflops = k1_flops / (k1_ms * 1e-3) / 1e12
+
+    cache0 = layers[0].cache
+    m_outs = [cache0.arena_out[c] if c != diag else cache0.diag_out for c in range(C)]
+    m_lses = [cache0.arena_lse[c] if c != diag else cache0.diag_lse for c in range(C)]
+    dst_o = torch.empty(B, Sq, H, D, dtype=torch.float32, device=dev)
+    dst_l = torch.empty(B, Sq, H, 1, dtype=torch.float32, device=dev)
+    k2_ms = time_kernel(lambda: _hip.merge_states(m_outs, m_lses, dst_out=dst_o, dst_lse=dst_l), reps)
+    k2_bytes = rows * (C * (2 * D + 4) + (4 * D + 4))
+    k2_gbs = k2_bytes / (k2_ms * 1e-3) / 1e9
+
+    k3s_ms = time_kernel(lambda: _hip.cache_store(dst_o, dst_l, out_s, lse_s), reps)
+    k3s_gbs = rows * ((4 * D + 4) + (2 * D + 4)) / (k3s_ms * 1e-3) / 1e9
+    slot2_o, slot2_l = torch.empty_like(out_s), torch.empty_like(lse_s)
+    k3c_ms = time_kernel(lambda: _hip.cache_store(out_s, lse_s, slot2_o, slot2_l), reps)
+    k3c_gbs = rows * 2 * (2 * D + 4) / (k3c_ms * 1e-3) / 1e9
+    k3l_ms = time_kernel(lambda: _hip.cache_load(out_s, lse_s, torch.float32, True), reps)
+    k3l_gbs = rows * ((2 * D + 4) + (4 * D + 4)) / (k3l_ms * 1e-3) / 1e9
+
+    dmask = torch.from_numpy(mask).to(dev)
+    k4_ms = time_kernel(lambda: _hip.build_schedule_table(dmask, diag), reps)
+
+    result = {
+        "metric": "ms/layer", "value": round(ms_per_step, 4), "unit": "ms", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": label, "B": B, "H": H, "D": D, "Sq": Sq, "kv_chunks": C, "Sk": lens[0],
+                   "mask": f"Bernoulli({p}) seed 0 over {T}x{L}x{C}, diag {diag}", "layers_instantiated": L_run,
+                   "mean_chunks_computed_per_call": round(mean_computed, 3)},
+        "layer_attn_tflops": round(flops_per_chunk * mean_computed / (ms_per_step * 1e-3) / 1e12, 1),
+        "roofline": {"kernel": "attn_fwd_kernel<%d>" % D, "bound": "mfma", "achieved": round(k1_tflops, 1),
+                     "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(k1_tflops / PEAK_BF16_TFLOPS, 4),
+                     "traffic": None, "launch_ms": round(k1_ms, 4), "flop_per_launch": k1_flops},
+        "roofline_merge": {"kernel": "merge_states_kernel<%d>" % D, "bound": "hbm", "achieved": round(k2_gbs, 1),
+                           "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(k2_gbs / PEAK_HBM_GBS, 4),
+                           "traffic": None, "launch_us": round(k2_ms * 1e3, 2), "bytes_per_launch": k2_bytes,
+                           "states": C},
+        "cache_gbs": {"store_fp32_to_slot": round(k3s_gbs, 1), "store_bf16_to_slot": round(k3c_gbs, 1),
+                      "load_slot_to_fp32": round(k3l_gbs, 1), "peak": PEAK_HBM_GBS,
+                      "frac_store_bf16": round(k3c_gbs / PEAK_HBM_GBS, 4), "frac_load": round(k3l_gbs / PEAK_HBM_GBS, 4)},
+        "schedule_builder_us": round(k4_ms * 1e3, 2),
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(B, H, D, Sq, lens, mean_computed, C, norm)
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -282,6 +282,20 @@ class RedundancyMap:
         self.sched_counts_host = None
 
 
+def make_bernoulli_mask(num_timesteps: int, num_layers: int, num_chunks: int, reuse_prob: float, seed: int,
+                        diag: int = -1, cold_first_step: bool = True) -> np.ndarray:
+    """Seeded per-chunk reuse mask ``[T, L, C]`` uint8: entry = 1 with probability
+    ``reuse_prob`` (``numpy.random.default_rng(seed).random() < reuse_prob``); the local
+    chunk ``diag`` is never reused and step 0 reuses nothing (the cache is cold)."""
+    rng = np.random.default_rng(seed)
+    m = (rng.random((num_timesteps, num_layers, num_chunks)) < reuse_prob).astype(np.uint8)
+    if 0 <= diag < num_chunks:
+        m[:, :, diag] = 0
+    if cold_first_step:
+        m[0] = 0
+    return m
+
+
 def print_redundancy_map(logger_=None):
     """:628-658"""
     rm = get_redundancy_map()
