@@ -10,8 +10,8 @@
 //     each) so one wave's softmax VALU work overlaps another's MFMA work.
 //   * KV is consumed in tiles of 64 keys.  K is staged in LDS as [key][d],
 //     V is transposed on the way in and staged as [d][key]; both are
-//     double-buffered and XOR-swizzled in 16-byte units so that the MFMA
-//     operand reads (ds_read_b128) are bank-conflict free.
+//     double-buffered and padded by 16 bytes per row so that the MFMA operand
+//     reads (ds_read_b128 with immediate offsets) are bank-conflict free.
 //   * Scores are computed TRANSPOSED, S^T = K Q^T, with v_mfma_f32_32x32x16_bf16:
 //     in the accumulator layout a lane then owns ONE query (column lane%32) and
 //     16 of the 32 keys of the tile, so the online-softmax max/sum are
@@ -21,8 +21,9 @@
 //     are 8 CONSECUTIVE keys.  Rounded to bf16 they are directly the B operand
 //     of the second MFMA, O^T += V^T P^T, whose A operand is one 16-byte read of
 //     8 consecutive keys of one d-row of the transposed V tile.
-//   * O^T stays in registers as [d][query]: the per-tile rescale is a multiply by
-//     a per-lane scalar.  The epilogue transposes through LDS so that the global
+//   * O^T stays in registers as [d][query]: a rescale is a multiply by a per-lane
+//     scalar, and it is only done when some query's running maximum grew by more
+//     than 2^8 (the reference maximum may lag; the lse stays exact).  The epilogue transposes through LDS so that the global
 //     stores are 16 bytes per lane, 16 lanes per 256-byte row.
 //   * Workgroups are mapped to (head, query tile) so that the 8 XCDs each work
 //     through a contiguous range of heads: the workgroups that share an XCD's
@@ -56,32 +57,47 @@ __device__ __forceinline__ int key_of_row(int i) {
 
 template <int D>
 struct Tile {
-  static constexpr int kRowBytesK = D * 2;            // one key, all d
+  // LDS tiles are padded by 16 bytes per row instead of swizzled: every operand read is then
+  // "lane base + compile-time constant", i.e. a ds_read_b128 with an immediate offset and no
+  // address arithmetic in the loop, and 16 consecutive rows still fall into 16 distinct
+  // 16-byte bank groups (pitch mod 256 is 16 or 144).
+  static constexpr int kPitchK = D * 2 + 16;          // one key, all d
+  static constexpr int kPitchV = kBK * 2 + 16;        // one d, 64 keys
   static constexpr int kChunksK = D / 8;              // 16-byte chunks per K row
-  static constexpr int kBytesK = kBK * kRowBytesK;
-  static constexpr int kBytesV = D * kBK * 2;         // [d][64 keys]
+  static constexpr int kBytesK = kBK * kPitchK;
+  static constexpr int kBytesV = D * kPitchV;
   static constexpr int kBytesBuf = kBytesK + kBytesV;
   static constexpr int kLoadsK = kBK * kChunksK / kThreads;  // 16-byte loads per thread
+  static constexpr int kRowStepK = kThreads / kChunksK;
   static constexpr int kDV = D / 16;                  // d values per thread in the V transpose
   static constexpr int kVW = kDV / 2;                 // dwords per V load
   static constexpr int kPitchO = D * 2 + 16;          // epilogue row pitch
-
-  // byte offset of 16-byte chunk c of K row `key`
-  __device__ static __forceinline__ int k_off(int key, int c) {
-    if (kChunksK == 16) return key * kRowBytesK + ((c ^ (key & 15)) << 4);
-    return key * kRowBytesK + ((c ^ ((key >> 1) & 7)) << 4);
-  }
-  // byte offset of 16-byte chunk c (8 keys) of V^T row d
-  __device__ static __forceinline__ int v_off(int d, int c) {
-    return d * (kBK * 2) + ((c ^ (((d >> 1) ^ (d >> 4)) & 7)) << 4);
-  }
+  static constexpr int kLdsBytes = 2 * kBytesBuf;
 };
+
+// Raw buffer descriptor word 3 for gfx9-family targets (32-bit data format, no swizzle).
+constexpr int kRsrcFlags = 0x00020000;
+
+template <int W>
+__device__ __forceinline__ typename VecOf<W>::type buffer_load_v(__amdgpu_buffer_rsrc_t r, int voff);
+template <>
+__device__ __forceinline__ u32x4 buffer_load_v<4>(__amdgpu_buffer_rsrc_t r, int voff) {
+  return __builtin_amdgcn_raw_buffer_load_b128(r, voff, 0, 0);
+}
+template <>
+__device__ __forceinline__ u32x2 buffer_load_v<2>(__amdgpu_buffer_rsrc_t r, int voff) {
+  return __builtin_amdgcn_raw_buffer_load_b64(r, voff, 0, 0);
+}
+
+// Largest growth of the running maximum (in log2 units of the scaled scores) that is
+// tolerated without rescaling the accumulators: probabilities then stay below 2^kTau.
+constexpr float kTau = 8.0f;
 
 template <int D>
 __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a) {
   using T = Tile<D>;
   using VLoad = typename VecOf<T::kVW>::type;
-  __shared__ __attribute__((aligned(16))) uint8_t lds[2 * T::kBytesBuf];
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
   // ---- which (job, batch, head, query tile) ------------------------------------------
   const int job = blockIdx.y;
@@ -139,50 +155,78 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   int n_tiles = 0;
   for (int s = seg_begin; s < seg_end; ++s) n_tiles += (a.kv_len[chunk_of(s)] + kBK - 1) / kBK;
 
-  // load cursor (one tile ahead of the compute cursor)
-  int ld_seg = seg_begin, ld_k0 = 0;
-  int cp_seg = seg_begin, cp_k0 = 0;
-  while (ld_seg < seg_end && a.kv_len[chunk_of(ld_seg)] == 0) ++ld_seg;
-  cp_seg = ld_seg;
+  // Two cursors walk the job's chunks tile by tile, all in scalar registers: the load cursor
+  // (one tile ahead: base pointers of the tile and keys left in its chunk) and the compute
+  // cursor (keys left in the chunk of the tile being consumed).
+  int ld_seg = seg_begin - 1, ld_left = 0;
+  const uint8_t* ld_k = nullptr;
+  const uint8_t* ld_v = nullptr;
+  int cp_seg = seg_begin - 1, cp_left = 0;
+  auto ld_next_chunk = [&]() {
+    do { ++ld_seg; } while (ld_seg < seg_end && a.kv_len[chunk_of(ld_seg)] == 0);
+    if (ld_seg < seg_end) {
+      const int cid = chunk_of(ld_seg);
+      const int64_t head_off = (int64_t)b * a.kv_sb[cid] + (int64_t)h * a.kv_sh;
+      ld_k = reinterpret_cast<const uint8_t*>(a.k[cid] + head_off);
+      ld_v = reinterpret_cast<const uint8_t*>(a.v[cid] + head_off);
+      ld_left = a.kv_len[cid];
+    }
+  };
+  auto cp_next_chunk = [&]() {
+    do { ++cp_seg; } while (cp_seg < seg_end && a.kv_len[chunk_of(cp_seg)] == 0);
+    if (cp_seg < seg_end) cp_left = a.kv_len[chunk_of(cp_seg)];
+  };
+  ld_next_chunk();
+  cp_next_chunk();
 
-  // thread -> K tile elements
-  const int kc = tid % T::kChunksK;            // 16-byte chunk within the row
-  const int kr0 = tid / T::kChunksK;           // first key row
-  constexpr int kRowStep = kThreads / T::kChunksK;
-  // thread -> V tile elements: 4 keys x kDV d
-  const int vdg = tid & 15;
-  const int vkg = tid >> 4;
+  // thread -> K tile elements: 16-byte chunk kc of rows kr0 + i*kRowStepK
+  const int kc = tid % T::kChunksK;
+  const int kr0 = tid / T::kChunksK;
+  // thread -> V tile elements: keys 4*vkg..+3, d kDV*vdg..+kDV-1.  A half wavefront covers
+  // 16 key groups of one d group, so its transposed 8-byte LDS writes fill whole rows.
+  const int vkg = tid & 15;
+  const int vdg = tid >> 4;
+  const uint32_t row_bytes = (uint32_t)a.kv_ss * 2u;
+  // byte offsets from the tile's first key, loop invariant for full tiles
+  uint32_t koff[T::kLoadsK], voff[4];
+#pragma unroll
+  for (int i = 0; i < T::kLoadsK; ++i) koff[i] = (uint32_t)(kr0 + i * T::kRowStepK) * row_bytes + 16u * kc;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) voff[r] = (uint32_t)(4 * vkg + r) * row_bytes + (uint32_t)(T::kDV * 2 * vdg);
 
   u32x4 kreg[T::kLoadsK];
   VLoad vreg[4];
 
-  auto load_tile = [&](int seg, int k0) {
-    const int cid = chunk_of(seg);
-    const int len = a.kv_len[cid];
-    const __bf16* kb = a.k[cid] + (int64_t)b * a.kv_sb[cid] + (int64_t)h * a.kv_sh;
-    const __bf16* vb = a.v[cid] + (int64_t)b * a.kv_sb[cid] + (int64_t)h * a.kv_sh;
+  const int64_t tile_bytes = (int64_t)kBK * row_bytes;
+  // Loads the tile under the load cursor into registers and moves the cursor on.  The loads
+  // are raw buffer loads: the descriptor (base of the tile's first key for this batch and
+  // head, number of valid bytes) lives in scalar registers, the lane offsets are loop
+  // invariant, and rows past the end of the chunk are out of range for the hardware bounds
+  // check and come back as zeros (their scores are masked to -inf; zero V rows add nothing).
+  auto load_tile = [&]() {
+    const uint32_t valid = (uint32_t)(ld_left - 1) * row_bytes + (uint32_t)(D * 2);
+    const __amdgpu_buffer_rsrc_t rk =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(ld_k), 0, (int)valid, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t rv =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(ld_v), 0, (int)valid, kRsrcFlags);
 #pragma unroll
-    for (int i = 0; i < T::kLoadsK; ++i) {
-      int key = k0 + kr0 + i * kRowStep;
-      if (key > len - 1) key = len - 1;  // clamped rows are masked out of the softmax
-      kreg[i] = *reinterpret_cast<const u32x4*>(kb + (int64_t)key * a.kv_ss + 8 * kc);
-    }
+    for (int i = 0; i < T::kLoadsK; ++i) kreg[i] = __builtin_amdgcn_raw_buffer_load_b128(rk, (int)koff[i], 0, 0);
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      int key = k0 + 4 * vkg + r;
-      if (key > len - 1) key = len - 1;  // weight of a clamped row is exactly 0
-      vreg[r] = *reinterpret_cast<const VLoad*>(vb + (int64_t)key * a.kv_ss + T::kDV * vdg);
-    }
+    for (int r = 0; r < 4; ++r) vreg[r] = buffer_load_v<T::kVW>(rv, (int)voff[r]);
+    ld_left -= kBK;
+    ld_k += tile_bytes;
+    ld_v += tile_bytes;
+    if (ld_left <= 0) ld_next_chunk();
   };
 
+  // LDS write addresses of this thread (per buffer: + buf * kBytesBuf)
+  const int kst = kr0 * T::kPitchK + 16 * kc;
+  const int vst = T::kBytesK + (T::kDV * vdg) * T::kPitchV + 8 * vkg;
   auto store_tile = [&](int buf) {
-    uint8_t* kl = lds + buf * T::kBytesBuf;
-    uint8_t* vl = kl + T::kBytesK;
+    uint8_t* base = lds + buf * T::kBytesBuf;
 #pragma unroll
-    for (int i = 0; i < T::kLoadsK; ++i) {
-      const int key = kr0 + i * kRowStep;
-      *reinterpret_cast<u32x4*>(kl + T::k_off(key, kc)) = kreg[i];
-    }
+    for (int i = 0; i < T::kLoadsK; ++i)
+      *reinterpret_cast<u32x4*>(base + kst + i * T::kRowStepK * T::kPitchK) = kreg[i];
     // transpose 4 keys x kDV d -> kDV rows of 4 keys
 #pragma unroll
     for (int jj = 0; jj < T::kDV; ++jj) {
@@ -191,17 +235,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
       u32x2 o;
       o.x = __builtin_amdgcn_perm(vreg[1][w], vreg[0][w], sel);
       o.y = __builtin_amdgcn_perm(vreg[3][w], vreg[2][w], sel);
-      const int d = T::kDV * vdg + jj;
-      *reinterpret_cast<u32x2*>(vl + T::v_off(d, vkg >> 1) + ((vkg & 1) << 3)) = o;
-    }
-  };
-
-  auto advance = [&](int& seg, int& k0) {
-    k0 += kBK;
-    if (k0 >= a.kv_len[chunk_of(seg)]) {
-      k0 = 0;
-      ++seg;
-      while (seg < seg_end && a.kv_len[chunk_of(seg)] == 0) ++seg;
+      *reinterpret_cast<u32x2*>(base + vst + jj * T::kPitchV) = o;
     }
   };
 
@@ -211,26 +245,28 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   for (int i = 0; i < D / 32; ++i)
 #pragma unroll
     for (int r = 0; r < 16; ++r) o_acc[i][r] = 0.f;
-  float m_run = -INFINITY;  // running max of the raw scores of this lane's query
+  float m_ref = -INFINITY;  // reference maximum (raw scores) the accumulators are scaled to
   float l_run = 0.f;        // running sum over THIS lane's keys (halves combined at the end)
   const float c = a.scale_log2;
 
   if (n_tiles > 0) {
-    load_tile(ld_seg, ld_k0);
+    load_tile();
     store_tile(0);
-    advance(ld_seg, ld_k0);
   }
   __syncthreads();
 
-  const int krow = key_of_row(col);
+  // operand read addresses of this lane (per buffer: + buf * kBytesBuf)
+  const int kld = key_of_row(col) * T::kPitchK + 16 * hh;
+  const int vld = T::kBytesK + col * T::kPitchV + 16 * hh;
 
   for (int t = 0; t < n_tiles; ++t) {
     const bool has_next = (t + 1 < n_tiles);
-    if (has_next) load_tile(ld_seg, ld_k0);
+    if (has_next) load_tile();
 
-    const uint8_t* kl = lds + (t & 1) * T::kBytesBuf;
-    const uint8_t* vl = kl + T::kBytesK;
-    const int kvalid = a.kv_len[chunk_of(cp_seg)] - cp_k0;  // >= 1
+    const uint8_t* buf = lds + (t & 1) * T::kBytesBuf;
+    const uint8_t* kl = buf + kld;
+    const uint8_t* vl = buf + vld;
+    const int kvalid = cp_left;  // keys of this tile that exist (>= 1; a full tile has >= 64 left)
 
     // ---- S^T = K Q^T : two 32-key halves ------------------------------------------------
     f32x16 s_acc[2];
@@ -238,34 +274,45 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) s_acc[kb][r] = 0.f;
-      const int row = 32 * kb + krow;
 #pragma unroll
       for (int s = 0; s < D / 16; ++s) {
-        const bf16x8 ka = *reinterpret_cast<const bf16x8*>(kl + T::k_off(row, 2 * s + hh));
+        const bf16x8 ka = *reinterpret_cast<const bf16x8*>(kl + kb * 32 * T::kPitchK + 32 * s);
         s_acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[s], s_acc[kb], 0, 0, 0);
       }
     }
     if (kvalid < kBK) {
+      // the empty asm has side effects as far as the compiler knows, which keeps this a real
+      // branch: otherwise the selects below are hoisted out and run for every tile
+      asm volatile("" ::: "memory");
+      const int lim = kvalid;
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int key = 32 * kb + 16 * (r >> 3) + 8 * hh + (r & 7);
-          if (key >= kvalid) s_acc[kb][r] = -INFINITY;
+          if (key >= lim) s_acc[kb][r] = -INFINITY;
         }
     }
 
-    // ---- online softmax -----------------------------------------------------------------
+    // ---- online softmax with lazy rescaling -------------------------------------------------
     float mx = s_acc[0][0];
 #pragma unroll
     for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s_acc[0][r]);
 #pragma unroll
     for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s_acc[1][r]);
     mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const float m_new = fmaxf(m_run, mx);
-    const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c);
-    const float mc = m_new * c;
-    m_run = m_new;
+    // rescale only if some query's maximum grew by more than kTau (always true on the first tile)
+    if (__any((mx - m_ref) * c > kTau)) {
+      const float m_new = fmaxf(m_ref, mx);
+      const float alpha = __builtin_amdgcn_exp2f((m_ref - m_new) * c);
+      m_ref = m_new;
+      l_run *= alpha;
+#pragma unroll
+      for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o_acc[i][r] *= alpha;
+    }
+    const float mc = m_ref * c;
     float rs = 0.f;
     bf16x8 pf[2][2];
 #pragma unroll
@@ -280,37 +327,30 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
         pf[kb][r >> 3][r & 7] = pb.x;
         pf[kb][r >> 3][(r & 7) + 1] = pb.y;
       }
-    l_run = l_run * alpha + rs;
-#pragma unroll
-    for (int i = 0; i < D / 32; ++i)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) o_acc[i][r] *= alpha;
+    l_run += rs;
 
     // ---- O^T += V^T P^T -----------------------------------------------------------------
 #pragma unroll
     for (int db = 0; db < D / 32; ++db) {
-      const int d = 32 * db + col;
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
-          const bf16x8 va = *reinterpret_cast<const bf16x8*>(vl + T::v_off(d, 4 * kb + 2 * half + hh));
+          const bf16x8 va = *reinterpret_cast<const bf16x8*>(vl + db * 32 * T::kPitchV + 64 * kb + 32 * half);
           o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pf[kb][half], o_acc[db], 0, 0, 0);
         }
     }
 
-    advance(cp_seg, cp_k0);
-    if (has_next) {
-      store_tile((t + 1) & 1);
-      advance(ld_seg, ld_k0);
-    }
+    cp_left -= kBK;
+    if (cp_left <= 0) cp_next_chunk();
+    if (has_next) store_tile((t + 1) & 1);
     __syncthreads();
   }
 
   // ---- epilogue -------------------------------------------------------------------------
   const float l_tot = l_run + __shfl_xor(l_run, 32);
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-  const float lse = l_tot > 0.f ? (m_run * c + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f : -INFINITY;
+  const float lse = l_tot > 0.f ? (m_ref * c + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f : -INFINITY;
   const int qrow = q0 + col;
   if (hh == 0 && qrow < a.Sq) lse_ptr[((int64_t)b * a.H + h) * a.Sq + qrow] = lse;
 
@@ -350,19 +390,30 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   }
 }
 
+template <int D>
+static int launch_one(const AttnArgs& a, dim3 grid, hipStream_t stream) {
+  // more than 64 KB of dynamic LDS has to be allowed once per kernel and device
+  static thread_local int allowed_dev = -1;
+  int dev = 0;
+  if (int rc = hip_fail(hipGetDevice(&dev), "hipGetDevice")) return rc;
+  if (allowed_dev != dev) {
+    if (int rc = hip_fail(hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_fwd_kernel<D>),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, Tile<D>::kLdsBytes),
+                          "hipFuncSetAttribute"))
+      return rc;
+    allowed_dev = dev;
+  }
+  hipLaunchKernelGGL(attn_fwd_kernel<D>, grid, dim3(kThreads), Tile<D>::kLdsBytes, stream, a);
+  return hip_fail(hipGetLastError(), "attn_fwd launch");
+}
+
 int launch_attn(const AttnArgs& a, int D, int n_jobs, hipStream_t stream) {
   if (n_jobs <= 0 || a.total <= 0) return DT_OK;
   dim3 grid((unsigned)(a.per_xcd * kXcds), (unsigned)n_jobs, 1);
-  dim3 block(kThreads, 1, 1);
-  if (D == 128) {
-    hipLaunchKernelGGL(attn_fwd_kernel<128>, grid, block, 0, stream, a);
-  } else if (D == 64) {
-    hipLaunchKernelGGL(attn_fwd_kernel<64>, grid, block, 0, stream, a);
-  } else {
-    set_error("head dim %d not built (64 and 128 are)", D);
-    return DT_ERR_UNSUPPORTED;
-  }
-  return hip_fail(hipGetLastError(), "attn_fwd launch");
+  if (D == 128) return launch_one<128>(a, grid, stream);
+  if (D == 64) return launch_one<64>(a, grid, stream);
+  set_error("head dim %d not built (64 and 128 are)", D);
+  return DT_ERR_UNSUPPORTED;
 }
 
 }  // namespace dt

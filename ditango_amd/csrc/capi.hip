@@ -83,6 +83,10 @@ static int fill_common(AttnArgs& a, const void* q, int32_t B, int32_t Sq, int32_
       set_error("chunk %d: null or misaligned k/v", i);
       return DT_ERR_INVALID;
     }
+    if ((int64_t)kv_lens[i] * kv_ss * 2 >= (1ll << 31)) {
+      set_error("chunk %d: one (batch, head) plane spans 2 GiB or more; split the chunk", i);
+      return DT_ERR_INVALID;
+    }
     a.k[i] = static_cast<const __bf16*>(k_ptrs[i]);
     a.v[i] = static_cast<const __bf16*>(v_ptrs[i]);
     a.kv_len[i] = kv_lens[i];
@@ -131,7 +135,7 @@ extern "C" int dt_attn_jobs_fwd(const void* q, int32_t B, int32_t Sq, int32_t H,
       set_error("job chunk reference %d is outside the chunk table", job_chunks[e]);
       return DT_ERR_INVALID;
     }
-    a.job_chunks[e] = (uint8_t)job_chunks[e];
+    a.job_chunks[e] = job_chunks[e];
   }
   return launch_attn(a, D, n_jobs, (hipStream_t)stream);
 }

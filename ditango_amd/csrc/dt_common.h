@@ -31,7 +31,7 @@ struct AttnArgs {
   __bf16* job_out[DT_MAX_JOBS];
   float* job_lse[DT_MAX_JOBS];
   int32_t job_begin[DT_MAX_JOBS + 1];
-  uint8_t job_chunks[DT_MAX_JOB_ENTRIES];
+  int32_t job_chunks[DT_MAX_JOB_ENTRIES];
   // device-listed jobs (dev_ids != nullptr): job j computes chunk dev_ids[j] if j < *dev_count
   const int32_t* dev_ids;
   const int32_t* dev_count;
