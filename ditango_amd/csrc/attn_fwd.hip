@@ -5,13 +5,23 @@
 // of the reference.
 //
 // Shape of the computation
-//   * One workgroup = 4 wavefronts = 128 queries of one (batch, head); each
-//     wavefront owns 32 queries.  Two workgroups per CU (8 waves/CU, 256 VGPRs
-//     each) so one wave's softmax VALU work overlaps another's MFMA work.
-//   * KV is consumed in tiles of 64 keys.  K is staged in LDS as [key][d],
-//     V is transposed on the way in and staged as [d][key]; both are
-//     double-buffered and padded by 16 bytes per row so that the MFMA operand
-//     reads (ds_read_b128 with immediate offsets) are bank-conflict free.
+//   * One workgroup = 8 wavefronts = 256 queries of one (batch, head); each
+//     wavefront owns 32 queries.  One workgroup per CU, two wavefronts per SIMD
+//     (256 VGPRs each).
+//   * The 8 wavefronts form two groups of 4 that run the same loop ONE PHASE
+//     APART ("ping-pong"): while group A issues the MFMAs of a tile
+//     (O^T += V^T P^T of the previous tile, then S^T = K Q^T of this one), group B
+//     runs the VALU half (online softmax of its tile, transposing and storing the
+//     next K/V tile into LDS), and vice versa; a workgroup barrier separates the
+//     phases.  Each SIMD holds one wavefront of either group, so its matrix pipe
+//     and its vector ALU are busy at the same time instead of taking turns.
+//   * KV is consumed in tiles of 64 keys.  K is staged in LDS as [key][d] (two
+//     buffers), V is transposed on the way in and staged as [d][key] (three
+//     buffers, because the P V product of a tile runs one phase after its
+//     scores).  Rows are padded by 16 bytes so that the MFMA operand reads
+//     (ds_read_b128 with immediate offsets) are bank-conflict free.  Tiles come
+//     in through raw buffer loads: descriptor in scalar registers, loop-invariant
+//     lane offsets, and rows past the end of a chunk read as zeros.
 //   * Scores are computed TRANSPOSED, S^T = K Q^T, with v_mfma_f32_32x32x16_bf16:
 //     in the accumulator layout a lane then owns ONE query (column lane%32) and
 //     16 of the 32 keys of the tile, so the online-softmax max/sum are
@@ -23,8 +33,8 @@
 //     8 consecutive keys of one d-row of the transposed V tile.
 //   * O^T stays in registers as [d][query]: a rescale is a multiply by a per-lane
 //     scalar, and it is only done when some query's running maximum grew by more
-//     than 2^8 (the reference maximum may lag; the lse stays exact).  The epilogue transposes through LDS so that the global
-//     stores are 16 bytes per lane, 16 lanes per 256-byte row.
+//     than 2^8 (the reference maximum may lag; the lse stays exact).  The epilogue
+//     transposes through LDS so that the global stores are 16 bytes per lane.
 //   * Workgroups are mapped to (head, query tile) so that the 8 XCDs each work
 //     through a contiguous range of heads: the workgroups that share an XCD's
 //     L2 stream the same K/V.
@@ -40,40 +50,23 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-constexpr int kWaves = 4;
+constexpr int kWaves = 8;
 constexpr int kThreads = kWaves * 64;
-constexpr int kBQ = 128;  // queries per workgroup
-constexpr int kBK = 64;   // keys per tile
+constexpr int kBQ = kWaves * 32;  // queries per workgroup
+constexpr int kBK = 64;           // keys per tile
 constexpr int kXcds = 8;
+constexpr int kNumKBuf = 2;
+constexpr int kNumVBuf = 3;
 
 template <int N> struct VecOf;
 template <> struct VecOf<4> { typedef u32x4 type; };
 template <> struct VecOf<2> { typedef u32x2 type; };
+template <> struct VecOf<1> { typedef uint32_t type; };
 
 // Row permutation of the K operand: MFMA row i -> key (within a 32-key half tile).
 __device__ __forceinline__ int key_of_row(int i) {
   return (i & 19) | ((i & 4) << 1) | ((i & 8) >> 1);
 }
-
-template <int D>
-struct Tile {
-  // LDS tiles are padded by 16 bytes per row instead of swizzled: every operand read is then
-  // "lane base + compile-time constant", i.e. a ds_read_b128 with an immediate offset and no
-  // address arithmetic in the loop, and 16 consecutive rows still fall into 16 distinct
-  // 16-byte bank groups (pitch mod 256 is 16 or 144).
-  static constexpr int kPitchK = D * 2 + 16;          // one key, all d
-  static constexpr int kPitchV = kBK * 2 + 16;        // one d, 64 keys
-  static constexpr int kChunksK = D / 8;              // 16-byte chunks per K row
-  static constexpr int kBytesK = kBK * kPitchK;
-  static constexpr int kBytesV = D * kPitchV;
-  static constexpr int kBytesBuf = kBytesK + kBytesV;
-  static constexpr int kLoadsK = kBK * kChunksK / kThreads;  // 16-byte loads per thread
-  static constexpr int kRowStepK = kThreads / kChunksK;
-  static constexpr int kDV = D / 16;                  // d values per thread in the V transpose
-  static constexpr int kVW = kDV / 2;                 // dwords per V load
-  static constexpr int kPitchO = D * 2 + 16;          // epilogue row pitch
-  static constexpr int kLdsBytes = 2 * kBytesBuf;
-};
 
 // Raw buffer descriptor word 3 for gfx9-family targets (32-bit data format, no swizzle).
 constexpr int kRsrcFlags = 0x00020000;
@@ -88,10 +81,76 @@ template <>
 __device__ __forceinline__ u32x2 buffer_load_v<2>(__amdgpu_buffer_rsrc_t r, int voff) {
   return __builtin_amdgcn_raw_buffer_load_b64(r, voff, 0, 0);
 }
+template <>
+__device__ __forceinline__ uint32_t buffer_load_v<1>(__amdgpu_buffer_rsrc_t r, int voff) {
+  return __builtin_amdgcn_raw_buffer_load_b32(r, voff, 0, 0);
+}
+__device__ __forceinline__ uint32_t dword_of(uint32_t v, int) { return v; }
+__device__ __forceinline__ uint32_t dword_of(u32x2 v, int w) { return v[w]; }
+__device__ __forceinline__ uint32_t dword_of(u32x4 v, int w) { return v[w]; }
+
+// Workgroup barrier between the phases.  Waits for this wavefront's LDS traffic only:
+// global loads issued for a later tile stay in flight across it.
+__device__ __forceinline__ void phase_barrier() {
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+}
+// The same barrier with the results of the finished phase routed through it as in/out
+// operands.  Register-only code may otherwise migrate across an asm statement; tied to it,
+// the phase's work stays on its own side (the vector phase produces P^T, the matrix phase
+// produces S^T and updates O^T).
+template <typename V>
+__device__ __forceinline__ void phase_barrier_after_vector(V (&p)[2][2]) {
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier"
+               : "+v"(p[0][0]), "+v"(p[0][1]), "+v"(p[1][0]), "+v"(p[1][1])
+               :
+               : "memory");
+  __builtin_amdgcn_sched_barrier(0);
+}
+template <typename V, int NO>
+__device__ __forceinline__ void phase_barrier_after_matrix(V (&sa)[2], V (&oa)[NO]) {
+  __builtin_amdgcn_sched_barrier(0);
+  if constexpr (NO == 4) {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier"
+                 : "+v"(sa[0]), "+v"(sa[1]), "+v"(oa[0]), "+v"(oa[1]), "+v"(oa[2]), "+v"(oa[3])
+                 :
+                 : "memory");
+  } else {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier"
+                 : "+v"(sa[0]), "+v"(sa[1]), "+v"(oa[0]), "+v"(oa[1])
+                 :
+                 : "memory");
+  }
+  __builtin_amdgcn_sched_barrier(0);
+}
 
 // Largest growth of the running maximum (in log2 units of the scaled scores) that is
 // tolerated without rescaling the accumulators: probabilities then stay below 2^kTau.
 constexpr float kTau = 8.0f;
+
+template <int D>
+struct Tile {
+  // LDS tiles are padded by 16 bytes per row instead of swizzled: every operand read is then
+  // "lane base + compile-time constant", i.e. a ds_read_b128 with an immediate offset and no
+  // address arithmetic in the loop, and 16 consecutive rows still fall into 16 distinct
+  // 16-byte bank groups (pitch mod 256 is 16 or 144).
+  static constexpr int kPitchK = D * 2 + 16;          // one key, all d
+  static constexpr int kPitchV = kBK * 2 + 16;        // one d, 64 keys
+  static constexpr int kChunksK = D / 8;              // 16-byte chunks per K row
+  static constexpr int kBytesK = kBK * kPitchK;
+  static constexpr int kBytesV = D * kPitchV;
+  static constexpr int kOffV = kNumKBuf * kBytesK;    // V buffers follow the K buffers
+  static constexpr int kLoadsK = kBK * kChunksK / kThreads;  // 16-byte K loads per thread (2 or 1)
+  static constexpr int kRowStepK = kThreads / kChunksK;
+  static constexpr int kDV = D / 32;                  // d values per thread in the V transpose (4 keys x kDV d)
+  static constexpr int kVW = kDV / 2;                 // dwords per V load
+  static constexpr int kPitchO = D * 2 + 16;          // epilogue row pitch
+  static constexpr int kLdsTiles = kNumKBuf * kBytesK + kNumVBuf * kBytesV;
+  static constexpr int kLdsEpilogue = kWaves * 32 * kPitchO;
+  static constexpr int kLdsBytes = kLdsTiles > kLdsEpilogue ? kLdsTiles : kLdsEpilogue;
+};
 
 template <int D>
 __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a) {
@@ -115,7 +174,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   float* lse_ptr;
   if (a.dev_ids != nullptr) {
     if (job >= *a.dev_count) return;
-    single = a.dev_ids[job];
+    single = __builtin_amdgcn_readfirstlane(a.dev_ids[job]);  // uniform by construction; tell the compiler
     if (single < 0 || single >= a.n_chunks) return;  // never index the tables with a bad id
     seg_begin = 0;
     seg_end = 1;
@@ -132,13 +191,14 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     out_ptr = a.job_out[job];
     lse_ptr = a.job_lse[job];
   }
-  auto chunk_of = [&](int seg) -> int { return single >= 0 ? single : (int)a.job_chunks[seg]; };
+  auto chunk_of = [&](int seg) -> int { return single >= 0 ? single : a.job_chunks[seg]; };
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int col = lane & 31;   // query column (B operand) / operand row (A operand)
-  const int hh = lane >> 5;    // which half of the contraction dimension this lane feeds
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: keeps group/buffer arithmetic scalar
+  const int group = wave >> 2;  // 0: leads, 1: runs one phase behind
+  const int col = lane & 31;    // query column (B operand) / operand row (A operand)
+  const int hh = lane >> 5;     // which half of the contraction dimension this lane feeds
   const int q0 = qt * kBQ + wave * 32;
 
   // ---- Q fragments: B operand of S^T = K Q^T, kept in registers ----------------------
@@ -156,8 +216,8 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   for (int s = seg_begin; s < seg_end; ++s) n_tiles += (a.kv_len[chunk_of(s)] + kBK - 1) / kBK;
 
   // Two cursors walk the job's chunks tile by tile, all in scalar registers: the load cursor
-  // (one tile ahead: base pointers of the tile and keys left in its chunk) and the compute
-  // cursor (keys left in the chunk of the tile being consumed).
+  // (ahead of the compute cursor: base pointers of the tile and keys left in its chunk) and
+  // the compute cursor (keys left in the chunk of the tile whose scores are being computed).
   int ld_seg = seg_begin - 1, ld_left = 0;
   const uint8_t* ld_k = nullptr;
   const uint8_t* ld_v = nullptr;
@@ -182,12 +242,12 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   // thread -> K tile elements: 16-byte chunk kc of rows kr0 + i*kRowStepK
   const int kc = tid % T::kChunksK;
   const int kr0 = tid / T::kChunksK;
-  // thread -> V tile elements: keys 4*vkg..+3, d kDV*vdg..+kDV-1.  A half wavefront covers
-  // 16 key groups of one d group, so its transposed 8-byte LDS writes fill whole rows.
+  // thread -> V tile elements: keys 4*vkg..+3, d kDV*vdg..+kDV-1.  A quarter wavefront covers
+  // the 16 key groups of one d group, so the transposed 8-byte LDS writes fill whole rows.
   const int vkg = tid & 15;
   const int vdg = tid >> 4;
   const uint32_t row_bytes = (uint32_t)a.kv_ss * 2u;
-  // byte offsets from the tile's first key, loop invariant for full tiles
+  // byte offsets from the tile's first key, loop invariant
   uint32_t koff[T::kLoadsK], voff[4];
 #pragma unroll
   for (int i = 0; i < T::kLoadsK; ++i) koff[i] = (uint32_t)(kr0 + i * T::kRowStepK) * row_bytes + 16u * kc;
@@ -198,11 +258,11 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   VLoad vreg[4];
 
   const int64_t tile_bytes = (int64_t)kBK * row_bytes;
-  // Loads the tile under the load cursor into registers and moves the cursor on.  The loads
-  // are raw buffer loads: the descriptor (base of the tile's first key for this batch and
-  // head, number of valid bytes) lives in scalar registers, the lane offsets are loop
-  // invariant, and rows past the end of the chunk are out of range for the hardware bounds
-  // check and come back as zeros (their scores are masked to -inf; zero V rows add nothing).
+  // Loads this thread's share of the tile under the load cursor into registers and moves the
+  // cursor on.  Raw buffer loads: the descriptor (base of the tile's first key for this batch
+  // and head, number of valid bytes) lives in scalar registers, and rows past the end of the
+  // chunk fail the hardware bounds check and come back as zeros (their scores are masked to
+  // -inf; zero V rows add nothing).
   auto load_tile = [&]() {
     const uint32_t valid = (uint32_t)(ld_left - 1) * row_bytes + (uint32_t)(D * 2);
     const __amdgpu_buffer_rsrc_t rk =
@@ -219,23 +279,24 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     if (ld_left <= 0) ld_next_chunk();
   };
 
-  // LDS write addresses of this thread (per buffer: + buf * kBytesBuf)
+  // LDS write addresses of this thread within a K / V buffer
   const int kst = kr0 * T::kPitchK + 16 * kc;
-  const int vst = T::kBytesK + (T::kDV * vdg) * T::kPitchV + 8 * vkg;
-  auto store_tile = [&](int buf) {
-    uint8_t* base = lds + buf * T::kBytesBuf;
+  const int vst = (T::kDV * vdg) * T::kPitchV + 8 * vkg;
+  auto store_tile = [&](int tile) {
+    uint8_t* kbuf = lds + (tile % kNumKBuf) * T::kBytesK;
+    uint8_t* vbuf = lds + T::kOffV + (tile % kNumVBuf) * T::kBytesV;
 #pragma unroll
     for (int i = 0; i < T::kLoadsK; ++i)
-      *reinterpret_cast<u32x4*>(base + kst + i * T::kRowStepK * T::kPitchK) = kreg[i];
+      *reinterpret_cast<u32x4*>(kbuf + kst + i * T::kRowStepK * T::kPitchK) = kreg[i];
     // transpose 4 keys x kDV d -> kDV rows of 4 keys
 #pragma unroll
     for (int jj = 0; jj < T::kDV; ++jj) {
       const int w = jj >> 1;
       const uint32_t sel = (jj & 1) ? 0x07060302u : 0x05040100u;
       u32x2 o;
-      o.x = __builtin_amdgcn_perm(vreg[1][w], vreg[0][w], sel);
-      o.y = __builtin_amdgcn_perm(vreg[3][w], vreg[2][w], sel);
-      *reinterpret_cast<u32x2*>(base + vst + jj * T::kPitchV) = o;
+      o.x = __builtin_amdgcn_perm(dword_of(vreg[1], w), dword_of(vreg[0], w), sel);
+      o.y = __builtin_amdgcn_perm(dword_of(vreg[3], w), dword_of(vreg[2], w), sel);
+      *reinterpret_cast<u32x2*>(vbuf + vst + jj * T::kPitchV) = o;
     }
   };
 
@@ -249,27 +310,17 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   float l_run = 0.f;        // running sum over THIS lane's keys (halves combined at the end)
   const float c = a.scale_log2;
 
-  if (n_tiles > 0) {
-    load_tile();
-    store_tile(0);
-  }
-  __syncthreads();
-
-  // operand read addresses of this lane (per buffer: + buf * kBytesBuf)
+  // operand read addresses of this lane within a K / V buffer
   const int kld = key_of_row(col) * T::kPitchK + 16 * hh;
-  const int vld = T::kBytesK + col * T::kPitchV + 16 * hh;
+  const int vld = T::kOffV + col * T::kPitchV + 16 * hh;
 
-  for (int t = 0; t < n_tiles; ++t) {
-    const bool has_next = (t + 1 < n_tiles);
-    if (has_next) load_tile();
+  f32x16 s_acc[2];       // S^T of the tile whose softmax comes next
+  bf16x8 p_frag[2][2];   // P^T of the tile whose P V product comes next
+  int cp_valid = 0;      // keys that exist in the tile held in s_acc
 
-    const uint8_t* buf = lds + (t & 1) * T::kBytesBuf;
-    const uint8_t* kl = buf + kld;
-    const uint8_t* vl = buf + vld;
-    const int kvalid = cp_left;  // keys of this tile that exist (>= 1; a full tile has >= 64 left)
-
-    // ---- S^T = K Q^T : two 32-key halves ------------------------------------------------
-    f32x16 s_acc[2];
+  // S^T = K Q^T for tile `tile` only (first matrix phase)
+  auto qk_only = [&](int tile) {
+    const uint8_t* kl = lds + kld + (tile % kNumKBuf) * T::kBytesK;
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
@@ -280,11 +331,97 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
         s_acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[s], s_acc[kb], 0, 0, 0);
       }
     }
-    if (kvalid < kBK) {
+  };
+
+  // One matrix phase: O^T += V^T P^T for tile `tile`, then S^T = K Q^T for tile `tile + 1`,
+  // as ONE stream of MFMAs fed by a ring of LDS reads kept kRing fragments ahead, so that the
+  // single wavefront of this SIMD that is in its matrix phase never waits for LDS latency.
+  // (After the last tile the second half recomputes scores on a stale K buffer; they are unused.)
+  constexpr int kPV = D / 32 * 4;       // fragments of the P V product
+  constexpr int kQK = 2 * (D / 16);     // fragments of the score product
+  constexpr int kFrags = kPV + kQK;
+  constexpr int kRing = 8;
+  auto matrix_phase = [&](int tile) {
+    const uint8_t* vl = lds + vld + (tile % kNumVBuf) * T::kBytesV;
+    const uint8_t* kl = lds + kld + ((tile + 1) % kNumKBuf) * T::kBytesK;
+    auto frag = [&](int i) -> bf16x8 {
+      if (i < kPV) {
+        const int db = i >> 2, kb = (i >> 1) & 1, half = i & 1;
+        return *reinterpret_cast<const bf16x8*>(vl + db * 32 * T::kPitchV + 64 * kb + 32 * half);
+      }
+      const int j = i - kPV;
+      const int kb = j / (D / 16), sidx = j % (D / 16);
+      return *reinterpret_cast<const bf16x8*>(kl + kb * 32 * T::kPitchK + 32 * sidx);
+    };
+    bf16x8 ring[kRing];
+#pragma unroll
+    for (int i = 0; i < kRing; ++i) ring[i] = frag(i);
+#pragma unroll
+    for (int i = 0; i < kFrags; ++i) {
+      const bf16x8 cur = ring[i % kRing];
+      if (i + kRing < kFrags) ring[i % kRing] = frag(i + kRing);
+      if (i < kPV) {
+        const int db = i >> 2, kb = (i >> 1) & 1, half = i & 1;
+        o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur, p_frag[kb][half], o_acc[db], 0, 0, 0);
+      } else {
+        const int j = i - kPV;
+        const int kb = j / (D / 16), sidx = j % (D / 16);
+        if (sidx == 0) {
+          f32x16 zero;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) zero[r] = 0.f;
+          s_acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur, qf[sidx], zero, 0, 0, 0);
+        } else {
+          s_acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur, qf[sidx], s_acc[kb], 0, 0, 0);
+        }
+      }
+    }
+    // pin the order: kRing reads up front, then one read behind every MFMA
+    __builtin_amdgcn_sched_group_barrier(0x100, kRing, 0);
+#pragma unroll
+    for (int i = 0; i < kFrags - kRing; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, kRing, 0);
+  };
+
+  // ---- prologue: tile 0 from everybody; the trailing group also brings its share of tile 1
+  //      and then waits one phase, which is what staggers the two groups ---------------------
+  const int pf = 1 + group;  // how many tiles ahead of its softmax a group stores
+  int n_loaded = 0;          // tiles this thread has written its share of
+  if (n_tiles > 0) {
+    load_tile();
+    store_tile(0);
+    n_loaded = 1;
+  }
+  if (group == 1 && n_tiles > 1) load_tile();
+  phase_barrier();
+  if (group == 1) {
+    if (n_tiles > 1) {
+      store_tile(1);
+      n_loaded = 2;
+    }
+    phase_barrier();
+  }
+  // first matrix phase: fetch ahead, scores of tile 0
+  bool fetched = (n_loaded < n_tiles);
+  if (fetched) load_tile();
+  if (n_tiles > 0) {
+    qk_only(0);
+    cp_valid = cp_left;
+    cp_left -= kBK;
+    if (cp_left <= 0) cp_next_chunk();
+  }
+  phase_barrier_after_matrix(s_acc, o_acc);
+
+  for (int t = 0; t < n_tiles; ++t) {
+    // ======== vector phase: online softmax of tile t, LDS fill of the fetched tile ========
+    if (cp_valid < kBK) {
       // the empty asm has side effects as far as the compiler knows, which keeps this a real
       // branch: otherwise the selects below are hoisted out and run for every tile
       asm volatile("" ::: "memory");
-      const int lim = kvalid;
+      const int lim = cp_valid;
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -293,8 +430,6 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
           if (key >= lim) s_acc[kb][r] = -INFINITY;
         }
     }
-
-    // ---- online softmax with lazy rescaling -------------------------------------------------
     float mx = s_acc[0][0];
 #pragma unroll
     for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s_acc[0][r]);
@@ -313,8 +448,12 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
         for (int r = 0; r < 16; ++r) o_acc[i][r] *= alpha;
     }
     const float mc = m_ref * c;
-    float rs = 0.f;
-    bf16x8 pf[2][2];
+    // The row sum is taken over the bf16-ROUNDED probabilities, i.e. exactly the weights the
+    // P V product uses, two per instruction (v_dot2c_f32_bf16 against (1, 1)).
+    float rs0 = 0.f, rs1 = 0.f;
+    bf16x2 ones;
+    ones.x = (__bf16)1.0f;
+    ones.y = (__bf16)1.0f;
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -322,30 +461,30 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
         f32x2 p;
         p.x = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[kb][r], c, -mc));
         p.y = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[kb][r + 1], c, -mc));
-        rs += p.x + p.y;
         const bf16x2 pb = __builtin_convertvector(p, bf16x2);
-        pf[kb][r >> 3][r & 7] = pb.x;
-        pf[kb][r >> 3][(r & 7) + 1] = pb.y;
+        if (r & 2) rs1 = __builtin_amdgcn_fdot2_f32_bf16(pb, ones, rs1, false);
+        else rs0 = __builtin_amdgcn_fdot2_f32_bf16(pb, ones, rs0, false);
+        p_frag[kb][r >> 3][r & 7] = pb.x;
+        p_frag[kb][r >> 3][(r & 7) + 1] = pb.y;
       }
-    l_run += rs;
-
-    // ---- O^T += V^T P^T -----------------------------------------------------------------
-#pragma unroll
-    for (int db = 0; db < D / 32; ++db) {
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int half = 0; half < 2; ++half) {
-          const bf16x8 va = *reinterpret_cast<const bf16x8*>(vl + db * 32 * T::kPitchV + 64 * kb + 32 * half);
-          o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pf[kb][half], o_acc[db], 0, 0, 0);
-        }
+    l_run += rs0 + rs1;
+    if (fetched) {
+      store_tile(n_loaded);
+      ++n_loaded;
     }
+    phase_barrier_after_vector(p_frag);
 
+    // ======== matrix phase: fetch ahead, O^T += V^T P^T (tile t), S^T = K Q^T (tile t+1) ========
+    fetched = (n_loaded < n_tiles);
+    if (fetched) load_tile();
+    matrix_phase(t);
+    cp_valid = cp_left;
     cp_left -= kBK;
     if (cp_left <= 0) cp_next_chunk();
-    if (has_next) store_tile((t + 1) & 1);
-    __syncthreads();
+    phase_barrier_after_matrix(s_acc, o_acc);
   }
+  // the leading group waits out the phase it is ahead
+  if (group == 0) phase_barrier();
 
   // ---- epilogue -------------------------------------------------------------------------
   const float l_tot = l_run + __shfl_xor(l_run, 32);
@@ -355,7 +494,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   if (hh == 0 && qrow < a.Sq) lse_ptr[((int64_t)b * a.H + h) * a.Sq + qrow] = lse;
 
   // O^T (registers, [d][query]) -> LDS [query][d] bf16 -> coalesced 16-byte stores.
-  // The loop ended with a barrier, so the tile buffers are free.
+  phase_barrier();  // every wavefront is done with the tile buffers
   uint8_t* ol = lds + wave * (32 * T::kPitchO);
 #pragma unroll
   for (int db = 0; db < D / 32; ++db)
@@ -373,7 +512,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
       const int d = 32 * db + 8 * g + 4 * hh;
       *reinterpret_cast<bf16x4*>(ol + col * T::kPitchO + d * 2) = pk;
     }
-  __syncthreads();
+  phase_barrier();
   constexpr int kLanesPerRow = D / 8;
   constexpr int kRowsPerPass = 64 / kLanesPerRow;
   const int rr = lane / kLanesPerRow;

@@ -64,7 +64,7 @@ static int fill_common(AttnArgs& a, const void* q, int32_t B, int32_t Sq, int32_
   a.q = static_cast<const __bf16*>(q);
   a.q_sb = q_sb; a.q_ss = q_ss; a.q_sh = q_sh;
   a.B = B; a.H = H; a.Sq = Sq;
-  a.nqt = (Sq + 127) / 128;
+  a.nqt = (Sq + 255) / 256;  // 256 queries per workgroup
   const int64_t total = (int64_t)B * H * a.nqt;
   if (total > (1 << 28)) {
     set_error("too many query tiles (%lld)", (long long)total);
