@@ -210,6 +210,12 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
 #pragma unroll
     for (int s = 0; s < D / 16; ++s) qf[s] = *reinterpret_cast<const bf16x8*>(qp + 16 * s);
   }
+  // Route the fragments through an empty asm: they are then defined by it, not by loads.  The
+  // compiler otherwise keeps "Q may still be in flight" alive round the loop and waits for ALL
+  // outstanding vector-memory loads (including the K/V prefetch just issued) before the first
+  // MFMA that reads Q in every iteration.
+#pragma unroll
+  for (int s = 0; s < D / 16; ++s) asm volatile("" : "+v"(qf[s]));
 
   // ---- tile bookkeeping -----------------------------------------------------------------
   int n_tiles = 0;
