@@ -4,7 +4,7 @@
 //   * schedule builder      (per-chunk generalisation of core/attention.py:90-116)
 //   * relative-L1 sums      (utils.py:214-241)
 //
-// Work decomposition of the row kernels: one workgroup handles kRowsPerWg
+// Work decomposition of the row kernels: one workgroup handles a run of
 // consecutive queries of ONE (batch, head).  A group of D/8 lanes owns one row
 // (query, head) and moves 16 bytes of bf16 (8 elements) per lane per state, so a
 // row is one contiguous 128/256-byte access, and the lse values of consecutive
@@ -17,7 +17,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kThreads = 256;
-constexpr int kQPerWg = 64;  // queries per workgroup (several passes)
+constexpr int kBatch = 8;  // states whose loads are in flight together
 
 struct MergeArgs {
   int32_t n;
@@ -36,18 +36,45 @@ __device__ __forceinline__ int64_t lse_index(bool bsh, int b, int h, int s, int 
   return bsh ? ((int64_t)b * Sq + s) * H + h : ((int64_t)b * H + h) * Sq + s;
 }
 
-__device__ __forceinline__ void load8(const void* base, bool fp32, int64_t elem, float (&x)[8]) {
+// A lane owns 8 elements of its row: [4c, 4c+4) and [D/2 + 4c, D/2 + 4c + 4), c = lane index
+// within the row's lane group.  Every load/store instruction is then contiguous across the
+// group (8 bytes per lane for bf16, 16 bytes per lane for fp32), for either dtype on either
+// side; a lane owning 8 consecutive elements would write fp32 as two interleaved half-sector
+// streams.
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+struct Row8 {
+  u32x4 lo, hi;  // bf16: lo.xy = first group, lo.zw = second group; fp32: lo / hi = the two groups
+};
+
+template <int D>
+__device__ __forceinline__ Row8 load_row8(const void* base, bool fp32, int64_t row_elem, int c) {
+  Row8 r;
   if (fp32) {
-    const f32x4* p = reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(base) + elem);
-    const f32x4 a = p[0], b = p[1];
-    x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w;
-    x[4] = b.x; x[5] = b.y; x[6] = b.z; x[7] = b.w;
+    const float* p = reinterpret_cast<const float*>(base) + row_elem + 4 * c;
+    r.lo = *reinterpret_cast<const u32x4*>(p);
+    r.hi = *reinterpret_cast<const u32x4*>(p + D / 2);
   } else {
-    const u32x4 v = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(base) + elem);
+    const uint16_t* p = reinterpret_cast<const uint16_t*>(base) + row_elem + 4 * c;
+    const u32x2 g0 = *reinterpret_cast<const u32x2*>(p);
+    const u32x2 g1 = *reinterpret_cast<const u32x2*>(p + D / 2);
+    r.lo.x = g0.x; r.lo.y = g0.y; r.lo.z = g1.x; r.lo.w = g1.y;
+    r.hi = r.lo;
+  }
+  return r;
+}
+
+__device__ __forceinline__ void unpack_row8(const Row8& r, bool fp32, float (&x)[8]) {
+  if (fp32) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      x[2 * i] = __uint_as_float(v[i] << 16);
-      x[2 * i + 1] = __uint_as_float(v[i] & 0xffff0000u);
+      x[i] = __uint_as_float(r.lo[i]);
+      x[4 + i] = __uint_as_float(r.hi[i]);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      x[2 * i] = __uint_as_float(r.lo[i] << 16);
+      x[2 * i + 1] = __uint_as_float(r.lo[i] & 0xffff0000u);
     }
   }
 }
@@ -62,67 +89,163 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, b);
 }
 
-__device__ __forceinline__ void store8(void* base, bool fp32, int64_t elem, const float (&x)[8]) {
+template <int D>
+__device__ __forceinline__ void store_row8(void* base, bool fp32, int64_t row_elem, int c, const float (&x)[8]) {
   if (fp32) {
-    f32x4* p = reinterpret_cast<f32x4*>(reinterpret_cast<float*>(base) + elem);
-    f32x4 a, b;
-    a.x = x[0]; a.y = x[1]; a.z = x[2]; a.w = x[3];
-    b.x = x[4]; b.y = x[5]; b.z = x[6]; b.w = x[7];
-    p[0] = a;
-    p[1] = b;
-  } else {
-    u32x4 v;
+    float* p = reinterpret_cast<float*>(base) + row_elem + 4 * c;
+    u32x4 a, b;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) v[i] = pack_bf16x2(x[2 * i], x[2 * i + 1]);
-    *reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(base) + elem) = v;
+    for (int i = 0; i < 4; ++i) {
+      a[i] = __float_as_uint(x[i]);
+      b[i] = __float_as_uint(x[4 + i]);
+    }
+    *reinterpret_cast<u32x4*>(p) = a;
+    *reinterpret_cast<u32x4*>(p + D / 2) = b;
+  } else {
+    uint16_t* p = reinterpret_cast<uint16_t*>(base) + row_elem + 4 * c;
+    u32x2 g0, g1;
+    g0.x = pack_bf16x2(x[0], x[1]);
+    g0.y = pack_bf16x2(x[2], x[3]);
+    g1.x = pack_bf16x2(x[4], x[5]);
+    g1.y = pack_bf16x2(x[6], x[7]);
+    __builtin_nontemporal_store(g0, reinterpret_cast<u32x2*>(p));
+    __builtin_nontemporal_store(g1, reinterpret_cast<u32x2*>(p + D / 2));
   }
 }
 
-template <int D>
+// Workgroup -> (query run, batch*head) with the head index fastest: workgroups that run at
+// the same time then cover whole [query][head][d] rows, i.e. contiguous memory, in every
+// stream, instead of one 2*D-byte slice out of every H*2*D bytes.
+__device__ __forceinline__ void decode_wg(int wg, int B, int H, int& st, int& b, int& h) {
+  const int bh_count = B * H;
+  st = wg / bh_count;
+  const int bh = wg - st * bh_count;
+  b = bh / H;
+  h = bh - b * H;
+}
+
+// Running state of one output row while states are folded in.
+struct RowAcc {
+  float acc[8];
+  float m, den;
+};
+
+// Folds states [i0, i0 + NB) into kMergeRows rows at once.  Branch free: all NB x kMergeRows
+// lse loads and row loads are issued back to back before the first use (the pointers come
+// from the kernel arguments with a uniform index, so they are scalar loads issued together).
+constexpr int kMergeRows = 2;
+
+template <int D, int NB, bool ALL_BF16>
+__device__ __forceinline__ void merge_batch(const MergeArgs& a, int i0, int b, int h, const int (&s)[kMergeRows],
+                                            const bool (&live)[kMergeRows], const int64_t (&elem)[kMergeRows], int cc,
+                                            RowAcc (&ra)[kMergeRows]) {
+  float l[kMergeRows][NB];
+  Row8 r[kMergeRows][NB];
+  u32x4 rb[kMergeRows][NB];
+#pragma unroll
+  for (int j = 0; j < NB; ++j) {
+    const int i = i0 + j;
+    const float* lp = a.lse[i];
+    const void* op = a.out[i];
+    const bool bsh = (a.bsh_mask >> i) & 1;
+#pragma unroll
+    for (int p = 0; p < kMergeRows; ++p) {
+      if (live[p]) {
+        l[p][j] = lp[lse_index(bsh, b, h, s[p], a.H, a.Sq)];
+        if (ALL_BF16) {
+          const uint16_t* q = reinterpret_cast<const uint16_t*>(op) + elem[p] + 4 * cc;
+          const u32x2 g0 = *reinterpret_cast<const u32x2*>(q);
+          const u32x2 g1 = *reinterpret_cast<const u32x2*>(q + D / 2);
+          rb[p][j].x = g0.x; rb[p][j].y = g0.y; rb[p][j].z = g1.x; rb[p][j].w = g1.y;
+        } else {
+          r[p][j] = load_row8<D>(op, (a.fp32_mask >> i) & 1, elem[p], cc);
+        }
+      } else {
+        l[p][j] = -INFINITY;
+      }
+    }
+  }
+#pragma unroll
+  for (int p = 0; p < kMergeRows; ++p) {
+    float m_new = ra[p].m;
+#pragma unroll
+    for (int j = 0; j < NB; ++j) m_new = fmaxf(m_new, l[p][j]);
+    if (m_new > -INFINITY) {
+      const float rescale = __expf(ra[p].m - m_new);  // exp(-inf) = 0 on the first non-empty batch
+      ra[p].den *= rescale;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) ra[p].acc[k] *= rescale;
+#pragma unroll
+      for (int j = 0; j < NB; ++j) {
+        const float w = __expf(l[p][j] - m_new);
+        float x[8];
+        if (ALL_BF16) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            x[2 * q] = __uint_as_float(rb[p][j][q] << 16);
+            x[2 * q + 1] = __uint_as_float(rb[p][j][q] & 0xffff0000u);
+          }
+        } else {
+          unpack_row8(r[p][j], (a.fp32_mask >> (i0 + j)) & 1, x);
+        }
+        ra[p].den += w;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) ra[p].acc[k] = __builtin_fmaf(w, x[k], ra[p].acc[k]);
+      }
+      ra[p].m = m_new;
+    }
+  }
+}
+
+// One workgroup = kMergeRows * 256/(D/8) consecutive queries of one (batch, head); a group of
+// D/8 lanes owns kMergeRows rows.  States are consumed in batches of kBatch (the remainder
+// through a fully unrolled smaller batch) and folded with the running-maximum rescale.
+template <int D, bool ALL_BF16>
 __global__ __launch_bounds__(kThreads) void merge_states_kernel(const MergeArgs a) {
   constexpr int kLanesPerRow = D / 8;
   constexpr int kRowsPerPass = kThreads / kLanesPerRow;
-  const int n_st = (a.Sq + kQPerWg - 1) / kQPerWg;
-  const int wg = blockIdx.x;
-  const int st = wg % n_st;
-  const int bh = wg / n_st;
-  const int b = bh / a.H;
-  const int h = bh - b * a.H;
+  constexpr int kRowsPerWg = kRowsPerPass * kMergeRows;
+  int st, b, h;
+  decode_wg(blockIdx.x, a.B, a.H, st, b, h);
   const int rr = threadIdx.x / kLanesPerRow;
   const int cc = threadIdx.x % kLanesPerRow;
-#pragma unroll 1
-  for (int p = 0; p < kQPerWg / kRowsPerPass; ++p) {
-    const int s = st * kQPerWg + p * kRowsPerPass + rr;
-    if (s >= a.Sq) break;
-    const int64_t elem = (((int64_t)b * a.Sq + s) * a.H + h) * D + cc * 8;
-    // pass 1: the maximum lse
-    float m = -INFINITY;
-    for (int i = 0; i < a.n; ++i) {
-      const float l = a.lse[i][lse_index((a.bsh_mask >> i) & 1, b, h, s, a.H, a.Sq)];
-      m = fmaxf(m, l);
-    }
-    float acc[8];
+  int s[kMergeRows];
+  bool live[kMergeRows];
+  int64_t elem[kMergeRows];
+  RowAcc ra[kMergeRows];
 #pragma unroll
-    for (int k = 0; k < 8; ++k) acc[k] = 0.f;
-    float den = 0.f;
-    if (m > -INFINITY) {
-#pragma unroll 4
-      for (int i = 0; i < a.n; ++i) {
-        const float l = a.lse[i][lse_index((a.bsh_mask >> i) & 1, b, h, s, a.H, a.Sq)];
-        const float w = __expf(l - m);
-        float x[8];
-        load8(a.out[i], (a.fp32_mask >> i) & 1, elem, x);
-        den += w;
+  for (int p = 0; p < kMergeRows; ++p) {
+    s[p] = st * kRowsPerWg + p * kRowsPerPass + rr;
+    live[p] = s[p] < a.Sq;
+    elem[p] = (((int64_t)b * a.Sq + s[p]) * a.H + h) * D;
+    ra[p].m = -INFINITY;
+    ra[p].den = 0.f;
 #pragma unroll
-        for (int k = 0; k < 8; ++k) acc[k] = __builtin_fmaf(w, x[k], acc[k]);
-      }
-    }
-    const float inv = den > 0.f ? 1.f / den : 0.f;
+    for (int k = 0; k < 8; ++k) ra[p].acc[k] = 0.f;
+  }
+  int i0 = 0;
+  for (; i0 + kBatch <= a.n; i0 += kBatch) merge_batch<D, kBatch, ALL_BF16>(a, i0, b, h, s, live, elem, cc, ra);
+  switch (a.n - i0) {
+    case 1: merge_batch<D, 1, ALL_BF16>(a, i0, b, h, s, live, elem, cc, ra); break;
+    case 2: merge_batch<D, 2, ALL_BF16>(a, i0, b, h, s, live, elem, cc, ra); break;
+    case 3: merge_batch<D, 3, ALL_BF16>(a, i0, b, h, s, live, elem, cc, ra); break;
+    case 4: merge_batch<D, 4, ALL_BF16>(a, i0, b, h, s, live, elem, cc, ra); break;
+    case 5: merge_batch<D, 5, ALL_BF16>(a, i0, b, h, s, live, elem, cc, ra); break;
+    case 6: merge_batch<D, 6, ALL_BF16>(a, i0, b, h, s, live, elem, cc, ra); break;
+    case 7: merge_batch<D, 7, ALL_BF16>(a, i0, b, h, s, live, elem, cc, ra); break;
+    default: break;
+  }
 #pragma unroll
-    for (int k = 0; k < 8; ++k) acc[k] *= inv;
-    store8(a.dst_out, a.dst_fp32 != 0, elem, acc);
+  for (int p = 0; p < kMergeRows; ++p) {
+    if (!live[p]) continue;
+    const float inv = ra[p].den > 0.f ? 1.f / ra[p].den : 0.f;
+    float o[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) o[k] = ra[p].acc[k] * inv;
+    store_row8<D>(a.dst_out, a.dst_fp32 != 0, elem[p], cc, o);
     if (cc == 0 && a.dst_lse != nullptr)
-      a.dst_lse[lse_index(a.dst_bsh != 0, b, h, s, a.H, a.Sq)] = den > 0.f ? m + __logf(den) : -INFINITY;
+      a.dst_lse[lse_index(a.dst_bsh != 0, b, h, s[p], a.H, a.Sq)] =
+          ra[p].den > 0.f ? ra[p].m + __logf(ra[p].den) : -INFINITY;
   }
 }
 
@@ -135,29 +258,38 @@ struct CopyArgs {
   int32_t src_fp32, src_bsh, dst_fp32, dst_bsh;
 };
 
+constexpr int kCopyRows = 2;  // rows per lane group, both in flight
+
 template <int D>
 __global__ __launch_bounds__(kThreads) void state_copy_kernel(const CopyArgs a) {
   constexpr int kLanesPerRow = D / 8;
   constexpr int kRowsPerPass = kThreads / kLanesPerRow;
-  const int n_st = (a.Sq + kQPerWg - 1) / kQPerWg;
-  const int wg = blockIdx.x;
-  const int st = wg % n_st;
-  const int bh = wg / n_st;
-  const int b = bh / a.H;
-  const int h = bh - b * a.H;
+  constexpr int kRowsPerWg = kRowsPerPass * kCopyRows;
+  int st, b, h;
+  decode_wg(blockIdx.x, a.B, a.H, st, b, h);
   const int rr = threadIdx.x / kLanesPerRow;
   const int cc = threadIdx.x % kLanesPerRow;
+  Row8 r[kCopyRows];
+  float l[kCopyRows];
+  const bool copy_lse = (cc == 0 && a.dst_lse != nullptr && a.src_lse != nullptr);
 #pragma unroll
-  for (int p = 0; p < kQPerWg / kRowsPerPass; ++p) {
-    const int s = st * kQPerWg + p * kRowsPerPass + rr;
+  for (int p = 0; p < kCopyRows; ++p) {
+    const int s = st * kRowsPerWg + p * kRowsPerPass + rr;
     if (s < a.Sq) {
-      const int64_t elem = (((int64_t)b * a.Sq + s) * a.H + h) * D + cc * 8;
+      const int64_t elem = (((int64_t)b * a.Sq + s) * a.H + h) * D;
+      r[p] = load_row8<D>(a.src_out, a.src_fp32 != 0, elem, cc);
+      if (copy_lse) l[p] = a.src_lse[lse_index(a.src_bsh != 0, b, h, s, a.H, a.Sq)];
+    }
+  }
+#pragma unroll
+  for (int p = 0; p < kCopyRows; ++p) {
+    const int s = st * kRowsPerWg + p * kRowsPerPass + rr;
+    if (s < a.Sq) {
+      const int64_t elem = (((int64_t)b * a.Sq + s) * a.H + h) * D;
       float x[8];
-      load8(a.src_out, a.src_fp32 != 0, elem, x);
-      store8(a.dst_out, a.dst_fp32 != 0, elem, x);
-      if (cc == 0 && a.dst_lse != nullptr && a.src_lse != nullptr)
-        a.dst_lse[lse_index(a.dst_bsh != 0, b, h, s, a.H, a.Sq)] =
-            a.src_lse[lse_index(a.src_bsh != 0, b, h, s, a.H, a.Sq)];
+      unpack_row8(r[p], a.src_fp32 != 0, x);
+      store_row8<D>(a.dst_out, a.dst_fp32 != 0, elem, cc, x);
+      if (copy_lse) a.dst_lse[lse_index(a.dst_bsh != 0, b, h, s, a.H, a.Sq)] = l[p];
     }
   }
 }
@@ -244,17 +376,21 @@ __global__ __launch_bounds__(kThreads) void rel_l1_sums_kernel(const float* a, c
 // ---- host-side launchers ---------------------------------------------------------------
 
 int launch_merge(const MergeArgs& a, int D, hipStream_t stream) {
-  const int n_st = (a.Sq + kQPerWg - 1) / kQPerWg;
+  const int rows_per_wg = kThreads / (D / 8) * kMergeRows;
+  const int n_st = (a.Sq + rows_per_wg - 1) / rows_per_wg;
   const int64_t wgs = (int64_t)a.B * a.H * n_st;
   if (wgs <= 0) return DT_OK;
   if (wgs > 0x7fffffffLL) {
     set_error("merge grid too large");
     return DT_ERR_INVALID;
   }
+  const bool all_bf16 = (a.fp32_mask == 0);
   if (D == 128) {
-    hipLaunchKernelGGL(merge_states_kernel<128>, dim3((unsigned)wgs), dim3(kThreads), 0, stream, a);
+    if (all_bf16) hipLaunchKernelGGL((merge_states_kernel<128, true>), dim3((unsigned)wgs), dim3(kThreads), 0, stream, a);
+    else hipLaunchKernelGGL((merge_states_kernel<128, false>), dim3((unsigned)wgs), dim3(kThreads), 0, stream, a);
   } else if (D == 64) {
-    hipLaunchKernelGGL(merge_states_kernel<64>, dim3((unsigned)wgs), dim3(kThreads), 0, stream, a);
+    if (all_bf16) hipLaunchKernelGGL((merge_states_kernel<64, true>), dim3((unsigned)wgs), dim3(kThreads), 0, stream, a);
+    else hipLaunchKernelGGL((merge_states_kernel<64, false>), dim3((unsigned)wgs), dim3(kThreads), 0, stream, a);
   } else {
     set_error("head dim %d not built (64 and 128 are)", D);
     return DT_ERR_UNSUPPORTED;
@@ -263,7 +399,8 @@ int launch_merge(const MergeArgs& a, int D, hipStream_t stream) {
 }
 
 int launch_copy(const CopyArgs& a, int D, hipStream_t stream) {
-  const int n_st = (a.Sq + kQPerWg - 1) / kQPerWg;
+  const int rows_per_wg = kThreads / (D / 8) * kCopyRows;
+  const int n_st = (a.Sq + rows_per_wg - 1) / rows_per_wg;
   const int64_t wgs = (int64_t)a.B * a.H * n_st;
   if (wgs <= 0) return DT_OK;
   if (wgs > 0x7fffffffLL) {
