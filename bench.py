@@ -118,6 +118,8 @@ def main():
     ap.add_argument("--reuse", type=float, default=None, help="override the mask's reuse probability")
     ap.add_argument("--kernel-reps", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--kernels-only", action="store_true",
+                    help="run only the per-kernel roofline launches (short; for rocprofv3 counter passes)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one sequence-parallel rank's share on ONE GPU; --gpus > 1 is not part of this build",
@@ -171,6 +173,9 @@ def main():
         update_timestep(t)
         return layers[l].attn(q, ks[rank], vs[rank])
 
+    if args.kernels_only:
+        args.warmup, args.steps = 0, 1
+        seq = seq[:1]
     for t, l in seq[:args.warmup]:
         run(t, l)
     torch.cuda.synchronize()
@@ -191,9 +196,19 @@ def main():
     reps = args.kernel_reps
     out_s = torch.empty(B, Sq, H, D, dtype=torch.bfloat16, device=dev)
     lse_s = torch.empty(B, H, Sq, dtype=torch.float32, device=dev)
-    k1_ms = time_kernel(lambda: _hip.attn_chunk_fwd(q, ks[0], vs[0], out=out_s, lse=lse_s), reps)
-    k1_flops = 4.0 * B * H * Sq * lens[0] * D
+    # the dominant kernel in its typical launch: as many single-chunk states as a layer call
+    # computes on average (rounded), written into cache slots, one launch
+    n_typ = max(1, min(C, int(round(mean_computed))))
+    table = _hip.ChunkTable(ks, vs)
+    typ_jobs = [[c] for c in range(n_typ)]
+    typ_outs = [torch.empty_like(out_s) for _ in range(n_typ)]
+    typ_lses = [torch.empty_like(lse_s) for _ in range(n_typ)]
+    k1_ms = time_kernel(lambda: _hip.attn_jobs_fwd(q, table, typ_jobs, typ_outs, typ_lses), reps)
+    k1_flops = sum(4.0 * B * H * Sq * lens[c] * D for c in range(n_typ))
     k1_tflops = k1_flops / (k1_ms * 1e-3) / 1e12
+    k1s_ms = time_kernel(lambda: _hip.attn_chunk_fwd(q, ks[0], vs[0], out=out_s, lse=lse_s), reps)
+    k1s_tflops = 4.0 * B * H * Sq * lens[0] * D / (k1s_ms * 1e-3) / 1e12
+    del typ_outs, typ_lses
 
     cache0 = layers[0].cache
     m_outs = [cache0.arena_out[c] if c != diag else cache0.diag_out for c in range(C)]
@@ -214,6 +229,20 @@ def main():
 
     dmask = torch.from_numpy(mask).to(dev)
     k4_ms = time_kernel(lambda: _hip.build_schedule_table(dmask, diag), reps)
+    # a plain copy of known size: the yardstick the profiler's FETCH_SIZE / WRITE_SIZE counters are scaled by
+    ref_src = torch.empty(1 << 28, dtype=torch.float32, device=dev)   # 1 GiB
+    ref_dst = torch.empty_like(ref_src)
+    copy_ms = time_kernel(lambda: ref_dst.copy_(ref_src), max(3, reps // 4))
+    copy_gbs = 2 * ref_src.numel() * 4 / (copy_ms * 1e-3) / 1e9
+    del ref_src, ref_dst
+
+    # HBM bytes per launch measured offline with rocprofv3 counters (FETCH_SIZE + WRITE_SIZE),
+    # committed as text under profiles/; only meaningful for the default workload
+    traffic = {}
+    tpath = os.path.join(ROOT, "profiles", "hbm_traffic_hunyuanvideo.json")
+    if args.workload == "hunyuanvideo" and args.reuse is None and os.path.exists(tpath):
+        with open(tpath) as f:
+            traffic = json.load(f).get("bytes_per_launch", {})
 
     result = {
         "metric": "ms/layer", "value": round(ms_per_step, 4), "unit": "ms", "n_gpus": 1,
@@ -225,17 +254,20 @@ def main():
         "layer_attn_tflops": round(flops_per_chunk * mean_computed / (ms_per_step * 1e-3) / 1e12, 1),
         "roofline": {"kernel": "attn_fwd_kernel<%d>" % D, "bound": "mfma", "achieved": round(k1_tflops, 1),
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(k1_tflops / PEAK_BF16_TFLOPS, 4),
-                     "traffic": None, "launch_ms": round(k1_ms, 4), "flop_per_launch": k1_flops},
+                     "traffic": traffic.get("attn_fwd"), "launch_ms": round(k1_ms, 4), "flop_per_launch": k1_flops,
+                     "chunks_per_launch": n_typ, "single_chunk_launch_tflops": round(k1s_tflops, 1),
+                     "single_chunk_launch_ms": round(k1s_ms, 4)},
         "roofline_merge": {"kernel": "merge_states_kernel<%d>" % D, "bound": "hbm", "achieved": round(k2_gbs, 1),
                            "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(k2_gbs / PEAK_HBM_GBS, 4),
-                           "traffic": None, "launch_us": round(k2_ms * 1e3, 2), "bytes_per_launch": k2_bytes,
+                           "traffic": traffic.get("merge_states"), "launch_us": round(k2_ms * 1e3, 2), "bytes_per_launch": k2_bytes,
                            "states": C},
         "cache_gbs": {"store_fp32_to_slot": round(k3s_gbs, 1), "store_bf16_to_slot": round(k3c_gbs, 1),
                       "load_slot_to_fp32": round(k3l_gbs, 1), "peak": PEAK_HBM_GBS,
                       "frac_store_bf16": round(k3c_gbs / PEAK_HBM_GBS, 4), "frac_load": round(k3l_gbs / PEAK_HBM_GBS, 4)},
         "schedule_builder_us": round(k4_ms * 1e3, 2),
+        "plain_copy_1GiB_gbs": round(copy_gbs, 1),
     }
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and not args.kernels_only:
         result["cpu_baseline"] = cpu_baseline(B, H, D, Sq, lens, mean_computed, C, norm)
     print(json.dumps(result), flush=True)
 
