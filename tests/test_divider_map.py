@@ -20,15 +20,15 @@ MODELS = {
     "stepvideo": ("redundancy_map_50_48.pt", 48, [0, 0, 90], [8, 4, 2, 1]),
 }
 # Divider histograms and double-count tallies that an independent restatement of the same
-# reference functions produced for N=8 (survey of the reference); agreement of two
+# reference functions, written earlier and separately from this oracle, produced for N=8; agreement of two
 # independent restatements, not reference output.
-SURVEY_HIST = {
+INDEPENDENT_HIST = {
     "cogvideox-5b": {1: 381, 2: 946, 4: 773},
     "hunyuanvideo": {1: 560, 2: 1379, 4: 1061},
     "stepvideo": {1: 472, 2: 1928},
 }
-SURVEY_DOUBLE_COUNT = {"cogvideox-5b": 280, "hunyuanvideo": 356, "stepvideo": 0}
-SURVEY_MEAN_COMPUTED = {"cogvideox-5b": 4.49, "hunyuanvideo": 4.53, "stepvideo": 5.18}
+INDEPENDENT_DOUBLE_COUNT = {"cogvideox-5b": 280, "hunyuanvideo": 356, "stepvideo": 0}
+INDEPENDENT_MEAN_COMPUTED = {"cogvideox-5b": 4.49, "hunyuanvideo": 4.53, "stepvideo": 5.18}
 
 
 def _load(name):
@@ -64,7 +64,7 @@ def test_generated_map_rules_and_histogram(name):
     top = np.mean(body == dv[3])
     assert abs(top - (100 - pct[2]) / 100) < 0.01
     refined, changes = od.refine_divider_map(div)
-    assert dict(Counter(int(x) for x in refined.ravel())) == SURVEY_HIST[name]
+    assert dict(Counter(int(x) for x in refined.ravel())) == INDEPENDENT_HIST[name]
     # refined map: legal transitions in every layer, first three and last two steps full
     for l in range(L):
         assert legal_divider_column(refined[:, l])
@@ -95,8 +95,8 @@ def test_schedule_statistics_agree_with_independent_restatement(name):
                 computed += len(tr.computed)
                 calls += 1
     assert calls == N * L * T
-    assert double == SURVEY_DOUBLE_COUNT[name]
-    assert abs(computed / calls - SURVEY_MEAN_COMPUTED[name]) < 0.006
+    assert double == INDEPENDENT_DOUBLE_COUNT[name]
+    assert abs(computed / calls - INDEPENDENT_MEAN_COMPUTED[name]) < 0.006
 
 
 @pytest.mark.parametrize("name", list(MODELS))
