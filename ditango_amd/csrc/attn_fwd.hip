@@ -38,6 +38,8 @@
 //   * Workgroups are mapped to (head, query tile) so that the 8 XCDs each work
 //     through a contiguous range of heads: the workgroups that share an XCD's
 //     L2 stream the same K/V.
+#include <type_traits>
+
 #include "dt_common.h"
 
 namespace dt {
@@ -260,8 +262,11 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
 #pragma unroll
   for (int r = 0; r < 4; ++r) voff[r] = (uint32_t)(4 * vkg + r) * row_bytes + (uint32_t)(T::kDV * 2 * vdg);
 
-  u32x4 kreg[T::kLoadsK];
-  VLoad vreg[4];
+  // Two register sets: the loads of a tile are issued TWO iterations before its LDS fill, so
+  // that a first-touch miss all the way to HBM (the workgroup that leads on its XCD takes one
+  // on every tile) is still hidden.  Tile X of a group uses set (X - pf) & 1.
+  u32x4 kreg[2][T::kLoadsK];
+  VLoad vreg[2][4];
 
   const int64_t tile_bytes = (int64_t)kBK * row_bytes;
   // Loads this thread's share of the tile under the load cursor into registers and moves the
@@ -269,16 +274,17 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   // and head, number of valid bytes) lives in scalar registers, and rows past the end of the
   // chunk fail the hardware bounds check and come back as zeros (their scores are masked to
   // -inf; zero V rows add nothing).
-  auto load_tile = [&]() {
+  auto load_tile = [&](auto set_tag) {
+    constexpr int kSet = decltype(set_tag)::value;
     const uint32_t valid = (uint32_t)(ld_left - 1) * row_bytes + (uint32_t)(D * 2);
     const __amdgpu_buffer_rsrc_t rk =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(ld_k), 0, (int)valid, kRsrcFlags);
     const __amdgpu_buffer_rsrc_t rv =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(ld_v), 0, (int)valid, kRsrcFlags);
 #pragma unroll
-    for (int i = 0; i < T::kLoadsK; ++i) kreg[i] = __builtin_amdgcn_raw_buffer_load_b128(rk, (int)koff[i], 0, 0);
+    for (int i = 0; i < T::kLoadsK; ++i) kreg[kSet][i] = __builtin_amdgcn_raw_buffer_load_b128(rk, (int)koff[i], 0, 0);
 #pragma unroll
-    for (int r = 0; r < 4; ++r) vreg[r] = buffer_load_v<T::kVW>(rv, (int)voff[r]);
+    for (int r = 0; r < 4; ++r) vreg[kSet][r] = buffer_load_v<T::kVW>(rv, (int)voff[r]);
     ld_left -= kBK;
     ld_k += tile_bytes;
     ld_v += tile_bytes;
@@ -288,20 +294,21 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   // LDS write addresses of this thread within a K / V buffer
   const int kst = kr0 * T::kPitchK + 16 * kc;
   const int vst = (T::kDV * vdg) * T::kPitchV + 8 * vkg;
-  auto store_tile = [&](int tile) {
+  auto store_tile = [&](int tile, auto set_tag) {
+    constexpr int kSet = decltype(set_tag)::value;
     uint8_t* kbuf = lds + (tile % kNumKBuf) * T::kBytesK;
     uint8_t* vbuf = lds + T::kOffV + (tile % kNumVBuf) * T::kBytesV;
 #pragma unroll
     for (int i = 0; i < T::kLoadsK; ++i)
-      *reinterpret_cast<u32x4*>(kbuf + kst + i * T::kRowStepK * T::kPitchK) = kreg[i];
+      *reinterpret_cast<u32x4*>(kbuf + kst + i * T::kRowStepK * T::kPitchK) = kreg[kSet][i];
     // transpose 4 keys x kDV d -> kDV rows of 4 keys
 #pragma unroll
     for (int jj = 0; jj < T::kDV; ++jj) {
       const int w = jj >> 1;
       const uint32_t sel = (jj & 1) ? 0x07060302u : 0x05040100u;
       u32x2 o;
-      o.x = __builtin_amdgcn_perm(dword_of(vreg[1], w), dword_of(vreg[0], w), sel);
-      o.y = __builtin_amdgcn_perm(dword_of(vreg[3], w), dword_of(vreg[2], w), sel);
+      o.x = __builtin_amdgcn_perm(dword_of(vreg[kSet][1], w), dword_of(vreg[kSet][0], w), sel);
+      o.y = __builtin_amdgcn_perm(dword_of(vreg[kSet][3], w), dword_of(vreg[kSet][2], w), sel);
       *reinterpret_cast<u32x2*>(vbuf + vst + jj * T::kPitchV) = o;
     }
   };
@@ -346,7 +353,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   constexpr int kPV = D / 32 * 4;       // fragments of the P V product
   constexpr int kQK = 2 * (D / 16);     // fragments of the score product
   constexpr int kFrags = kPV + kQK;
-  constexpr int kRing = 8;
+  constexpr int kRing = 4;
   auto matrix_phase = [&](int tile) {
     const uint8_t* vl = lds + vld + (tile % kNumVBuf) * T::kBytesV;
     const uint8_t* kl = lds + kld + ((tile + 1) % kNumKBuf) * T::kBytesK;
@@ -394,25 +401,37 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
 
   // ---- prologue: tile 0 from everybody; the trailing group also brings its share of tile 1
   //      and then waits one phase, which is what staggers the two groups ---------------------
-  const int pf = 1 + group;  // how many tiles ahead of its softmax a group stores
+  using Set0 = std::integral_constant<int, 0>;
+  using Set1 = std::integral_constant<int, 1>;
+  const int pf = 1 + group;  // how many tiles ahead of its softmax a group fills LDS
+  int n_issued = 0;          // tiles whose loads this thread has issued
   int n_loaded = 0;          // tiles this thread has written its share of
   if (n_tiles > 0) {
-    load_tile();
-    store_tile(0);
-    n_loaded = 1;
+    load_tile(Set0{});
+    store_tile(0, Set0{});
+    n_issued = n_loaded = 1;
   }
-  if (group == 1 && n_tiles > 1) load_tile();
+  if (group == 1 && n_tiles > 1) {
+    load_tile(Set0{});
+    n_issued = 2;
+  }
   phase_barrier();
   if (group == 1) {
     if (n_tiles > 1) {
-      store_tile(1);
+      store_tile(1, Set0{});
       n_loaded = 2;
     }
     phase_barrier();
   }
-  // first matrix phase: fetch ahead, scores of tile 0
-  bool fetched = (n_loaded < n_tiles);
-  if (fetched) load_tile();
+  // first matrix phase: fetch two tiles ahead (sets 0 and 1), scores of tile 0
+  if (n_issued < n_tiles) {
+    load_tile(Set0{});
+    ++n_issued;
+  }
+  if (n_issued < n_tiles) {
+    load_tile(Set1{});
+    ++n_issued;
+  }
   if (n_tiles > 0) {
     qk_only(0);
     cp_valid = cp_left;
@@ -421,8 +440,16 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   }
   phase_barrier_after_matrix(s_acc, o_acc);
 
-  for (int t = 0; t < n_tiles; ++t) {
-    // ======== vector phase: online softmax of tile t, LDS fill of the fetched tile ========
+  // one iteration = vector phase of tile t, then matrix phase (P V of tile t, scores of t+1);
+  // iteration t fills LDS from register set t & 1 and then refills that set from memory
+  auto iteration = [&](int t, auto set_tag) {
+    // ======== vector phase: LDS fill of a fetched tile, online softmax of tile t ========
+    // The fill goes first: its registers were loaded two iterations ago, and the latency of
+    // the LDS writes (which compete with the other group's operand reads) hides behind the softmax.
+    if (n_loaded < n_issued) {
+      store_tile(n_loaded, set_tag);
+      ++n_loaded;
+    }
     if (cp_valid < kBK) {
       // the empty asm has side effects as far as the compiler knows, which keeps this a real
       // branch: otherwise the selects below are hoisted out and run for every tile
@@ -474,20 +501,22 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
         p_frag[kb][r >> 3][(r & 7) + 1] = pb.y;
       }
     l_run += rs0 + rs1;
-    if (fetched) {
-      store_tile(n_loaded);
-      ++n_loaded;
-    }
     phase_barrier_after_vector(p_frag);
 
     // ======== matrix phase: fetch ahead, O^T += V^T P^T (tile t), S^T = K Q^T (tile t+1) ========
-    fetched = (n_loaded < n_tiles);
-    if (fetched) load_tile();
+    if (n_issued < n_tiles) {
+      load_tile(set_tag);
+      ++n_issued;
+    }
     matrix_phase(t);
     cp_valid = cp_left;
     cp_left -= kBK;
     if (cp_left <= 0) cp_next_chunk();
     phase_barrier_after_matrix(s_acc, o_acc);
+  };
+  for (int t = 0; t < n_tiles; t += 2) {
+    iteration(t, Set0{});
+    if (t + 1 < n_tiles) iteration(t + 1, Set1{});
   }
   // the leading group waits out the phase it is ahead
   if (group == 0) phase_barrier();
