@@ -59,6 +59,12 @@ constexpr int kBK = 64;           // keys per tile
 constexpr int kXcds = 8;
 constexpr int kNumKBuf = 2;
 constexpr int kNumVBuf = 3;
+// true: two groups of 4 wavefronts run one phase apart with a barrier after every phase;
+// false: all wavefronts in the same phase, one barrier per tile.
+#ifndef DT_STAGGER
+#define DT_STAGGER 1
+#endif
+constexpr bool kStagger = DT_STAGGER;
 
 template <int N> struct VecOf;
 template <> struct VecOf<4> { typedef u32x4 type; };
@@ -114,7 +120,15 @@ __device__ __forceinline__ void phase_barrier_after_vector(V (&p)[2][2]) {
 template <typename V, int NO>
 __device__ __forceinline__ void phase_barrier_after_matrix(V (&sa)[2], V (&oa)[NO]) {
   __builtin_amdgcn_sched_barrier(0);
-  if constexpr (NO == 4) {
+  if constexpr (!kStagger) {
+    // no barrier between a wavefront's matrix phase and its next vector phase: the buffers the
+    // next fill overwrites were last read one iteration earlier
+    if constexpr (NO == 4) {
+      asm volatile("" : "+v"(sa[0]), "+v"(sa[1]), "+v"(oa[0]), "+v"(oa[1]), "+v"(oa[2]), "+v"(oa[3]));
+    } else {
+      asm volatile("" : "+v"(sa[0]), "+v"(sa[1]), "+v"(oa[0]), "+v"(oa[1]));
+    }
+  } else if constexpr (NO == 4) {
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier"
                  : "+v"(sa[0]), "+v"(sa[1]), "+v"(oa[0]), "+v"(oa[1]), "+v"(oa[2]), "+v"(oa[3])
                  :
@@ -198,7 +212,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: keeps group/buffer arithmetic scalar
-  const int group = wave >> 2;  // 0: leads, 1: runs one phase behind
+  const int group = kStagger ? (wave >> 2) : 0;  // 0: leads, 1: runs one phase behind
   const int col = lane & 31;    // query column (B operand) / operand row (A operand)
   const int hh = lane >> 5;     // which half of the contraction dimension this lane feeds
   const int q0 = qt * kBQ + wave * 32;
@@ -519,7 +533,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     if (t + 1 < n_tiles) iteration(t + 1, Set1{});
   }
   // the leading group waits out the phase it is ahead
-  if (group == 0) phase_barrier();
+  if (kStagger && group == 0) phase_barrier();
 
   // ---- epilogue -------------------------------------------------------------------------
   const float l_tot = l_run + __shfl_xor(l_run, 32);
