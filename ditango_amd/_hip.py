@@ -9,7 +9,7 @@ from __future__ import annotations
 import ctypes
 import os
 from pathlib import Path
-from typing import List, Optional, Sequence
+from typing import List, Optional, Sequence, Tuple
 
 import torch
 
@@ -33,6 +33,10 @@ _SIGNATURES = {
     "dt_attn_jobs_fwd": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i64, c_i64, c_i64,
                                         c_i32, _P(c_vp), _P(c_vp), _P(c_i32), _P(c_i64), c_i64, c_i64,
                                         c_i32, _P(c_i32), _P(c_i32), _P(c_vp), _P(c_vp), c_f32, c_vp]),
+    "dt_attn_seg_jobs_fwd": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i64, c_i64, c_i64,
+                                            c_i32, _P(c_vp), _P(c_vp), _P(c_i32), _P(c_i64), c_i64, c_i64,
+                                            c_i32, _P(c_i32), _P(c_i32), _P(c_i32), _P(c_i32), _P(c_i32), _P(c_i32),
+                                            _P(c_vp), _P(c_vp), c_f32, c_vp]),
     "dt_attn_sched_fwd": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i64, c_i64, c_i64,
                                          c_i32, _P(c_vp), _P(c_vp), _P(c_i32), _P(c_i64), c_i64, c_i64,
                                          c_vp, c_vp, c_i32, c_vp, c_i64, c_vp, c_i64, c_i32, c_vp, c_vp,
@@ -178,36 +182,65 @@ class ChunkTable:
 
 
 def attn_jobs_fwd(q: torch.Tensor, table: ChunkTable, jobs: Sequence[Sequence[int]],
-                  outs: Sequence[torch.Tensor], lses: Sequence[torch.Tensor], softmax_scale: float = 0.0) -> None:
-    """One launch; job j attends q to the concatenation of chunks ``jobs[j]`` and writes (outs[j], lses[j])."""
+                  outs: Sequence[torch.Tensor], lses: Sequence[torch.Tensor], softmax_scale: float = 0.0,
+                  q_ranges: Optional[Sequence[Tuple[int, int]]] = None,
+                  kv_ranges: Optional[Sequence[Sequence[Tuple[int, int]]]] = None) -> None:
+    """One launch; job j attends q to the concatenation of chunks ``jobs[j]`` and writes (outs[j], lses[j]).
+
+    ``q_ranges[j] = (begin, length)`` restricts job j to those query rows (the rest of its
+    destination is left untouched); ``kv_ranges[j][i] = (begin, length)`` restricts the i-th chunk
+    of job j to those keys.  Several jobs may share one destination if their rows are disjoint
+    (the segments of a packed variable-length batch).  Launches are split to respect the limits
+    of one launch."""
     lib = load_library()
     _check_qkv(q, "q")
     B, Sq, H, D = q.shape
     _require((B, H, D) == (table.B, table.H, table.D), "q and KV chunks disagree on B/H/D")
     nj = len(jobs)
-    _require(nj == len(outs) == len(lses) and nj <= DT_MAX_JOBS, f"need at most {DT_MAX_JOBS} jobs with one destination each")
-    if nj == 0:
-        return
-    begin = (c_i32 * (nj + 1))()
-    flat: List[int] = []
-    for j, ids in enumerate(jobs):
-        begin[j] = len(flat)
-        flat.extend(int(c) for c in ids)
-    begin[nj] = len(flat)
-    _require(len(flat) <= DT_MAX_JOB_ENTRIES, f"more than {DT_MAX_JOB_ENTRIES} chunk references in one launch")
-    chunks = (c_i32 * max(1, len(flat)))(*flat)
-    out_ptrs = (c_vp * nj)()
-    lse_ptrs = (c_vp * nj)()
+    _require(nj == len(outs) == len(lses), "one destination per job")
+    _require(q_ranges is None or len(q_ranges) == nj, "one query range per job")
+    _require(kv_ranges is None or len(kv_ranges) == nj, "one list of key ranges per job")
     for j in range(nj):
         o, l = outs[j], lses[j]
         _require(o.dtype == torch.bfloat16 and o.is_contiguous() and tuple(o.shape) == (B, Sq, H, D), f"outs[{j}] must be contiguous bf16 [B,Sq,H,D]")
         _require(l.dtype == torch.float32 and l.is_contiguous() and tuple(l.shape) == (B, H, Sq), f"lses[{j}] must be contiguous fp32 [B,H,Sq]")
-        out_ptrs[j] = o.data_ptr()
-        lse_ptrs[j] = l.data_ptr()
-    rc = lib.dt_attn_jobs_fwd(q.data_ptr(), B, Sq, H, D, q.stride(0), q.stride(1), q.stride(2),
-                              table.n, table.k_ptrs, table.v_ptrs, table.lens, table.sb, table.ss, table.sh,
-                              nj, begin, chunks, out_ptrs, lse_ptrs, float(softmax_scale), _stream())
-    _check(rc, "dt_attn_jobs_fwd")
+        _require(len(jobs[j]) <= DT_MAX_JOB_ENTRIES, f"job {j} references more than {DT_MAX_JOB_ENTRIES} chunks")
+    # split into launches that fit the per-launch limits
+    start = 0
+    while start < nj:
+        end, entries = start, 0
+        while end < nj and end - start < DT_MAX_JOBS and entries + len(jobs[end]) <= DT_MAX_JOB_ENTRIES:
+            entries += len(jobs[end])
+            end += 1
+        n = end - start
+        begin = (c_i32 * (n + 1))()
+        flat: List[int] = []
+        kvb: List[int] = []
+        kvl: List[int] = []
+        for jj in range(n):
+            j = start + jj
+            begin[jj] = len(flat)
+            for i, c in enumerate(jobs[j]):
+                c = int(c)
+                flat.append(c)
+                if kv_ranges is not None:
+                    kvb.append(int(kv_ranges[j][i][0]))
+                    kvl.append(int(kv_ranges[j][i][1]))
+        begin[n] = len(flat)
+        m = max(1, len(flat))
+        chunks = (c_i32 * m)(*flat)
+        a_kvb = (c_i32 * m)(*kvb) if kv_ranges is not None else None
+        a_kvl = (c_i32 * m)(*kvl) if kv_ranges is not None else None
+        a_qb = (c_i32 * n)(*[int(q_ranges[start + jj][0]) for jj in range(n)]) if q_ranges is not None else None
+        a_ql = (c_i32 * n)(*[int(q_ranges[start + jj][1]) for jj in range(n)]) if q_ranges is not None else None
+        out_ptrs = (c_vp * n)(*[outs[start + jj].data_ptr() for jj in range(n)])
+        lse_ptrs = (c_vp * n)(*[lses[start + jj].data_ptr() for jj in range(n)])
+        rc = lib.dt_attn_seg_jobs_fwd(q.data_ptr(), B, Sq, H, D, q.stride(0), q.stride(1), q.stride(2),
+                                      table.n, table.k_ptrs, table.v_ptrs, table.lens, table.sb, table.ss, table.sh,
+                                      n, begin, chunks, a_kvb, a_kvl, a_qb, a_ql, out_ptrs, lse_ptrs,
+                                      float(softmax_scale), _stream())
+        _check(rc, "dt_attn_seg_jobs_fwd")
+        start = end
 
 
 def attn_sched_fwd(q: torch.Tensor, table: ChunkTable, dev_compute_ids: torch.Tensor, dev_count: torch.Tensor,

@@ -169,6 +169,7 @@ class proAttention:
         self.dry_run = dry_run  # plan and book-keep only (host tests of the schedule); computes nothing
         self.last_plan: Optional[CallPlan] = None
         self.last_lse: Optional[torch.Tensor] = None  # merged lse of the last call, fp32 [B,S,H,1]
+        self._segments = None  # (cu_seqlens_q, chunk -> cu_seqlens_kv) while a variable-length call runs
         if self.layer_id == 0:
             logger.info(f"R{self.global_rank}L{layer_id} | cached block attention on HIP kernels (gfx950)")
 
@@ -214,7 +215,7 @@ class proAttention:
                     self.cache.out_block_cache[job.store_slot] = job.chunks
                     self.cache.lse_block_cache[job.store_slot] = job.chunks
         else:
-            out = self._execute(plan, query, key, value, merge_outs, merge_lses)
+            out = self._execute(plan, query, key, value, merge_outs, merge_lses, self._segments)
 
         # 4./5. pointer and cache management (:214, :219-220)
         self.target_chunk_id = new_target
@@ -252,7 +253,7 @@ class proAttention:
         else:
             cache.update_cache_blocks(nxt, next_target_block)
 
-    def _execute(self, plan: CallPlan, query, key, value, merge_outs, merge_lses) -> torch.Tensor:
+    def _execute(self, plan: CallPlan, query, key, value, merge_outs, merge_lses, segments=None) -> torch.Tensor:
         B, Sq, H, D = query.shape
         N, r = self.isp_size, self.local_chunk_id
         dev = query.device
@@ -269,6 +270,7 @@ class proAttention:
         # one launch for all distinct states; a chunk computed twice by the reference
         # (local + own) is computed once and merged twice
         job_lists, dests, seen = [], [], {}
+        q_ranges, kv_ranges = ([], []) if segments is not None else (None, None)
         states = []
         for job in plan.jobs:
             if job.chunks in seen and job.store_slot is None:
@@ -276,13 +278,23 @@ class proAttention:
                 continue
             o = torch.empty((B, Sq, H, D), dtype=torch.bfloat16, device=dev)
             l = torch.empty((B, H, Sq), dtype=torch.float32, device=dev)
-            job_lists.append([index[c] for c in job.chunks])
-            dests.append((o, l))
+            if segments is None:
+                job_lists.append([index[c] for c in job.chunks])
+                dests.append((o, l))
+            else:
+                # one kernel job per segment: its query rows against its key rows of every chunk
+                cu_q, cu_kv_of = segments
+                for i in range(len(cu_q) - 1):
+                    job_lists.append([index[c] for c in job.chunks])
+                    dests.append((o, l))
+                    q_ranges.append((cu_q[i], cu_q[i + 1] - cu_q[i]))
+                    kv_ranges.append([(cu_kv_of(c)[i], cu_kv_of(c)[i + 1] - cu_kv_of(c)[i]) for c in job.chunks])
             seen[job.chunks] = (o, l)
             states.append((o, l))
         if job_lists:
             table = _hip.ChunkTable(ks, vs)
-            _hip.attn_jobs_fwd(query, table, job_lists, [d[0] for d in dests], [d[1] for d in dests])
+            _hip.attn_jobs_fwd(query, table, job_lists, [d[0] for d in dests], [d[1] for d in dests],
+                               q_ranges=q_ranges, kv_ranges=kv_ranges)
         for job, (o, l) in zip(plan.jobs, states):
             if job.store_slot is not None:
                 self.cache.store_block(job.store_slot, o, l)  # :207-211
@@ -334,24 +346,36 @@ class proAttention:
     @get_timer("varlen oAttn")
     def varlen_attn(self, query, key, value, cu_seqlens_q=None, cu_seqlens_kv=None, max_seqlen_q=None,
                     max_seqlen_kv=None, batch_size=1):
-        """core/attention.py:239-419.  Without sequence lengths it is ``attn`` (:252-254).
-        With them, inputs are ``[B*S, H, D]``; the single-segment-per-sample case (every
-        sample one full-length segment) is the dense path on a reshaped view.  Several
-        segments per sample are not built yet and raise."""
+        """core/attention.py:239-419: the same state machine on a packed batch.
+
+        ``query/key/value`` are ``[total, H, D]``; segment ``i`` of the queries
+        (rows ``cu_seqlens_q[i]:cu_seqlens_q[i+1]``) attends to segment ``i`` of every KV chunk,
+        whose boundaries ``cu_seqlens_kv`` belong to the chunk (the local chunk's are the argument,
+        the others come with the chunks: ``LocalRingGroup.set_kv_chunks(..., cu_seqlens_kv=...)``).
+        Returns fp32 ``[total, H, D]``.  Without sequence lengths it is ``attn`` (:252-254).
+        Each segment runs as attention jobs on row/key sub-ranges of one launch
+        (``dt_attn_seg_jobs_fwd``); schedule, cache and merge are those of ``attn``."""
         if cu_seqlens_q is None and cu_seqlens_kv is None and max_seqlen_q is None and max_seqlen_kv is None:
             logger.warning("cu_seqlens_q not provided, using normal attention instead.")
             return self.attn(query, key, value)
+        rm = get_redundancy_map()
+        if rm is not None and rm.chunk_mask is not None:
+            raise NotImplementedError("the per-chunk mask mode takes dense [B,S,H,D] inputs")
         total_q, H, D = query.shape
-        total_k = key.shape[0]
-        cq = [int(x) for x in cu_seqlens_q.tolist()]
-        ck = [int(x) for x in cu_seqlens_kv.tolist()]
-        nb = len(cq) - 1
-        uniform = (len(ck) == len(cq) and total_q % nb == 0 and total_k % nb == 0
-                   and cq == [i * (total_q // nb) for i in range(nb + 1)]
-                   and ck == [i * (total_k // nb) for i in range(nb + 1)])
-        if not uniform:
-            raise NotImplementedError("varlen_attn with several (or ragged) segments per sample is not built yet; "
-                                      "only one full-length segment per sample is")
-        out = self.attn(query.view(nb, total_q // nb, H, D), key.view(nb, total_k // nb, H, D),
-                        value.view(nb, total_k // nb, H, D))
+        cu_q = [int(x) for x in (cu_seqlens_q.tolist() if hasattr(cu_seqlens_q, "tolist") else cu_seqlens_q)]
+        local_cu = [int(x) for x in (cu_seqlens_kv.tolist() if hasattr(cu_seqlens_kv, "tolist") else cu_seqlens_kv)]
+        assert cu_q[0] == 0 and cu_q[-1] <= total_q and len(local_cu) == len(cu_q), "malformed cu_seqlens"
+        r = self.local_chunk_id
+
+        def cu_kv_of(c):
+            return local_cu if c == r else self.group.kv_cu_seqlens(c)
+
+        self._segments = (cu_q, cu_kv_of)
+        try:
+            out = self.attn(query.view(1, total_q, H, D), key.view(1, key.shape[0], H, D),
+                            value.view(1, value.shape[0], H, D))
+        finally:
+            self._segments = None
+        if cu_q[-1] < total_q:
+            out[:, cu_q[-1]:] = 0  # rows outside every segment: flash_attn_varlen_func leaves zeros
         return out.view(total_q, H, D)

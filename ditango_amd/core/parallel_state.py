@@ -23,14 +23,30 @@ class LocalRingGroup:
         self.name = name
         self._k: List[Optional[torch.Tensor]] = [None] * world_size
         self._v: List[Optional[torch.Tensor]] = [None] * world_size
+        self._cu: List[Optional[Sequence[int]]] = [None] * world_size
 
-    def set_kv_chunks(self, k_chunks: Sequence[torch.Tensor], v_chunks: Sequence[torch.Tensor]) -> None:
-        """K/V of every ring position for the coming attention call ([B,Sk_c,H,D] each).
-        The entry at ``rank_in_group`` may be None: the local chunk is the (key, value)
-        passed to ``attn`` itself."""
+    def set_kv_chunks(self, k_chunks: Sequence[torch.Tensor], v_chunks: Sequence[torch.Tensor],
+                      cu_seqlens_kv: Optional[Sequence] = None) -> None:
+        """K/V of every ring position for the coming attention call ([B,Sk_c,H,D] each, or packed
+        [total_c,H,D] for the variable-length entry).  The entry at ``rank_in_group`` may be
+        None: the local chunk is the (key, value) passed to ``attn`` itself.
+        ``cu_seqlens_kv[c]`` are the segment boundaries of chunk ``c`` (they travel with K/V on
+        the reference's ring, core/attention.py:307-311)."""
         assert len(k_chunks) == self.world_size and len(v_chunks) == self.world_size
         self._k = list(k_chunks)
         self._v = list(v_chunks)
+        if cu_seqlens_kv is not None:
+            assert len(cu_seqlens_kv) == self.world_size
+            self._cu = [None if c is None else [int(x) for x in (c.tolist() if hasattr(c, "tolist") else c)]
+                        for c in cu_seqlens_kv]
+        else:
+            self._cu = [None] * self.world_size
+
+    def kv_cu_seqlens(self, chunk_id: int) -> Sequence[int]:
+        cu = self._cu[chunk_id]
+        if cu is None:
+            raise RuntimeError(f"segment boundaries of KV chunk {chunk_id} were not provided (set_kv_chunks)")
+        return cu
 
     def kv_chunk(self, chunk_id: int) -> Tuple[torch.Tensor, torch.Tensor]:
         k, v = self._k[chunk_id], self._v[chunk_id]

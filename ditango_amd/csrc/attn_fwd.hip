@@ -33,7 +33,8 @@
 //     8 consecutive keys of one d-row of the transposed V tile.
 //   * O^T stays in registers as [d][query]: a rescale is a multiply by a per-lane
 //     scalar, and it is only done when some query's running maximum grew by more
-//     than 2^8 (the reference maximum may lag; the lse stays exact).  The epilogue
+//     than 2^8 (the reference maximum may lag; the lse stays exact).  Row sums are
+//     accumulated in fp32 from the unrounded probabilities.  The epilogue
 //     transposes through LDS so that the global stores are 16 bytes per lane.
 //   * Workgroups are mapped to (head, query tile) so that the 8 XCDs each work
 //     through a contiguous range of heads: the workgroups that share an XCD's
@@ -186,6 +187,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   const int h = bh - b * a.H;
 
   int seg_begin, seg_end, single = -1;
+  int q_begin = 0, q_end = a.Sq;   // query rows of this job
   __bf16* out_ptr;
   float* lse_ptr;
   if (a.dev_ids != nullptr) {
@@ -206,8 +208,13 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     seg_end = a.job_begin[job + 1];
     out_ptr = a.job_out[job];
     lse_ptr = a.job_lse[job];
+    q_begin = a.job_q_begin[job];
+    q_end = q_begin + a.job_q_len[job];
+    if (qt * kBQ >= q_end - q_begin) return;  // the grid is sized for the longest job
   }
   auto chunk_of = [&](int seg) -> int { return single >= 0 ? single : a.job_chunks[seg]; };
+  auto kv_begin_of = [&](int seg) -> int { return single >= 0 ? 0 : a.entry_kv_begin[seg]; };
+  auto kv_len_of = [&](int seg) -> int { return single >= 0 ? a.kv_len[single] : a.entry_kv_len[seg]; };
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -215,13 +222,13 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   const int group = kStagger ? (wave >> 2) : 0;  // 0: leads, 1: runs one phase behind
   const int col = lane & 31;    // query column (B operand) / operand row (A operand)
   const int hh = lane >> 5;     // which half of the contraction dimension this lane feeds
-  const int q0 = qt * kBQ + wave * 32;
+  const int q0 = q_begin + qt * kBQ + wave * 32;
 
   // ---- Q fragments: B operand of S^T = K Q^T, kept in registers ----------------------
   bf16x8 qf[D / 16];
   {
     int qrow = q0 + col;
-    if (qrow > a.Sq - 1) qrow = a.Sq - 1;
+    if (qrow > q_end - 1) qrow = q_end - 1;
     const __bf16* qp = a.q + (int64_t)b * a.q_sb + (int64_t)qrow * a.q_ss + (int64_t)h * a.q_sh + 8 * hh;
 #pragma unroll
     for (int s = 0; s < D / 16; ++s) qf[s] = *reinterpret_cast<const bf16x8*>(qp + 16 * s);
@@ -235,7 +242,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
 
   // ---- tile bookkeeping -----------------------------------------------------------------
   int n_tiles = 0;
-  for (int s = seg_begin; s < seg_end; ++s) n_tiles += (a.kv_len[chunk_of(s)] + kBK - 1) / kBK;
+  for (int s = seg_begin; s < seg_end; ++s) n_tiles += (kv_len_of(s) + kBK - 1) / kBK;
 
   // Two cursors walk the job's chunks tile by tile, all in scalar registers: the load cursor
   // (ahead of the compute cursor: base pointers of the tile and keys left in its chunk) and
@@ -245,18 +252,19 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   const uint8_t* ld_v = nullptr;
   int cp_seg = seg_begin - 1, cp_left = 0;
   auto ld_next_chunk = [&]() {
-    do { ++ld_seg; } while (ld_seg < seg_end && a.kv_len[chunk_of(ld_seg)] == 0);
+    do { ++ld_seg; } while (ld_seg < seg_end && kv_len_of(ld_seg) == 0);
     if (ld_seg < seg_end) {
       const int cid = chunk_of(ld_seg);
-      const int64_t head_off = (int64_t)b * a.kv_sb[cid] + (int64_t)h * a.kv_sh;
+      const int64_t head_off =
+          (int64_t)b * a.kv_sb[cid] + (int64_t)h * a.kv_sh + (int64_t)kv_begin_of(ld_seg) * a.kv_ss;
       ld_k = reinterpret_cast<const uint8_t*>(a.k[cid] + head_off);
       ld_v = reinterpret_cast<const uint8_t*>(a.v[cid] + head_off);
-      ld_left = a.kv_len[cid];
+      ld_left = kv_len_of(ld_seg);
     }
   };
   auto cp_next_chunk = [&]() {
-    do { ++cp_seg; } while (cp_seg < seg_end && a.kv_len[chunk_of(cp_seg)] == 0);
-    if (cp_seg < seg_end) cp_left = a.kv_len[chunk_of(cp_seg)];
+    do { ++cp_seg; } while (cp_seg < seg_end && kv_len_of(cp_seg) == 0);
+    if (cp_seg < seg_end) cp_left = kv_len_of(cp_seg);
   };
   ld_next_chunk();
   cp_next_chunk();
@@ -495,12 +503,10 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
         for (int r = 0; r < 16; ++r) o_acc[i][r] *= alpha;
     }
     const float mc = m_ref * c;
-    // The row sum is taken over the bf16-ROUNDED probabilities, i.e. exactly the weights the
-    // P V product uses, two per instruction (v_dot2c_f32_bf16 against (1, 1)).
+    // The row sum is accumulated from the fp32 probabilities (before rounding to bf16): summing
+    // the rounded ones would be two per instruction, but for short key ranges their rounding
+    // errors do not average out and the lse drifts past 1e-3.
     float rs0 = 0.f, rs1 = 0.f;
-    bf16x2 ones;
-    ones.x = (__bf16)1.0f;
-    ones.y = (__bf16)1.0f;
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
@@ -508,9 +514,9 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
         f32x2 p;
         p.x = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[kb][r], c, -mc));
         p.y = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[kb][r + 1], c, -mc));
+        rs0 += p.x;
+        rs1 += p.y;
         const bf16x2 pb = __builtin_convertvector(p, bf16x2);
-        if (r & 2) rs1 = __builtin_amdgcn_fdot2_f32_bf16(pb, ones, rs1, false);
-        else rs0 = __builtin_amdgcn_fdot2_f32_bf16(pb, ones, rs0, false);
         p_frag[kb][r >> 3][r & 7] = pb.x;
         p_frag[kb][r >> 3][(r & 7) + 1] = pb.y;
       }
@@ -540,7 +546,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   const float lse = l_tot > 0.f ? (m_ref * c + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f : -INFINITY;
   const int qrow = q0 + col;
-  if (hh == 0 && qrow < a.Sq) lse_ptr[((int64_t)b * a.H + h) * a.Sq + qrow] = lse;
+  if (hh == 0 && qrow < q_end) lse_ptr[((int64_t)b * a.H + h) * a.Sq + qrow] = lse;
 
   // O^T (registers, [d][query]) -> LDS [query][d] bf16 -> coalesced 16-byte stores.
   phase_barrier();  // every wavefront is done with the tile buffers
@@ -571,7 +577,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     const int row = p * kRowsPerPass + rr;
     const int qg = q0 + row;
     const u32x4 val = *reinterpret_cast<const u32x4*>(ol + row * T::kPitchO + cc * 16);
-    if (qg < a.Sq) {
+    if (qg < q_end) {
       __bf16* dst = out_ptr + (((int64_t)b * a.Sq + qg) * a.H + h) * D + cc * 8;
       *reinterpret_cast<u32x4*>(dst) = val;
     }

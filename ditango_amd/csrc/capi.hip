@@ -98,11 +98,14 @@ static int fill_common(AttnArgs& a, const void* q, int32_t B, int32_t Sq, int32_
   return DT_OK;
 }
 
-extern "C" int dt_attn_jobs_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D, int64_t q_sb, int64_t q_ss,
-                                int64_t q_sh, int32_t n_chunks, const void* const* k_ptrs, const void* const* v_ptrs,
-                                const int32_t* kv_lens, const int64_t* kv_sb, int64_t kv_ss, int64_t kv_sh,
-                                int32_t n_jobs, const int32_t* job_begin, const int32_t* job_chunks,
-                                void* const* out_ptrs, float* const* lse_ptrs, float softmax_scale, void* stream) {
+extern "C" int dt_attn_seg_jobs_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D, int64_t q_sb,
+                                    int64_t q_ss, int64_t q_sh, int32_t n_chunks, const void* const* k_ptrs,
+                                    const void* const* v_ptrs, const int32_t* kv_lens, const int64_t* kv_sb,
+                                    int64_t kv_ss, int64_t kv_sh, int32_t n_jobs, const int32_t* job_begin,
+                                    const int32_t* job_chunks, const int32_t* entry_kv_begin,
+                                    const int32_t* entry_kv_len, const int32_t* job_q_begin,
+                                    const int32_t* job_q_len, void* const* out_ptrs, float* const* lse_ptrs,
+                                    float softmax_scale, void* stream) {
   AttnArgs a{};
   if (int rc = fill_common(a, q, B, Sq, H, D, q_sb, q_ss, q_sh, n_chunks, k_ptrs, v_ptrs, kv_lens, kv_sb, kv_ss, kv_sh,
                            softmax_scale))
@@ -116,6 +119,11 @@ extern "C" int dt_attn_jobs_fwd(const void* q, int32_t B, int32_t Sq, int32_t H,
     set_error("job_begin must start at 0 and end at most at %d", DT_MAX_JOB_ENTRIES);
     return DT_ERR_INVALID;
   }
+  if ((entry_kv_begin == nullptr) != (entry_kv_len == nullptr) || (job_q_begin == nullptr) != (job_q_len == nullptr)) {
+    set_error("range arrays come in (begin, len) pairs");
+    return DT_ERR_INVALID;
+  }
+  int32_t longest = 0;
   for (int j = 0; j < n_jobs; ++j) {
     if (job_begin[j + 1] < job_begin[j]) {
       set_error("job_begin is not monotone at job %d", j);
@@ -128,16 +136,48 @@ extern "C" int dt_attn_jobs_fwd(const void* q, int32_t B, int32_t Sq, int32_t H,
     a.job_out[j] = static_cast<__bf16*>(out_ptrs[j]);
     a.job_lse[j] = lse_ptrs[j];
     a.job_begin[j] = job_begin[j];
+    const int32_t qb = job_q_begin ? job_q_begin[j] : 0;
+    const int32_t ql = job_q_len ? job_q_len[j] : Sq;
+    if (qb < 0 || ql < 0 || (int64_t)qb + ql > Sq) {
+      set_error("job %d: query rows [%d, %d) outside [0, %d)", j, qb, qb + ql, Sq);
+      return DT_ERR_INVALID;
+    }
+    a.job_q_begin[j] = qb;
+    a.job_q_len[j] = ql;
+    longest = ql > longest ? ql : longest;
   }
   a.job_begin[n_jobs] = job_begin[n_jobs];
   for (int e = 0; e < job_begin[n_jobs]; ++e) {
-    if (job_chunks[e] < 0 || job_chunks[e] >= n_chunks) {
-      set_error("job chunk reference %d is outside the chunk table", job_chunks[e]);
+    const int32_t c = job_chunks[e];
+    if (c < 0 || c >= n_chunks) {
+      set_error("job chunk reference %d is outside the chunk table", c);
       return DT_ERR_INVALID;
     }
-    a.job_chunks[e] = job_chunks[e];
+    const int32_t kb = entry_kv_begin ? entry_kv_begin[e] : 0;
+    const int32_t kl = entry_kv_len ? entry_kv_len[e] : kv_lens[c];
+    if (kb < 0 || kl < 0 || (int64_t)kb + kl > kv_lens[c]) {
+      set_error("chunk reference %d: keys [%d, %d) outside chunk %d of length %d", e, kb, kb + kl, c, kv_lens[c]);
+      return DT_ERR_INVALID;
+    }
+    a.job_chunks[e] = c;
+    a.entry_kv_begin[e] = kb;
+    a.entry_kv_len[e] = kl;
   }
+  // size the grid for the longest job; shorter jobs leave their surplus workgroups at once
+  a.nqt = (longest + 255) / 256;
+  a.total = B * H * a.nqt;
+  a.per_xcd = (a.total + 7) / 8;
   return launch_attn(a, D, n_jobs, (hipStream_t)stream);
+}
+
+extern "C" int dt_attn_jobs_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D, int64_t q_sb, int64_t q_ss,
+                                int64_t q_sh, int32_t n_chunks, const void* const* k_ptrs, const void* const* v_ptrs,
+                                const int32_t* kv_lens, const int64_t* kv_sb, int64_t kv_ss, int64_t kv_sh,
+                                int32_t n_jobs, const int32_t* job_begin, const int32_t* job_chunks,
+                                void* const* out_ptrs, float* const* lse_ptrs, float softmax_scale, void* stream) {
+  return dt_attn_seg_jobs_fwd(q, B, Sq, H, D, q_sb, q_ss, q_sh, n_chunks, k_ptrs, v_ptrs, kv_lens, kv_sb, kv_ss, kv_sh,
+                              n_jobs, job_begin, job_chunks, nullptr, nullptr, nullptr, nullptr, out_ptrs, lse_ptrs,
+                              softmax_scale, stream);
 }
 
 extern "C" int dt_attn_chunk_fwd(const void* q, const void* k, const void* v, void* out, float* lse, int32_t B,

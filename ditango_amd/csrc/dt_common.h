@@ -32,6 +32,12 @@ struct AttnArgs {
   float* job_lse[DT_MAX_JOBS];
   int32_t job_begin[DT_MAX_JOBS + 1];
   int32_t job_chunks[DT_MAX_JOB_ENTRIES];
+  // query rows [job_q_begin, job_q_begin + job_q_len) of each job; keys [kv_begin, kv_begin + kv_len)
+  // of each chunk reference (a segment of a packed variable-length batch is a job on sub-ranges)
+  int32_t job_q_begin[DT_MAX_JOBS];
+  int32_t job_q_len[DT_MAX_JOBS];
+  int32_t entry_kv_begin[DT_MAX_JOB_ENTRIES];
+  int32_t entry_kv_len[DT_MAX_JOB_ENTRIES];
   // device-listed jobs (dev_ids != nullptr): job j computes chunk dev_ids[j] if j < *dev_count
   const int32_t* dev_ids;
   const int32_t* dev_count;

@@ -83,6 +83,30 @@ int dt_attn_jobs_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D,
                      float softmax_scale, void* stream);
 
 /*
+ * The same launch with sub-ranges: job j covers the query rows
+ * [job_q_begin[j], job_q_begin[j] + job_q_len[j]) only (other rows of its
+ * destination are left untouched) and chunk reference e covers the keys
+ * [entry_kv_begin[e], entry_kv_begin[e] + entry_kv_len[e]) of its chunk.  One
+ * segment of a packed variable-length batch is one such job, so this replaces
+ *   flash_attn_varlen_func(q, k, v, cu_seqlens_q, cu_seqlens_kv, max_seqlen_q,
+ *                          max_seqlen_kv, dropout_p=0.0, return_attn_probs=True)
+ * as called at core/attention.py:314-324 and :366-376, where q/k/v are packed
+ * [total, H, D] (pass B = 1, Sq = total) and the lse is [H, total].  A job
+ * without keys writes out = 0, lse = -inf.  Either pair of range arrays may be
+ * NULL (whole rows / whole chunks).  All range arrays are HOST arrays.
+ */
+int dt_attn_seg_jobs_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D,
+                         int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
+                         int32_t n_chunks, const void* const* k_ptrs, const void* const* v_ptrs,
+                         const int32_t* kv_lens, const int64_t* kv_stride_b,
+                         int64_t kv_stride_s, int64_t kv_stride_h,
+                         int32_t n_jobs, const int32_t* job_begin, const int32_t* job_chunks,
+                         const int32_t* entry_kv_begin, const int32_t* entry_kv_len,
+                         const int32_t* job_q_begin, const int32_t* job_q_len,
+                         void* const* out_ptrs, float* const* lse_ptrs,
+                         float softmax_scale, void* stream);
+
+/*
  * Same, driven by a schedule that lives in device memory (dt_build_schedule*):
  * job j (0 <= j < max_jobs) is active iff j < *dev_count and computes the
  * single chunk id dev_compute_ids[j], writing its state into cache slot

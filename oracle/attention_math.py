@@ -135,6 +135,27 @@ def full_attention(
     return chunk_attention(q, k, v, compute_dtype=compute_dtype)
 
 
+def varlen_chunk_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens_q: Sequence[int],
+                           cu_seqlens_kv: Sequence[int]) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``flash_attn_varlen_func`` as called at core/attention.py:314-324,366-376, by its
+    published contract: packed ``q [total_q,H,D]``, ``k/v [total_k,H,D]``; segment ``i`` of the
+    queries attends to segment ``i`` of the keys only.  Returns (out ``[total_q,H,D]``, lse
+    ``[H,total_q]``), both fp32.  Query rows outside every segment get out = 0; a segment
+    without keys gets out = 0, lse = -inf.  Each segment is the dense closed form."""
+    total_q, H, D = q.shape
+    out = torch.zeros(total_q, H, D, dtype=torch.float32)
+    lse = torch.full((H, total_q), -math.inf, dtype=torch.float32)
+    for i in range(len(cu_seqlens_q) - 1):
+        q0, q1 = int(cu_seqlens_q[i]), int(cu_seqlens_q[i + 1])
+        k0, k1 = int(cu_seqlens_kv[i]), int(cu_seqlens_kv[i + 1])
+        if q1 <= q0:
+            continue
+        o, l = chunk_attention(q[None, q0:q1], k[None, k0:k1], v[None, k0:k1])
+        out[q0:q1] = o[0]
+        lse[:, q0:q1] = l[0]
+    return out, lse
+
+
 def rel_l1(new: torch.Tensor, ori: torch.Tensor) -> float:
     """utils.py:202-267, tensor branch: ``mean|new-ori| / (mean|ori| + 1e-8)``
     over entries where neither is NaN; ``inf`` if nothing is valid; falls back

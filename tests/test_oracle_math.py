@@ -111,3 +111,25 @@ def test_rel_l1_closed_form():
     assert abs(om.rel_l1(a, b) - 0.25 / (1.75 + 1e-8)) < 1e-7
     assert om.rel_l1(torch.tensor([float("nan")]), torch.tensor([1.0])) == float("inf")
     assert om.rel_l1(torch.tensor([3.0, -5.0]), torch.tensor([0.0, 0.0])) == 4.0
+
+
+def test_varlen_attention_is_block_diagonal_attention():
+    g = torch.Generator().manual_seed(12)
+    q = torch.randn(20, 2, 16, generator=g)
+    k = torch.randn(30, 2, 16, generator=g)
+    v = torch.randn(30, 2, 16, generator=g)
+    # one segment spanning everything is the dense call
+    o, l = om.varlen_chunk_attention(q, k, v, [0, 20], [0, 30])
+    od, ld = om.chunk_attention(q[None], k[None], v[None])
+    assert torch.equal(o, od[0]) and torch.equal(l, ld[0])
+    # two segments == attention under a block-diagonal mask (library routine)
+    o, l = om.varlen_chunk_attention(q, k, v, [0, 12, 20], [0, 25, 30])
+    mask = torch.zeros(20, 30, dtype=torch.bool)
+    mask[:12, :25] = True
+    mask[12:, 25:] = True
+    ref = F.scaled_dot_product_attention(q.permute(1, 0, 2)[None], k.permute(1, 0, 2)[None], v.permute(1, 0, 2)[None],
+                                         attn_mask=mask)[0].permute(1, 0, 2)
+    assert torch.allclose(o, ref, atol=1e-5)
+    # a segment without keys is the neutral state; rows outside every segment stay zero
+    o, l = om.varlen_chunk_attention(q, k, v, [0, 12, 18], [0, 30, 30])
+    assert (o[12:] == 0).all() and torch.isinf(l[:, 12:]).all()

@@ -1,0 +1,141 @@
+"""The variable-length entry (HunyuanVideo): packed [total,H,D] inputs, segment i of the queries
+attends to segment i of every KV chunk; segment boundaries of a chunk travel with the chunk."""
+import pytest
+import torch
+
+from oracle import attention_math as om
+from oracle.state_machine import RingOracle, strides_from_dividers
+
+pytestmark = pytest.mark.gpu
+OUT_TOL, LSE_TOL = 2e-2, 1e-3
+
+
+@pytest.fixture
+def env(hip):
+    from ditango_amd.core import config, parallel_state, redundancy_map as rmod
+    from ditango_amd import utils
+
+    def make(N, rank, T, L):
+        parallel_state.init_local_groups(N, rank)
+        config.init_config(None, num_inference_steps=T, num_layers=L)
+        rmod.destroy_redundancy_map()
+        rmod._redundancy_map = rmod.RedundancyMap(config.get_config())
+        return rmod.get_redundancy_map()
+
+    yield make
+    from ditango_amd.core import parallel_state, redundancy_map as rmod
+    rmod.destroy_redundancy_map()
+    parallel_state.destroy_local_groups()
+    utils.update_timestep(0)
+
+
+@pytest.mark.parametrize("D,cu_q,cu_k", [
+    (128, [0, 300], [0, 333]),
+    (128, [0, 257, 300], [0, 300, 333]),
+    (64, [0, 100, 100, 290], [0, 64, 200, 333]),      # an empty query segment
+    (128, [0, 10, 280], [0, 0, 333]),                 # a segment without keys
+])
+def test_segment_jobs_match_varlen_oracle(hip, D, cu_q, cu_k):
+    H = 3
+    g = torch.Generator().manual_seed(len(cu_q) + D)
+    q = torch.randn(300, H, D, generator=g).bfloat16()
+    k = torch.randn(333, H, D, generator=g).bfloat16()
+    v = torch.randn(333, H, D, generator=g).bfloat16()
+    ref_out, ref_lse = om.varlen_chunk_attention(q, k, v, cu_q, cu_k)
+    dq, dk, dv = q.cuda()[None], k.cuda()[None], v.cuda()[None]
+    out = torch.zeros(1, 300, H, D, dtype=torch.bfloat16, device="cuda")
+    lse = torch.full((1, H, 300), float("-inf"), device="cuda")
+    table = hip.ChunkTable([dk], [dv])
+    nseg = len(cu_q) - 1
+    hip.attn_jobs_fwd(dq, table, [[0]] * nseg, [out] * nseg, [lse] * nseg,
+                      q_ranges=[(cu_q[i], cu_q[i + 1] - cu_q[i]) for i in range(nseg)],
+                      kv_ranges=[[(cu_k[i], cu_k[i + 1] - cu_k[i])] for i in range(nseg)])
+    torch.cuda.synchronize()
+    assert (out[0].float().cpu() - ref_out).abs().max() <= OUT_TOL
+    got, ref = lse[0].cpu(), ref_lse
+    finite = torch.isfinite(ref)
+    assert torch.equal(torch.isfinite(got), finite)
+    assert (got[finite] - ref[finite]).abs().max() <= LSE_TOL
+
+
+def test_single_segment_reduces_to_the_dense_path(env, hip):
+    from ditango_amd.core.attention import proAttention
+    from ditango_amd.core.parallel_state import get_usp_group
+    N, S, H, D = 2, 150, 2, 128
+    env(N, 0, 3, 1)
+    g = torch.Generator().manual_seed(1)
+    q = torch.randn(S, H, D, generator=g).bfloat16().cuda()
+    ks = [torch.randn(S, H, D, generator=g).bfloat16().cuda() for _ in range(N)]
+    vs = [torch.randn(S, H, D, generator=g).bfloat16().cuda() for _ in range(N)]
+    group = get_usp_group()
+    cu = torch.tensor([0, S], dtype=torch.int32)
+    group.set_kv_chunks(ks, vs, cu_seqlens_kv=[cu] * N)
+    a = proAttention(0, group).varlen_attn(q, ks[0], vs[0], cu, cu, S, S)
+    group.set_kv_chunks([k[None] for k in ks], [v[None] for v in vs])
+    b = proAttention(0, group).attn(q[None], ks[0][None], vs[0][None])
+    torch.cuda.synchronize()
+    assert tuple(a.shape) == (S, H, D) and torch.equal(a, b[0])
+    # no sequence lengths at all: the dense path (core/attention.py:252-254)
+    c = proAttention(0, group).varlen_attn(q[None], ks[0][None], vs[0][None])
+    assert torch.equal(c, b)
+
+
+def test_varlen_stride_mode_matches_numeric_oracle(env, hip):
+    """Two segments per sample (valid tokens | padding), different boundaries in every chunk,
+    over a divider sequence with reuse, coarsening and a full refresh."""
+    from ditango_amd.core.attention import proAttention
+    from ditango_amd.core.parallel_state import get_usp_group
+    from ditango_amd.utils import update_timestep
+    N, rank, H, D = 4, 2, 2, 128
+    col = (1, 1, 1, 4, 4, 2, 2, 1, 1)
+    T = len(col)
+    rm = env(N, rank, T, 1)
+    rm.divider_map[:, 0] = torch.tensor(col)
+    curr, nxt = strides_from_dividers(N, col)
+    total_q = 180
+    cu_q = [0, 150, 180]
+    lens = [170, 181, 160, 175]
+    cu_k = [[0, 140, 170], [0, 150, 181], [0, 131, 160], [0, 150, 175]]
+    g = torch.Generator().manual_seed(31)
+    q = torch.randn(total_q, H, D, generator=g)
+    ks = [torch.randn(n, H, D, generator=g) for n in lens]
+    vs = [torch.randn(n, H, D, generator=g) for n in lens]
+    state = {}
+
+    def attn_fn(r, c):
+        if r != rank:
+            return (c,)
+        o, l = om.varlen_chunk_attention(state["q"], state["ks"][c], state["vs"][c], cu_q, cu_k[c])
+        return (o[None], l[None])
+
+    def merge_fn(a, b):
+        if isinstance(b[0], int):
+            return tuple(b) if a is None else tuple(a) + tuple(b)
+        return om.update_out_and_lse(None if a is None else a[0], None if a is None else a[1], b[0], b[1])
+
+    def store_fn(s):
+        return s if isinstance(s[0], int) else (om.bf16_round(s[0]), s[1])
+
+    ring = RingOracle(N, attn_fn=attn_fn, merge_fn=merge_fn, store_fn=store_fn)
+    group = get_usp_group()
+    attn = proAttention(0, group)
+    for t in range(T):
+        print(f"case varlen t={t} curr={curr[t]} next={nxt[t]}", flush=True)
+        qb, kb, vb = q.bfloat16(), [k.bfloat16() for k in ks], [v.bfloat16() for v in vs]
+        state.update(q=qb, ks=kb, vs=vb)
+        tr = ring.call(t, curr[t], nxt[t])[rank]
+        update_timestep(t)
+        dk, dv = [k.cuda() for k in kb], [v.cuda() for v in vb]
+        group.set_kv_chunks(dk, dv, cu_seqlens_kv=[torch.tensor(c, dtype=torch.int32) for c in cu_k])
+        out = attn.varlen_attn(qb.cuda(), dk[rank], dv[rank], torch.tensor(cu_q, dtype=torch.int32),
+                               torch.tensor(cu_k[rank], dtype=torch.int32), max(150, 30), max(lens))
+        torch.cuda.synchronize()
+        assert attn.last_plan.computed == tr.computed and attn.last_plan.stores == tr.stores
+        ref_out, ref_lse = tr.out
+        err = (out.cpu() - ref_out[0]).abs().max().item()
+        lerr = (attn.last_lse.cpu().squeeze(-1)[0].transpose(0, 1) - ref_lse.squeeze(-1)[0].transpose(0, 1)).abs().max().item()
+        print(f"  out max-abs {err:.3e} lse {lerr:.3e}", flush=True)
+        assert err <= OUT_TOL and lerr <= LSE_TOL
+        q = q + 0.01 * torch.randn(q.shape, generator=g)
+        ks = [k + 0.01 * torch.randn(k.shape, generator=g) for k in ks]
+        vs = [v + 0.01 * torch.randn(v.shape, generator=g) for v in vs]
