@@ -32,9 +32,10 @@
 //     of the second MFMA, O^T += V^T P^T, whose A operand is one 16-byte read of
 //     8 consecutive keys of one d-row of the transposed V tile.
 //   * O^T stays in registers as [d][query]: a rescale is a multiply by a per-lane
-//     scalar, and it is only done when some query's running maximum grew by more
-//     than 2^8 (the reference maximum may lag; the lse stays exact).  Row sums are
-//     accumulated in fp32 from the unrounded probabilities.  The epilogue
+//     scalar.  The reference maximum the accumulators are scaled to may lag behind
+//     the true row maximum (the lse stays exact): the common path computes no row
+//     maximum at all, the fp32 row sum it needs anyway is the overflow detector,
+//     and only a tile whose sum exceeds 2^12 is redone with its exact maximum.  The epilogue
 //     transposes through LDS so that the global stores are 16 bytes per lane.
 //   * Workgroups are mapped to (head, query tile) so that the 8 XCDs each work
 //     through a contiguous range of heads: the workgroups that share an XCD's
@@ -143,9 +144,10 @@ __device__ __forceinline__ void phase_barrier_after_matrix(V (&sa)[2], V (&oa)[N
   __builtin_amdgcn_sched_barrier(0);
 }
 
-// Largest growth of the running maximum (in log2 units of the scaled scores) that is
-// tolerated without rescaling the accumulators: probabilities then stay below 2^kTau.
-constexpr float kTau = 8.0f;
+// A tile's per-lane sum of probabilities (32 of them) above which the tile is redone with an
+// exact row maximum.  Below it every probability is at most 2^12: harmless for the bf16
+// operand (same relative precision at any exponent) and for the fp32 accumulators.
+constexpr float kSumLimit = 4096.0f;
 
 template <int D>
 struct Tile {
@@ -485,27 +487,13 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
           if (key >= lim) s_acc[kb][r] = -INFINITY;
         }
     }
-    float mx = s_acc[0][0];
-#pragma unroll
-    for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s_acc[0][r]);
-#pragma unroll
-    for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s_acc[1][r]);
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    // rescale only if some query's maximum grew by more than kTau (always true on the first tile)
-    if (__any((mx - m_ref) * c > kTau)) {
-      const float m_new = fmaxf(m_ref, mx);
-      const float alpha = __builtin_amdgcn_exp2f((m_ref - m_new) * c);
-      m_ref = m_new;
-      l_run *= alpha;
-#pragma unroll
-      for (int i = 0; i < D / 32; ++i)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) o_acc[i][r] *= alpha;
-    }
-    const float mc = m_ref * c;
-    // The row sum is accumulated from the fp32 probabilities (before rounding to bf16): summing
-    // the rounded ones would be two per instruction, but for short key ranges their rounding
-    // errors do not average out and the lse drifts past 1e-3.
+    // Probabilities relative to the reference maximum the accumulators are scaled to.  The
+    // maximum of the tile is NOT computed on this path: the row sum, needed anyway, doubles as
+    // the overflow detector.  While it stays below kSumLimit every probability is bounded and a
+    // lagging reference is harmless (the lse stays exact); otherwise -- including the first tile,
+    // where the reference is -inf and the sum comes out inf or NaN -- the tile is redone below
+    // with its exact maximum.
+    float mc = m_ref * c;
     float rs0 = 0.f, rs1 = 0.f;
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
@@ -520,6 +508,39 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
         p_frag[kb][r >> 3][r & 7] = pb.x;
         p_frag[kb][r >> 3][(r & 7) + 1] = pb.y;
       }
+    if (__any(!(rs0 + rs1 <= kSumLimit))) {
+      float mx = s_acc[0][0];
+#pragma unroll
+      for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s_acc[0][r]);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s_acc[1][r]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      const float m_new = fmaxf(m_ref, mx);
+      const float alpha = m_new > -INFINITY ? __builtin_amdgcn_exp2f((m_ref - m_new) * c) : 1.f;
+      m_ref = m_new;
+      l_run *= alpha;
+#pragma unroll
+      for (int i = 0; i < D / 32; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o_acc[i][r] *= alpha;
+      // a row whose keys are all masked so far keeps m_ref = -inf: use 0 so that exp2(-inf - 0) = 0
+      mc = m_new > -INFINITY ? m_new * c : 0.f;
+      rs0 = 0.f;
+      rs1 = 0.f;
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) {
+          f32x2 p;
+          p.x = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[kb][r], c, -mc));
+          p.y = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[kb][r + 1], c, -mc));
+          rs0 += p.x;
+          rs1 += p.y;
+          const bf16x2 pb = __builtin_convertvector(p, bf16x2);
+          p_frag[kb][r >> 3][r & 7] = pb.x;
+          p_frag[kb][r >> 3][(r & 7) + 1] = pb.y;
+        }
+    }
     l_run += rs0 + rs1;
     phase_barrier_after_vector(p_frag);
 

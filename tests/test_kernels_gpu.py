@@ -200,3 +200,40 @@ def test_rel_l1_sums(hip):
     val = (s[0] / s[3]).item() / ((s[2] / s[3]).item() + 1e-8)
     assert s[3].item() == a.numel() - 2
     assert abs(val - ref) < 1e-5 * max(1.0, abs(ref))
+
+
+@pytest.mark.parametrize("case", ["ramp", "huge", "late_outlier", "descending"])
+def test_chunk_attention_with_drifting_maximum(hip, case):
+    """The kernel keeps a reference maximum that may lag behind the true row maximum and only
+    redoes a tile when its row sum overflows a bound: drive that logic with scores that grow
+    steadily along the keys, scores of huge magnitude, and one dominant key at the very end."""
+    B, Sq, Sk, H, D = 1, 130, 1000, 2, 128
+    g = torch.Generator().manual_seed(42)
+    q = torch.randn(B, Sq, H, D, generator=g)
+    k = torch.randn(B, Sk, H, D, generator=g)
+    v = torch.randn(B, Sk, H, D, generator=g)
+    qdir = q / q.norm(dim=-1, keepdim=True)
+    if case == "ramp":          # score of key j grows linearly from about -40 to +40
+        ramp = torch.linspace(-40, 40, Sk).view(1, Sk, 1, 1) * math.sqrt(D)
+        k = 0.1 * k + ramp * qdir.mean(dim=1, keepdim=True) / qdir.mean(dim=1, keepdim=True).norm(dim=-1, keepdim=True)
+        q = qdir.mean(dim=1, keepdim=True).expand_as(q) / qdir.mean(dim=1, keepdim=True).norm(dim=-1, keepdim=True) + 0.05 * q
+    elif case == "descending":  # the first tile holds the maximum, later probabilities shrink to nothing
+        ramp = torch.linspace(40, -40, Sk).view(1, Sk, 1, 1) * math.sqrt(D)
+        d0 = qdir.mean(dim=1, keepdim=True) / qdir.mean(dim=1, keepdim=True).norm(dim=-1, keepdim=True)
+        k = 0.1 * k + ramp * d0
+        q = d0.expand_as(q) + 0.05 * q
+    elif case == "huge":        # natural-log scores of magnitude in the hundreds
+        q = q * 6
+        k = k * 6
+    elif case == "late_outlier":
+        k[:, -1] = 30 * qdir[:, 7]
+    q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
+    ref_out, ref_lse = om.chunk_attention(q, k, v, compute_dtype=torch.float64)
+    out, lse = hip.attn_chunk_fwd(q.cuda(), k.cuda(), v.cuda())
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
+    err = (out.float().cpu() - ref_out.float()).abs().max().item()
+    lerr = ((lse.cpu().double() - ref_lse).abs() / ref_lse.abs().clamp_min(1.0)).max().item()
+    print(f"{case}: out max-abs {err:.3e}, lse max rel/abs {lerr:.3e}, lse range [{ref_lse.min():.1f}, {ref_lse.max():.1f}]", flush=True)
+    assert err <= OUT_TOL
+    assert lerr <= LSE_TOL
