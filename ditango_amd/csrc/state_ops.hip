@@ -99,8 +99,8 @@ __device__ __forceinline__ void store_row8(void* base, bool fp32, int64_t row_el
       a[i] = __float_as_uint(x[i]);
       b[i] = __float_as_uint(x[4 + i]);
     }
-    *reinterpret_cast<u32x4*>(p) = a;
-    *reinterpret_cast<u32x4*>(p + D / 2) = b;
+    __builtin_nontemporal_store(a, reinterpret_cast<u32x4*>(p));
+    __builtin_nontemporal_store(b, reinterpret_cast<u32x4*>(p + D / 2));
   } else {
     uint16_t* p = reinterpret_cast<uint16_t*>(base) + row_elem + 4 * c;
     u32x2 g0, g1;
