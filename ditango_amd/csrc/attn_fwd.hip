@@ -15,11 +15,12 @@
 //     next K/V tile into LDS), and vice versa; a workgroup barrier separates the
 //     phases.  Each SIMD holds one wavefront of either group, so its matrix pipe
 //     and its vector ALU are busy at the same time instead of taking turns.
-//   * KV is consumed in tiles of 64 keys.  K is staged in LDS as [key][d] (two
-//     buffers), V is transposed on the way in and staged as [d][key] (three
-//     buffers, because the P V product of a tile runs one phase after its
-//     scores).  Rows are padded by 16 bytes so that the MFMA operand reads
-//     (ds_read_b128 with immediate offsets) are bank-conflict free.  Tiles come
+//   * KV is consumed in tiles of 64 keys, staged in LDS as they come, [key][d]:
+//     K in two buffers, V in three (the P V product of a tile runs one phase
+//     after its scores).  The second MFMA needs V^T; the transposition is done
+//     by the LDS read itself (ds_read_b64_tr_b16), so filling a tile is eight
+//     16-byte copies per thread and no ALU work.  Rows are padded so that all
+//     operand reads are bank-conflict free and use immediate offsets.  Tiles come
 //     in through raw buffer loads: descriptor in scalar registers, loop-invariant
 //     lane offsets, and rows past the end of a chunk read as zeros.
 //   * Scores are computed TRANSPOSED, S^T = K Q^T, with v_mfma_f32_32x32x16_bf16:
@@ -29,8 +30,8 @@
 //   * The rows of the K operand are permuted (bits 2 and 3 of the row index
 //     swapped) so that the 8 accumulator registers a lane holds for a half tile
 //     are 8 CONSECUTIVE keys.  Rounded to bf16 they are directly the B operand
-//     of the second MFMA, O^T += V^T P^T, whose A operand is one 16-byte read of
-//     8 consecutive keys of one d-row of the transposed V tile.
+//     of the second MFMA, O^T += V^T P^T, whose A operand (8 consecutive keys of
+//     one d column) is two transposing reads of 4 keys each.
 //   * O^T stays in registers as [d][query]: a rescale is a multiply by a per-lane
 //     scalar.  The reference maximum the accumulators are scaled to may lag behind
 //     the true row maximum (the lse stays exact): the common path computes no row
@@ -80,24 +81,6 @@ __device__ __forceinline__ int key_of_row(int i) {
 
 // Raw buffer descriptor word 3 for gfx9-family targets (32-bit data format, no swizzle).
 constexpr int kRsrcFlags = 0x00020000;
-
-template <int W>
-__device__ __forceinline__ typename VecOf<W>::type buffer_load_v(__amdgpu_buffer_rsrc_t r, int voff);
-template <>
-__device__ __forceinline__ u32x4 buffer_load_v<4>(__amdgpu_buffer_rsrc_t r, int voff) {
-  return __builtin_amdgcn_raw_buffer_load_b128(r, voff, 0, 0);
-}
-template <>
-__device__ __forceinline__ u32x2 buffer_load_v<2>(__amdgpu_buffer_rsrc_t r, int voff) {
-  return __builtin_amdgcn_raw_buffer_load_b64(r, voff, 0, 0);
-}
-template <>
-__device__ __forceinline__ uint32_t buffer_load_v<1>(__amdgpu_buffer_rsrc_t r, int voff) {
-  return __builtin_amdgcn_raw_buffer_load_b32(r, voff, 0, 0);
-}
-__device__ __forceinline__ uint32_t dword_of(uint32_t v, int) { return v; }
-__device__ __forceinline__ uint32_t dword_of(u32x2 v, int w) { return v[w]; }
-__device__ __forceinline__ uint32_t dword_of(u32x4 v, int w) { return v[w]; }
 
 // Workgroup barrier between the phases.  Waits for this wavefront's LDS traffic only:
 // global loads issued for a later tile stay in flight across it.
@@ -151,30 +134,39 @@ constexpr float kSumLimit = 4096.0f;
 
 template <int D>
 struct Tile {
-  // LDS tiles are padded by 16 bytes per row instead of swizzled: every operand read is then
-  // "lane base + compile-time constant", i.e. a ds_read_b128 with an immediate offset and no
-  // address arithmetic in the loop, and 16 consecutive rows still fall into 16 distinct
-  // 16-byte bank groups (pitch mod 256 is 16 or 144).
-  static constexpr int kPitchK = D * 2 + 16;          // one key, all d
-  static constexpr int kPitchV = kBK * 2 + 16;        // one d, 64 keys
-  static constexpr int kChunksK = D / 8;              // 16-byte chunks per K row
+  // Both tiles sit in LDS as [key][d] rows, padded instead of swizzled: every operand read is
+  // then "lane base + compile-time constant" (immediate offsets, no address arithmetic in the
+  // loop).  K rows are padded by 16 bytes: the 16 lanes of a ds_read_b128 pass read 16 different
+  // rows at the same column and land in 16 distinct 16-byte bank groups.  V rows are padded by
+  // 64 bytes: a transposing 8-byte read pass touches 4 rows x 2 column groups, which 64-byte
+  // row shifts spread over all banks.
+  static constexpr int kPitchK = D * 2 + 16;
+  static constexpr int kPitchV = D * 2 + 64;
+  static constexpr int kChunks = D / 8;               // 16-byte chunks per row
   static constexpr int kBytesK = kBK * kPitchK;
-  static constexpr int kBytesV = D * kPitchV;
+  static constexpr int kBytesV = kBK * kPitchV;
   static constexpr int kOffV = kNumKBuf * kBytesK;    // V buffers follow the K buffers
-  static constexpr int kLoadsK = kBK * kChunksK / kThreads;  // 16-byte K loads per thread (2 or 1)
-  static constexpr int kRowStepK = kThreads / kChunksK;
-  static constexpr int kDV = D / 32;                  // d values per thread in the V transpose (4 keys x kDV d)
-  static constexpr int kVW = kDV / 2;                 // dwords per V load
+  static constexpr int kLoads = kBK * kChunks / kThreads;  // 16-byte loads per thread and tile (2 or 1)
+  static constexpr int kRowStep = kThreads / kChunks;
   static constexpr int kPitchO = D * 2 + 16;          // epilogue row pitch
   static constexpr int kLdsTiles = kNumKBuf * kBytesK + kNumVBuf * kBytesV;
   static constexpr int kLdsEpilogue = kWaves * 32 * kPitchO;
   static constexpr int kLdsBytes = kLdsTiles > kLdsEpilogue ? kLdsTiles : kLdsEpilogue;
 };
 
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+// Transposing LDS read (ds_read_b64_tr_b16).  Within each block of 16 lanes the 16 x 4 matrix of
+// 16-bit elements [source lane][element] is read as 4 rows of 16 (source lane 4j+m supplies
+// row j, columns 4m..4m+3) and lane i receives column i: element j = row j, column i.
+__device__ __forceinline__ s16x4 lds_read_tr(const uint8_t* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (s16x4 __attribute__((address_space(3)))*)(p));
+}
+
 template <int D>
 __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a) {
   using T = Tile<D>;
-  using VLoad = typename VecOf<T::kVW>::type;
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
   // ---- which (job, batch, head, query tile) ------------------------------------------
@@ -271,26 +263,20 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   ld_next_chunk();
   cp_next_chunk();
 
-  // thread -> K tile elements: 16-byte chunk kc of rows kr0 + i*kRowStepK
-  const int kc = tid % T::kChunksK;
-  const int kr0 = tid / T::kChunksK;
-  // thread -> V tile elements: keys 4*vkg..+3, d kDV*vdg..+kDV-1.  A quarter wavefront covers
-  // the 16 key groups of one d group, so the transposed 8-byte LDS writes fill whole rows.
-  const int vkg = tid & 15;
-  const int vdg = tid >> 4;
+  // thread -> tile elements, the same for K and V: 16-byte chunk kc of rows kr0 + i*kRowStep
+  const int kc = tid % T::kChunks;
+  const int kr0 = tid / T::kChunks;
   const uint32_t row_bytes = (uint32_t)a.kv_ss * 2u;
   // byte offsets from the tile's first key, loop invariant
-  uint32_t koff[T::kLoadsK], voff[4];
+  uint32_t koff[T::kLoads];
 #pragma unroll
-  for (int i = 0; i < T::kLoadsK; ++i) koff[i] = (uint32_t)(kr0 + i * T::kRowStepK) * row_bytes + 16u * kc;
-#pragma unroll
-  for (int r = 0; r < 4; ++r) voff[r] = (uint32_t)(4 * vkg + r) * row_bytes + (uint32_t)(T::kDV * 2 * vdg);
+  for (int i = 0; i < T::kLoads; ++i) koff[i] = (uint32_t)(kr0 + i * T::kRowStep) * row_bytes + 16u * kc;
 
   // Two register sets: the loads of a tile are issued TWO iterations before its LDS fill, so
   // that a first-touch miss all the way to HBM (the workgroup that leads on its XCD takes one
   // on every tile) is still hidden.  Tile X of a group uses set (X - pf) & 1.
-  u32x4 kreg[2][T::kLoadsK];
-  VLoad vreg[2][4];
+  u32x4 kreg[2][T::kLoads];
+  u32x4 vreg[2][T::kLoads];
 
   const int64_t tile_bytes = (int64_t)kBK * row_bytes;
   // Loads this thread's share of the tile under the load cursor into registers and moves the
@@ -306,35 +292,29 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     const __amdgpu_buffer_rsrc_t rv =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(ld_v), 0, (int)valid, kRsrcFlags);
 #pragma unroll
-    for (int i = 0; i < T::kLoadsK; ++i) kreg[kSet][i] = __builtin_amdgcn_raw_buffer_load_b128(rk, (int)koff[i], 0, 0);
+    for (int i = 0; i < T::kLoads; ++i) kreg[kSet][i] = __builtin_amdgcn_raw_buffer_load_b128(rk, (int)koff[i], 0, 0);
 #pragma unroll
-    for (int r = 0; r < 4; ++r) vreg[kSet][r] = buffer_load_v<T::kVW>(rv, (int)voff[r]);
+    for (int i = 0; i < T::kLoads; ++i) vreg[kSet][i] = __builtin_amdgcn_raw_buffer_load_b128(rv, (int)koff[i], 0, 0);
     ld_left -= kBK;
     ld_k += tile_bytes;
     ld_v += tile_bytes;
     if (ld_left <= 0) ld_next_chunk();
   };
 
-  // LDS write addresses of this thread within a K / V buffer
+  // LDS write addresses of this thread within a K / V buffer (V is stored as it comes, [key][d];
+  // the transposition the second MFMA needs is done by the transposing LDS read)
   const int kst = kr0 * T::kPitchK + 16 * kc;
-  const int vst = (T::kDV * vdg) * T::kPitchV + 8 * vkg;
+  const int vst = kr0 * T::kPitchV + 16 * kc;
   auto store_tile = [&](int tile, auto set_tag) {
     constexpr int kSet = decltype(set_tag)::value;
     uint8_t* kbuf = lds + (tile % kNumKBuf) * T::kBytesK;
     uint8_t* vbuf = lds + T::kOffV + (tile % kNumVBuf) * T::kBytesV;
 #pragma unroll
-    for (int i = 0; i < T::kLoadsK; ++i)
-      *reinterpret_cast<u32x4*>(kbuf + kst + i * T::kRowStepK * T::kPitchK) = kreg[kSet][i];
-    // transpose 4 keys x kDV d -> kDV rows of 4 keys
+    for (int i = 0; i < T::kLoads; ++i)
+      *reinterpret_cast<u32x4*>(kbuf + kst + i * T::kRowStep * T::kPitchK) = kreg[kSet][i];
 #pragma unroll
-    for (int jj = 0; jj < T::kDV; ++jj) {
-      const int w = jj >> 1;
-      const uint32_t sel = (jj & 1) ? 0x07060302u : 0x05040100u;
-      u32x2 o;
-      o.x = __builtin_amdgcn_perm(dword_of(vreg[kSet][1], w), dword_of(vreg[kSet][0], w), sel);
-      o.y = __builtin_amdgcn_perm(dword_of(vreg[kSet][3], w), dword_of(vreg[kSet][2], w), sel);
-      *reinterpret_cast<u32x2*>(vbuf + vst + jj * T::kPitchV) = o;
-    }
+    for (int i = 0; i < T::kLoads; ++i)
+      *reinterpret_cast<u32x4*>(vbuf + vst + i * T::kRowStep * T::kPitchV) = vreg[kSet][i];
   };
 
   // ---- accumulators ---------------------------------------------------------------------
@@ -349,7 +329,9 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
 
   // operand read addresses of this lane within a K / V buffer
   const int kld = key_of_row(col) * T::kPitchK + 16 * hh;
-  const int vld = T::kOffV + col * T::kPitchV + 16 * hh;
+  // V operand: this lane is source lane 4j+m of its 16-lane block and supplies keys 8*hh + j,
+  // d columns 16*(block parity) + 4m .. +3 of the fragment
+  const int vld = T::kOffV + (8 * hh + ((lane & 15) >> 2)) * T::kPitchV + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
 
   f32x16 s_acc[2];       // S^T of the tile whose softmax comes next
   bf16x8 p_frag[2][2];   // P^T of the tile whose P V product comes next
@@ -383,8 +365,13 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     const uint8_t* kl = lds + kld + ((tile + 1) % kNumKBuf) * T::kBytesK;
     auto frag = [&](int i) -> bf16x8 {
       if (i < kPV) {
+        // 8 consecutive keys of one d column = two transposing reads of 4 keys each
         const int db = i >> 2, kb = (i >> 1) & 1, half = i & 1;
-        return *reinterpret_cast<const bf16x8*>(vl + db * 32 * T::kPitchV + 64 * kb + 32 * half);
+        const uint8_t* p = vl + (32 * kb + 16 * half) * T::kPitchV + db * 64;
+        const s16x4 lo = lds_read_tr(p);
+        const s16x4 hi = lds_read_tr(p + 4 * T::kPitchV);
+        const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        return __builtin_bit_cast(bf16x8, both);
       }
       const int j = i - kPV;
       const int kb = j / (D / 16), sidx = j % (D / 16);
@@ -413,10 +400,17 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
         }
       }
     }
-    // pin the order: kRing reads up front, then one read behind every MFMA
-    __builtin_amdgcn_sched_group_barrier(0x100, kRing, 0);
+    // pin the order: the reads of kRing fragments up front (a V fragment is two reads), then the
+    // reads of one more fragment behind every MFMA
+    static_assert(kRing <= kPV, "the prefill is assumed to consist of V fragments");
+    __builtin_amdgcn_sched_group_barrier(0x100, 2 * kRing, 0);
 #pragma unroll
-    for (int i = 0; i < kFrags - kRing; ++i) {
+    for (int i = 0; i < kPV - kRing; ++i) {   // MFMAs whose refill is a V fragment
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < kQK; ++i) {           // MFMAs whose refill is a K fragment
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
