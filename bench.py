@@ -227,6 +227,21 @@ def main():
     k3l_ms = time_kernel(lambda: _hip.cache_load(out_s, lse_s, torch.float32, True), reps)
     k3l_gbs = rows * ((2 * D + 4) + (4 * D + 4)) / (k3l_ms * 1e-3) / 1e9
 
+    # producer step of the callers: RMSNorm + interleaved RoPE of K over the whole KV sequence, read in
+    # place from a fused QKV projection ("B L (K H D)"), written as the [B,S,H,D] bf16 the attention reads
+    S_all = int(sum(lens))
+    qkv = torch.randn(B, S_all, 3, H, D, device=dev, dtype=torch.bfloat16)
+    ang = torch.rand(S_all, D // 2, device=dev) * 6.28
+    p_cos = ang.cos().repeat_interleave(2, -1).contiguous()
+    p_sin = ang.sin().repeat_interleave(2, -1).contiguous()
+    p_w = torch.ones(D, device=dev)
+    p_out = torch.empty(B, S_all, H, D, dtype=torch.bfloat16, device=dev)
+    kp_ms = time_kernel(lambda: _hip.qk_norm_rope(qkv[:, :, 1], norm=_hip.DT_NORM_RMS, weight=p_w, rope=_hip.DT_ROPE_INTERLEAVED,
+                                                  cos=p_cos, sin=p_sin, out=p_out), reps, warm=10)
+    kp_bytes = B * S_all * H * D * 4 + S_all * D * 8
+    kp_gbs = kp_bytes / (kp_ms * 1e-3) / 1e9
+    del qkv, ang, p_cos, p_sin, p_out
+
     dmask = torch.from_numpy(mask).to(dev)
     k4_ms = time_kernel(lambda: _hip.build_schedule_table(dmask, diag), reps)
     # a plain copy of known size: the yardstick the profiler's FETCH_SIZE / WRITE_SIZE counters are scaled by
@@ -264,6 +279,10 @@ def main():
         "cache_gbs": {"store_fp32_to_slot": round(k3s_gbs, 1), "store_bf16_to_slot": round(k3c_gbs, 1),
                       "load_slot_to_fp32": round(k3l_gbs, 1), "peak": PEAK_HBM_GBS,
                       "frac_store_bf16": round(k3c_gbs / PEAK_HBM_GBS, 4), "frac_load": round(k3l_gbs / PEAK_HBM_GBS, 4)},
+        "producer": {"kernel": "qk_norm_rope_kernel<%d>" % D, "bound": "hbm", "achieved": round(kp_gbs, 1),
+                     "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(kp_gbs / PEAK_HBM_GBS, 4),
+                     "launch_us": round(kp_ms * 1e3, 2), "bytes_per_launch": kp_bytes, "tokens": S_all,
+                     "what": "RMSNorm + interleaved RoPE of K over the whole KV sequence, strided read from a fused QKV tensor"},
         "schedule_builder_us": round(k4_ms * 1e3, 2),
         "plain_copy_1GiB_gbs": round(copy_gbs, 1),
     }

@@ -17,6 +17,9 @@ LIB_PATH = Path(__file__).resolve().parent / "lib" / "libditango_hip.so"
 
 DT_BF16, DT_FP32 = 0, 1
 DT_LSE_BHS, DT_LSE_BSH = 0, 1
+DT_NORM_NONE, DT_NORM_RMS, DT_NORM_LAYER = 0, 1, 2
+DT_ROPE_NONE, DT_ROPE_INTERLEAVED, DT_ROPE_HALVES = 0, 1, 2
+DT_ROUND_NORM_BF16, DT_ROUND_ROPE_BF16 = 1, 2
 DT_MAX_CHUNKS = 40
 DT_MAX_JOBS = 40
 DT_MAX_JOB_ENTRIES = 64
@@ -48,6 +51,9 @@ _SIGNATURES = {
     "dt_build_schedule": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp, c_vp]),
     "dt_build_schedule_table": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp, c_vp]),
     "dt_rel_l1_sums": (ctypes.c_int, [c_vp, c_vp, c_i64, c_vp, c_vp]),
+    "dt_qk_norm_rope": (ctypes.c_int, [c_vp, c_i64, c_i64, c_i64, c_vp, c_i32, c_i32, c_i32, c_i32,
+                                       c_i32, c_vp, c_vp, c_f32, c_i32, c_vp, c_vp, c_i64, c_i32, c_i32,
+                                       _P(c_i32), c_i32, c_i32, c_vp]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
@@ -374,3 +380,44 @@ def rel_l1_sums(a: torch.Tensor, b: torch.Tensor, sums: Optional[torch.Tensor] =
     rc = lib.dt_rel_l1_sums(a.data_ptr(), b.data_ptr(), a.numel(), sums.data_ptr(), _stream())
     _check(rc, "dt_rel_l1_sums")
     return sums
+
+
+def qk_norm_rope(x: torch.Tensor, *, norm: int = DT_NORM_NONE, weight: Optional[torch.Tensor] = None,
+                 bias: Optional[torch.Tensor] = None, eps: float = 1e-6, rope: int = DT_ROPE_NONE,
+                 cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None,
+                 rope_begin: int = 0, rope_end: Optional[int] = None, sections: Sequence[int] = (),
+                 rounding: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x bf16 ``[B,S,H,D]`` (any strides with a contiguous last dimension) -> bf16 ``[B,S,H,D]`` contiguous,
+    normalised over D and rotated on token rows ``[rope_begin, rope_end)``.  cos/sin are fp32
+    ``[rope_end-rope_begin, D]`` or ``[B, rope_end-rope_begin, D]``."""
+    lib = load_library()
+    _require(x.is_cuda and x.dtype == torch.bfloat16 and x.dim() == 4 and x.stride(3) == 1, "x must be bf16 [B,S,H,D] on the GPU")
+    B, S, H, D = x.shape
+    if out is None:
+        out = torch.empty((B, S, H, D), dtype=torch.bfloat16, device=x.device)
+    _require(out.is_cuda and out.dtype == torch.bfloat16 and out.is_contiguous() and tuple(out.shape) == (B, S, H, D),
+             "out must be a contiguous bf16 [B,S,H,D]")
+    for name, t in (("weight", weight), ("bias", bias)):
+        _require(t is None or (t.is_cuda and t.dtype == torch.float32 and t.is_contiguous() and t.numel() == D),
+                 f"{name} must be fp32 [D] on the GPU")
+    if rope_end is None:
+        rope_end = S
+    tab_sb = 0
+    if rope != DT_ROPE_NONE and rope_end > rope_begin:
+        rows = rope_end - rope_begin
+        for name, t in (("cos", cos), ("sin", sin)):
+            _require(t is not None and t.is_cuda and t.dtype == torch.float32 and t.is_contiguous()
+                     and t.shape[-1] == D and t.shape[-2] == rows and t.dim() in (2, 3),
+                     f"{name} must be a contiguous fp32 [rows, D] or [B, rows, D] table on the GPU")
+        _require(cos.shape == sin.shape, "cos and sin must have one shape")
+        if cos.dim() == 3:
+            _require(cos.shape[0] == B, "batched tables need B leading entries")
+            tab_sb = rows * D
+    sec = (c_i32 * max(1, len(sections)))(*[int(v) for v in sections])
+    rc = lib.dt_qk_norm_rope(x.data_ptr(), x.stride(0), x.stride(1), x.stride(2), out.data_ptr(), B, S, H, D,
+                             int(norm), weight.data_ptr() if weight is not None else None,
+                             bias.data_ptr() if bias is not None else None, float(eps), int(rope),
+                             cos.data_ptr() if cos is not None else None, sin.data_ptr() if sin is not None else None,
+                             tab_sb, int(rope_begin), int(rope_end), sec, len(sections), int(rounding), _stream())
+    _check(rc, "dt_qk_norm_rope")
+    return out

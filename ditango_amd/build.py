@@ -18,7 +18,7 @@ ROOT = PKG.parent
 CSRC = PKG / "csrc"
 LIB_DIR = PKG / "lib"
 LIB_PATH = LIB_DIR / "libditango_hip.so"
-SOURCES = ["attn_fwd.hip", "state_ops.hip", "capi.hip"]
+SOURCES = ["attn_fwd.hip", "state_ops.hip", "producer.hip", "capi.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 COMMON = [

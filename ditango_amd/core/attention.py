@@ -169,6 +169,10 @@ class proAttention:
         self.dry_run = dry_run  # plan and book-keep only (host tests of the schedule); computes nothing
         self.last_plan: Optional[CallPlan] = None
         self.last_lse: Optional[torch.Tensor] = None  # merged lse of the last call, fp32 [B,S,H,1]
+        # dtype of the returned tensor.  The reference returns fp32 and every caller casts right away
+        # (attention_processor.py:80, step/attentions.py:98); torch.bfloat16 here lets the merge kernel
+        # write the bf16 the out-projection consumes: half the result bytes and no separate cast pass.
+        self.out_dtype = torch.float32
         self._segments = None  # (cu_seqlens_q, chunk -> cu_seqlens_kv) while a variable-length call runs
         if self.layer_id == 0:
             logger.info(f"R{self.global_rank}L{layer_id} | cached block attention on HIP kernels (gfx950)")
@@ -300,7 +304,7 @@ class proAttention:
                 self.cache.store_block(job.store_slot, o, l)  # :207-211
             merge_outs.append(o)
             merge_lses.append(l)
-        out, lse = _hip.merge_states(merge_outs, merge_lses, dst_dtype=torch.float32, dst_lse_bsh=True)
+        out, lse = _hip.merge_states(merge_outs, merge_lses, dst_dtype=self.out_dtype, dst_lse_bsh=True)
         self.last_lse = lse
         return out
 
@@ -337,7 +341,7 @@ class proAttention:
                     cache.arena_valid[c] = True
                 outs.append(cache.arena_out[c])
                 lses.append(cache.arena_lse[c])
-        out, lse = _hip.merge_states(outs, lses, dst_dtype=torch.float32, dst_lse_bsh=True)
+        out, lse = _hip.merge_states(outs, lses, dst_dtype=self.out_dtype, dst_lse_bsh=True)
         self.last_lse = lse
         rm.record_out_redundancy(timestep=t, layer_id=l, curr_out=out)
         return out

@@ -40,6 +40,17 @@ extern "C" {
 #define DT_LSE_BHS 0
 #define DT_LSE_BSH 1
 
+#define DT_NORM_NONE 0
+#define DT_NORM_RMS 1    /* x * rsqrt(mean(x^2) + eps) * weight */
+#define DT_NORM_LAYER 2  /* (x - mean) * rsqrt(var + eps) * weight + bias */
+
+#define DT_ROPE_NONE 0
+#define DT_ROPE_INTERLEAVED 1 /* pairs (2i, 2i+1) rotate together */
+#define DT_ROPE_HALVES 2      /* element d pairs with d +- half of its section ("rotate_half") */
+
+#define DT_ROUND_NORM_BF16 1 /* round to bf16 where the callers' bf16 norm modules do */
+#define DT_ROUND_ROPE_BF16 2 /* RoPE products and their sum each rounded to bf16 */
+
 #define DT_MAX_CHUNKS 40       /* KV chunks one launch can address */
 #define DT_MAX_JOBS 40         /* attention states one launch can produce */
 #define DT_MAX_JOB_ENTRIES 64  /* total chunk references over all jobs of a launch */
@@ -184,6 +195,38 @@ int dt_build_schedule_table(const uint8_t* mask, int32_t T, int32_t L, int32_t C
  * (core/redundancy_map.py:174-197).  a, b are fp32, n elements.
  */
 int dt_rel_l1_sums(const float* a, const float* b, int64_t n, double* sums, void* stream);
+
+/*
+ * Producer side of an attention call: normalise every head row of x over D, apply the
+ * rotary position embedding to the token rows [rope_begin, rope_end) and write the result
+ * as bf16 [B,S,H,D] contiguous, the layout the attention entry points read -- one pass over
+ * HBM.  Replaces the eager chains in front of proAttention.attn / varlen_attn at
+ *   executor/cogvideox/attention_processor.py:55-71 (attn.norm_q / norm_k = LayerNorm over D;
+ *     apply_rotary_emb on query[:, :, text_seqlen:] only; transpose + contiguous),
+ *   executor/hunyuanvideo/hunyuan_transformer.py:177-191 (RMSNorm over D; apply_rotary_emb with
+ *     interleaved pairs),
+ *   executor/step/blocks.py:66-75 with executor/step/rope.py:13-90 (RMSNorm; rotate_half RoPE
+ *     applied separately to the sections [64,32,32] of D).
+ * x is bf16 with element strides (x_stride_b, x_stride_s, x_stride_h) and a contiguous last
+ * dimension, so q, k or v can be read in place out of a fused QKV projection; with
+ * norm = rope = 0 the call is the strided-to-contiguous copy of v.  y may alias x when x is
+ * already contiguous [B,S,H,D].
+ * weight / bias: fp32 [D] or NULL (1 / 0).  cos / sin: fp32 [rope_end - rope_begin, D], row
+ * s - rope_begin belongs to token s; batch b reads its tables at + b * table_stride_b
+ * elements (0 = shared).  out[d] = x[d] * cos[d] + rot(x)[d] * sin[d] with
+ *   DT_ROPE_INTERLEAVED: rot(x)[2i] = -x[2i+1], rot(x)[2i+1] = x[2i];
+ *   DT_ROPE_HALVES: inside each section [lo, hi): rot(x)[d] = -x[d + (hi-lo)/2] in the first
+ *     half, x[d - (hi-lo)/2] in the second.  sections (HOST array, n_sections <= 3, each a
+ *     multiple of 16, summing to D; n_sections = 0 means one section of D).
+ * rounding = 0 computes in fp32 and rounds once on the way out; the DT_ROUND_* bits reproduce
+ * the intermediate bf16 roundings of the callers' eager modules.
+ */
+int dt_qk_norm_rope(const void* x, int64_t x_stride_b, int64_t x_stride_s, int64_t x_stride_h, void* y,
+                    int32_t B, int32_t S, int32_t H, int32_t D,
+                    int32_t norm, const float* weight, const float* bias, float eps,
+                    int32_t rope, const float* cos, const float* sin, int64_t table_stride_b,
+                    int32_t rope_begin, int32_t rope_end, const int32_t* sections, int32_t n_sections,
+                    int32_t rounding, void* stream);
 
 #ifdef __cplusplus
 }

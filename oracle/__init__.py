@@ -18,6 +18,10 @@ Modules (each function cites the reference file:line it restates):
   (``utils.py:202-267``).
 * ``mask_schedule``   the explicit per-chunk mask mode (a generalisation the
   reference cannot express; semantics documented in that module).
+* ``producer``        QK normalisation + rotary embedding in front of the
+  attention call (``executor/cogvideox/attention_processor.py:55-71``,
+  ``executor/hunyuanvideo/hunyuan_transformer.py:177-191``,
+  ``executor/step/blocks.py:66-75``, ``executor/step/rope.py:13-90``).
 
 Pinning status (what fixes each function besides "it restates the source"):
 
@@ -38,4 +42,11 @@ Pinning status (what fixes each function besides "it restates the source"):
   ``_refine_divider_map`` and by the divider histograms an independent
   restatement produced; a golden map produced by running the reference itself
   does not exist, so that part is **parity unpinned** beyond those checks.
+* producer: RMSNorm / LayerNorm pinned against ``torch.nn.functional.rms_norm``
+  / ``layer_norm``; interleaved RoPE against complex multiplication
+  (``torch.view_as_complex``); rotate-half RoPE against explicit 2x2 rotations,
+  norm preservation and the relative-position property; the Step-Video tables
+  against a direct evaluation of cos/sin at the mesh positions.  Where the
+  third-party modules (diffusers 0.31.0, hyvideo, stepvideo) place their
+  intermediate bf16 roundings is **parity unpinned**.
 """

@@ -276,3 +276,41 @@ def test_profiling_mode_records_rel_l1(env):
     assert rm.redundancy_map[0, 0] == 0
     for t in (1, 2):
         assert abs(rm.redundancy_map[t, 0].item() - om.rel_l1(outs[t], outs[t - 1])) < 1e-5
+
+
+def test_bf16_result_and_producer_feed_the_attention(env):
+    """The caller-side chain in one piece: q/k/v read in place from a fused QKV projection, RMSNorm +
+    RoPE by dt_qk_norm_rope, cached block attention, result written as bf16 by the merge
+    (out_dtype); against the oracle's norm + RoPE + full attention on the same inputs."""
+    from oracle import producer as P
+    from ditango_amd.core.attention import proAttention
+    from ditango_amd.core.parallel_state import get_usp_group
+    from ditango_amd.producer import prepare_qk
+    from ditango_amd.utils import update_timestep
+
+    C, B, H, D, Sq = 4, 1, 5, 128, 96
+    rm = env(C, 0, 2, 1)
+    rm.set_chunk_mask(np.zeros((2, 1, C), dtype=np.uint8), diag=0)
+    g = torch.Generator().manual_seed(31)
+    qkv = torch.randn(B, C * Sq, 3, H, D, generator=g).bfloat16()
+    wq, wk = torch.rand(D, generator=g) + 0.5, torch.rand(D, generator=g) + 0.5
+    th = torch.rand(C * Sq, D // 2, generator=g) * 6.28
+    cos, sin = th.cos().repeat_interleave(2, -1), th.sin().repeat_interleave(2, -1)
+    # oracle
+    qn = P.qk_norm_rope(qkv[:, :, 0], P.NORM_RMS, wq, None, 1e-6, P.ROPE_INTERLEAVED, cos, sin).bfloat16()
+    kn = P.qk_norm_rope(qkv[:, :, 1], P.NORM_RMS, wk, None, 1e-6, P.ROPE_INTERLEAVED, cos, sin).bfloat16()
+    ref_out, ref_lse = om.chunk_attention(qn[:, :Sq], kn, qkv[:, :, 2])
+    # product
+    dev = qkv.cuda()
+    qd = prepare_qk(dev[:, :, 0], norm="rms", weight=wq, rope="interleaved", freqs_cis=(cos, sin))
+    kd = prepare_qk(dev[:, :, 1], norm="rms", weight=wk, rope="interleaved", freqs_cis=(cos, sin))
+    vd = prepare_qk(dev[:, :, 2])
+    group = get_usp_group()
+    group.set_kv_chunks(list(kd.split(Sq, dim=1)), list(vd.split(Sq, dim=1)))
+    layer = proAttention(0, group)
+    layer.out_dtype = torch.bfloat16
+    update_timestep(0)
+    out = layer.attn(qd[:, :Sq], kd[:, :Sq], vd[:, :Sq])
+    torch.cuda.synchronize()
+    assert out.dtype == torch.bfloat16 and out.shape == (B, Sq, H, D)
+    _cmp(out, layer.last_lse, ref_out, ref_lse, "producer + attention + bf16 result")
