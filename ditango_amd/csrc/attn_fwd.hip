@@ -286,7 +286,12 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   // -inf; zero V rows add nothing).
   auto load_tile = [&](auto set_tag) {
     constexpr int kSet = decltype(set_tag)::value;
-    const uint32_t valid = (uint32_t)(ld_left - 1) * row_bytes + (uint32_t)(D * 2);
+    // Past the last tile the loads are still issued, against an empty descriptor (they return
+    // zeros without touching memory): with the same number of loads in every iteration the
+    // counter the LDS fill waits on is static, and a fill waits for ITS tile only, not for the
+    // loads issued one iteration later.
+    const bool have = __builtin_expect(ld_seg < seg_end, 1);
+    const uint32_t valid = have ? (uint32_t)(ld_left - 1) * row_bytes + (uint32_t)(D * 2) : 0u;
     const __amdgpu_buffer_rsrc_t rk =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(ld_k), 0, (int)valid, kRsrcFlags);
     const __amdgpu_buffer_rsrc_t rv =
@@ -295,10 +300,12 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     for (int i = 0; i < T::kLoads; ++i) kreg[kSet][i] = __builtin_amdgcn_raw_buffer_load_b128(rk, (int)koff[i], 0, 0);
 #pragma unroll
     for (int i = 0; i < T::kLoads; ++i) vreg[kSet][i] = __builtin_amdgcn_raw_buffer_load_b128(rv, (int)koff[i], 0, 0);
-    ld_left -= kBK;
-    ld_k += tile_bytes;
-    ld_v += tile_bytes;
-    if (ld_left <= 0) ld_next_chunk();
+    if (have) {
+      ld_left -= kBK;
+      ld_k += tile_bytes;
+      ld_v += tile_bytes;
+      if (__builtin_expect(ld_left <= 0, 0)) ld_next_chunk();
+    }
   };
 
   // LDS write addresses of this thread within a K / V buffer (V is stored as it comes, [key][d];
@@ -422,34 +429,17 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   using Set0 = std::integral_constant<int, 0>;
   using Set1 = std::integral_constant<int, 1>;
   const int pf = 1 + group;  // how many tiles ahead of its softmax a group fills LDS
-  int n_issued = 0;          // tiles whose loads this thread has issued
-  int n_loaded = 0;          // tiles this thread has written its share of
-  if (n_tiles > 0) {
-    load_tile(Set0{});
-    store_tile(0, Set0{});
-    n_issued = n_loaded = 1;
-  }
-  if (group == 1 && n_tiles > 1) {
-    load_tile(Set0{});
-    n_issued = 2;
-  }
+  load_tile(Set0{});
+  store_tile(0, Set0{});
+  if (group == 1) load_tile(Set0{});
   phase_barrier();
   if (group == 1) {
-    if (n_tiles > 1) {
-      store_tile(1, Set0{});
-      n_loaded = 2;
-    }
+    store_tile(1, Set0{});
     phase_barrier();
   }
   // first matrix phase: fetch two tiles ahead (sets 0 and 1), scores of tile 0
-  if (n_issued < n_tiles) {
-    load_tile(Set0{});
-    ++n_issued;
-  }
-  if (n_issued < n_tiles) {
-    load_tile(Set1{});
-    ++n_issued;
-  }
+  load_tile(Set0{});
+  load_tile(Set1{});
   if (n_tiles > 0) {
     qk_only(0);
     cp_valid = cp_left;
@@ -464,11 +454,8 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     // ======== vector phase: LDS fill of a fetched tile, online softmax of tile t ========
     // The fill goes first: its registers were loaded two iterations ago, and the latency of
     // the LDS writes (which compete with the other group's operand reads) hides behind the softmax.
-    if (n_loaded < n_issued) {
-      store_tile(n_loaded, set_tag);
-      ++n_loaded;
-    }
-    if (cp_valid < kBK) {
+    store_tile(t + pf, set_tag);
+    if (__builtin_expect(cp_valid < kBK, 0)) {
       // the empty asm has side effects as far as the compiler knows, which keeps this a real
       // branch: otherwise the selects below are hoisted out and run for every tile
       asm volatile("" ::: "memory");
@@ -502,7 +489,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
         p_frag[kb][r >> 3][r & 7] = pb.x;
         p_frag[kb][r >> 3][(r & 7) + 1] = pb.y;
       }
-    if (__any(!(rs0 + rs1 <= kSumLimit))) {
+    if (__builtin_expect(__any(!(rs0 + rs1 <= kSumLimit)), 0)) {
       float mx = s_acc[0][0];
 #pragma unroll
       for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s_acc[0][r]);
@@ -539,19 +526,19 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     phase_barrier_after_vector(p_frag);
 
     // ======== matrix phase: fetch ahead, O^T += V^T P^T (tile t), S^T = K Q^T (tile t+1) ========
-    if (n_issued < n_tiles) {
-      load_tile(set_tag);
-      ++n_issued;
-    }
+    load_tile(set_tag);
     matrix_phase(t);
     cp_valid = cp_left;
     cp_left -= kBK;
     if (cp_left <= 0) cp_next_chunk();
     phase_barrier_after_matrix(s_acc, o_acc);
   };
-  for (int t = 0; t < n_tiles; t += 2) {
+  // Iterations come in pairs (one per register set); an odd tile count is rounded up with a tile
+  // that has no keys: its loads hit the empty descriptor, its scores are masked, it adds zeros.
+  const int n_iter = (n_tiles + 1) & ~1;
+  for (int t = 0; t < n_iter; t += 2) {
     iteration(t, Set0{});
-    if (t + 1 < n_tiles) iteration(t + 1, Set1{});
+    iteration(t + 1, Set1{});
   }
   // the leading group waits out the phase it is ahead
   if (kStagger && group == 0) phase_barrier();
