@@ -237,7 +237,7 @@ def main():
     p_w = torch.ones(D, device=dev)
     p_out = torch.empty(B, S_all, H, D, dtype=torch.bfloat16, device=dev)
     kp_ms = time_kernel(lambda: _hip.qk_norm_rope(qkv[:, :, 1], norm=_hip.DT_NORM_RMS, weight=p_w, rope=_hip.DT_ROPE_INTERLEAVED,
-                                                  cos=p_cos, sin=p_sin, out=p_out), reps, warm=10)
+                                                  cos=p_cos, sin=p_sin, out=p_out), reps, warm=40)
     kp_bytes = B * S_all * H * D * 4 + S_all * D * 8
     kp_gbs = kp_bytes / (kp_ms * 1e-3) / 1e9
     del qkv, ang, p_cos, p_sin, p_out

@@ -62,6 +62,9 @@ constexpr int kBK = 64;           // keys per tile
 constexpr int kXcds = 8;
 constexpr int kNumKBuf = 2;
 constexpr int kNumVBuf = 3;
+#ifndef DT_RING
+#define DT_RING 4
+#endif
 // true: two groups of 4 wavefronts run one phase apart with a barrier after every phase;
 // false: all wavefronts in the same phase, one barrier per tile.
 #ifndef DT_STAGGER
@@ -366,27 +369,35 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   constexpr int kPV = D / 32 * 4;       // fragments of the P V product
   constexpr int kQK = 2 * (D / 16);     // fragments of the score product
   constexpr int kFrags = kPV + kQK;
-  constexpr int kRing = 4;
+  constexpr int kRing = DT_RING;
+  // The operand ring lives across the barrier in front of a matrix phase: its first kRing
+  // fragments (V fragments of a tile completed at least a phase ago) are read at the END of the
+  // preceding vector phase, so their LDS latency passes while the wavefront waits at the barrier
+  // instead of in front of the first MFMA.
+  bf16x8 ring[kRing];
+  auto v_frag = [&](const uint8_t* vl, int i) __attribute__((always_inline)) -> bf16x8 {
+    // 8 consecutive keys of one d column = two transposing reads of 4 keys each
+    const int db = i >> 2, kb = (i >> 1) & 1, half = i & 1;
+    const uint8_t* p = vl + (32 * kb + 16 * half) * T::kPitchV + db * 64;
+    const s16x4 lo = lds_read_tr(p);
+    const s16x4 hi = lds_read_tr(p + 4 * T::kPitchV);
+    const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(bf16x8, both);
+  };
+  auto ring_prefill = [&](int tile) __attribute__((always_inline)) {
+    const uint8_t* vl = lds + vld + (tile % kNumVBuf) * T::kBytesV;
+#pragma unroll
+    for (int i = 0; i < kRing; ++i) ring[i] = v_frag(vl, i);
+  };
   auto matrix_phase = [&](int tile) {
     const uint8_t* vl = lds + vld + (tile % kNumVBuf) * T::kBytesV;
     const uint8_t* kl = lds + kld + ((tile + 1) % kNumKBuf) * T::kBytesK;
     auto frag = [&](int i) -> bf16x8 {
-      if (i < kPV) {
-        // 8 consecutive keys of one d column = two transposing reads of 4 keys each
-        const int db = i >> 2, kb = (i >> 1) & 1, half = i & 1;
-        const uint8_t* p = vl + (32 * kb + 16 * half) * T::kPitchV + db * 64;
-        const s16x4 lo = lds_read_tr(p);
-        const s16x4 hi = lds_read_tr(p + 4 * T::kPitchV);
-        const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        return __builtin_bit_cast(bf16x8, both);
-      }
+      if (i < kPV) return v_frag(vl, i);
       const int j = i - kPV;
       const int kb = j / (D / 16), sidx = j % (D / 16);
       return *reinterpret_cast<const bf16x8*>(kl + kb * 32 * T::kPitchK + 32 * sidx);
     };
-    bf16x8 ring[kRing];
-#pragma unroll
-    for (int i = 0; i < kRing; ++i) ring[i] = frag(i);
 #pragma unroll
     for (int i = 0; i < kFrags; ++i) {
       const bf16x8 cur = ring[i % kRing];
@@ -410,7 +421,6 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     // pin the order: the reads of kRing fragments up front (a V fragment is two reads), then the
     // reads of one more fragment behind every MFMA
     static_assert(kRing <= kPV, "the prefill is assumed to consist of V fragments");
-    __builtin_amdgcn_sched_group_barrier(0x100, 2 * kRing, 0);
 #pragma unroll
     for (int i = 0; i < kPV - kRing; ++i) {   // MFMAs whose refill is a V fragment
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
@@ -523,6 +533,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
         }
     }
     l_run += rs0 + rs1;
+    ring_prefill(t);
     phase_barrier_after_vector(p_frag);
 
     // ======== matrix phase: fetch ahead, O^T += V^T P^T (tile t), S^T = K Q^T (tile t+1) ========
