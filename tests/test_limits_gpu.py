@@ -1,0 +1,113 @@
+"""The per-launch limits of the C ABI (40 chunks, 40 states, 64 chunk references, 40-way merge),
+the splitting of larger requests on the host side, tile counts around the pairing of iterations,
+and the error behaviour at the boundary (return code + message, never a launch)."""
+import ctypes
+
+import pytest
+import torch
+
+from oracle import attention_math as om
+
+pytestmark = pytest.mark.gpu
+
+OUT_TOL, LSE_TOL = 2e-2, 1e-3
+
+
+def _check(out, lse, ref_out, ref_lse, what):
+    err = (out.float().cpu() - ref_out).abs().max().item()
+    lerr = (lse.cpu() - ref_lse).abs().max().item()
+    assert err <= OUT_TOL and lerr <= LSE_TOL, f"{what}: out {err:.3e} lse {lerr:.3e}"
+
+
+def _rand(shape, g):
+    return torch.randn(*shape, generator=g).bfloat16()
+
+
+def test_forty_chunks_in_one_job(hip):
+    B, Sq, H, D, C = 1, 70, 2, 128, hip.DT_MAX_CHUNKS
+    g = torch.Generator().manual_seed(1)
+    lens = [1 + (7 * i) % 50 for i in range(C)]
+    q = _rand((B, Sq, H, D), g)
+    ks = [_rand((B, n, H, D), g) for n in lens]
+    vs = [_rand((B, n, H, D), g) for n in lens]
+    ref_out, ref_lse = om.full_attention(q, ks, vs)
+    table = hip.ChunkTable([k.cuda() for k in ks], [v.cuda() for v in vs])
+    out = torch.empty(B, Sq, H, D, dtype=torch.bfloat16, device="cuda")
+    lse = torch.empty(B, H, Sq, dtype=torch.float32, device="cuda")
+    hip.attn_jobs_fwd(q.cuda(), table, [list(range(C))], [out], [lse])
+    torch.cuda.synchronize()
+    _check(out, lse, ref_out, ref_lse, "40 chunks, one job")
+    with pytest.raises(hip.DitangoHipError):
+        hip.ChunkTable([k.cuda() for k in ks] + [ks[0].cuda()], [v.cuda() for v in vs] + [vs[0].cuda()])
+
+
+def test_more_jobs_than_one_launch_holds(hip):
+    """45 single-chunk states and then jobs whose chunk references exceed 64: the binding splits launches."""
+    B, Sq, H, D, C = 1, 40, 1, 64, 9
+    g = torch.Generator().manual_seed(2)
+    q = _rand((B, Sq, H, D), g)
+    ks = [_rand((B, 30 + i, H, D), g) for i in range(C)]
+    vs = [_rand((B, 30 + i, H, D), g) for i in range(C)]
+    refs = [om.chunk_attention(q, k, v) for k, v in zip(ks, vs)]
+    table = hip.ChunkTable([k.cuda() for k in ks], [v.cuda() for v in vs])
+    dq = q.cuda()
+    jobs = [[j % C] for j in range(45)]
+    outs = [torch.empty(B, Sq, H, D, dtype=torch.bfloat16, device="cuda") for _ in jobs]
+    lses = [torch.empty(B, H, Sq, dtype=torch.float32, device="cuda") for _ in jobs]
+    hip.attn_jobs_fwd(dq, table, jobs, outs, lses)
+    torch.cuda.synchronize()
+    for j in range(45):
+        _check(outs[j], lses[j], *refs[j % C], f"job {j}")
+    # 12 jobs of 9 references each = 108 references > 64 per launch
+    jobs = [list(range(C)) for _ in range(12)]
+    full = om.full_attention(q, ks, vs)
+    hip.attn_jobs_fwd(dq, table, jobs, outs[:12], lses[:12])
+    torch.cuda.synchronize()
+    for j in range(12):
+        _check(outs[j], lses[j], *full, f"full job {j}")
+
+
+def test_forty_way_merge_and_its_limit(hip):
+    B, Sq, H, D, n = 1, 50, 2, 128, hip.DT_MAX_MERGE
+    g = torch.Generator().manual_seed(3)
+    outs = [_rand((B, Sq, H, D), g) for _ in range(n)]
+    lses = [torch.randn(B, H, Sq, generator=g) * 3 for _ in range(n)]
+    lses[7].fill_(float("-inf"))
+    ref_out, ref_lse = om.merge_states_closed_form([o.float() for o in outs], lses)
+    o, l = hip.merge_states([x.cuda() for x in outs], [x.cuda() for x in lses])
+    torch.cuda.synchronize()
+    assert (o.cpu() - ref_out).abs().max() <= 1e-5 and (l.cpu() - ref_lse).abs().max() <= 1e-5
+    with pytest.raises(hip.DitangoHipError):
+        hip.merge_states([x.cuda() for x in outs] + [outs[0].cuda()], [x.cuda() for x in lses] + [lses[0].cuda()])
+
+
+@pytest.mark.parametrize("Sk", [63, 64, 65, 127, 128, 129, 191, 193, 320])
+def test_tile_counts_around_the_iteration_pairs(hip, Sk):
+    """1, 2, 3, 4 and 5 key tiles, full and ragged: odd counts run one key-less tile extra."""
+    B, Sq, H, D = 1, 96, 1, 128
+    g = torch.Generator().manual_seed(Sk)
+    q, k, v = _rand((B, Sq, H, D), g), _rand((B, Sk, H, D), g), _rand((B, Sk, H, D), g)
+    ref = om.chunk_attention(q, k, v)
+    out, lse = hip.attn_chunk_fwd(q.cuda(), k.cuda(), v.cuda())
+    torch.cuda.synchronize()
+    _check(out, lse, *ref, f"Sk={Sk}")
+
+
+def test_c_abi_rejects_without_launching(hip):
+    lib = hip.load_library()
+    q = torch.zeros(1, 8, 1, 128, dtype=torch.bfloat16, device="cuda")
+    out = torch.full((1, 8, 1, 128), 7.0, dtype=torch.bfloat16, device="cuda")
+    lse = torch.zeros(1, 1, 8, device="cuda")
+
+    def call(qp, D=128, Sk=8, stride_s=128):
+        return lib.dt_attn_chunk_fwd(qp, q.data_ptr(), q.data_ptr(), out.data_ptr(), lse.data_ptr(), 1, 8, Sk, 1, D,
+                                     8 * 128, stride_s, 128, 8 * 128, 128, 128, ctypes.c_float(0.0), None)
+
+    assert call(q.data_ptr() + 2) == -1 and b"aligned" in lib.dt_last_error()       # DT_ERR_INVALID
+    assert call(q.data_ptr(), D=96) == -2 and b"96" in lib.dt_last_error()           # DT_ERR_UNSUPPORTED
+    assert call(q.data_ptr(), Sk=-1) == -1
+    assert call(q.data_ptr(), stride_s=130) == -1
+    assert call(None) == -1
+    torch.cuda.synchronize()
+    assert (out.float() == 7.0).all()                                                # nothing ran
+    assert call(q.data_ptr()) == 0
