@@ -464,6 +464,11 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     // ======== vector phase: LDS fill of a fetched tile, online softmax of tile t ========
     // The fill goes first: its registers were loaded two iterations ago, and the latency of
     // the LDS writes (which compete with the other group's operand reads) hides behind the softmax.
+    // The vector phase runs at raised wave priority: where the two wavefronts of a SIMD compete for
+    // the vector issue port, the one doing the softmax goes first.  With equal priorities the older
+    // wavefront wins in either role and the phases of the two groups come out unequal (measured
+    // 1.43k vs 1.24k cycles of vector work), so every other barrier waits for a squeezed softmax.
+    __builtin_amdgcn_s_setprio(1);
     store_tile(t + pf, set_tag);
     if (__builtin_expect(cp_valid < kBK, 0)) {
       // the empty asm has side effects as far as the compiler knows, which keeps this a real
@@ -537,6 +542,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     phase_barrier_after_vector(p_frag);
 
     // ======== matrix phase: fetch ahead, O^T += V^T P^T (tile t), S^T = K Q^T (tile t+1) ========
+    __builtin_amdgcn_s_setprio(0);
     load_tile(set_tag);
     matrix_phase(t);
     cp_valid = cp_left;
