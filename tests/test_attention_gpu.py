@@ -314,3 +314,82 @@ def test_bf16_result_and_producer_feed_the_attention(env):
     torch.cuda.synchronize()
     assert out.dtype == torch.bfloat16 and out.shape == (B, Sq, H, D)
     _cmp(out, layer.last_lse, ref_out, ref_lse, "producer + attention + bf16 result")
+
+
+def test_profiling_to_divider_map_end_to_end(hip, tmp_path):
+    """redundancy_preprocess (two "prompts") -> finish_auto_setting -> .pt on disk -> init_redundancy_map
+    -> dividers -> a generation pass that reuses cached states.  The recorded map equals the oracle's
+    rel_l1 sums, the dividers equal the oracle's generate + refine on that map, and the cached pass
+    follows the lock-step oracle of the state machine."""
+    from oracle import divider_map as od
+    from ditango_amd.core import config, parallel_state, redundancy_map as rmod
+    from ditango_amd.core.attention import proAttention
+    from ditango_amd.utils import update_timestep
+
+    N, T, L, B, H, D, S = 4, 8, 2, 1, 2, 64, 72
+    pct, dv = [0, 40, 90], [4, 2, 1, 1]
+    parallel_state.init_local_groups(N, 1)
+    cfg = config.init_config(None, num_inference_steps=T, num_layers=L, stride_percentiles=pct, stride_dividers=dv,
+                             ditango_base=str(tmp_path), model_name="toy")
+    rmod.destroy_redundancy_map()
+    try:
+        rm = rmod.init_redundancy_map(cfg, quiet=True)          # nothing on disk yet: full stride
+        group = parallel_state.get_usp_group()
+        recorded = torch.zeros(T, L)
+
+        def make_inputs(seed):
+            g = torch.Generator().manual_seed(seed)
+            base = _inputs(B, S, [S] * N, H, D, seed=seed, norm="rms")
+            steps = []
+            q, ks, vs = base
+            for t in range(T):
+                steps.append((q.bfloat16(), [k.bfloat16() for k in ks], [v.bfloat16() for v in vs]))
+                q, ks, vs = _perturb(q, g), [_perturb(k, g) for k in ks], [_perturb(v, g) for v in vs]
+            return steps
+
+        def generate(prompt, seed_of, check=None):
+            layers = [proAttention(l, group) for l in range(L)]
+            steps = make_inputs(seed_of[prompt])
+            prev = [None] * L
+            for t in range(T):
+                update_timestep(t)
+                qb, kb, vb = steps[t]
+                group.set_kv_chunks([k.cuda() for k in kb], [v.cuda() for v in vb])
+                for l in range(L):
+                    out = layers[l].attn(qb.cuda(), group.kv_chunk(1)[0], group.kv_chunk(1)[1]).cpu()
+                    if check is None:
+                        if prev[l] is not None:
+                            recorded[t, l] += om.rel_l1(out, prev[l])
+                        prev[l] = out
+                    else:
+                        check(t, l, layers[l], out, steps[t])
+
+        seeds = {"a": 5, "b": 6}
+        rmod.redundancy_preprocess(generate, {"seed_of": seeds}, prompt_list=["a", "b"])
+        assert not rm.auto_setting
+        path = tmp_path / "configs" / "toy" / f"redundancy_map_{T}_{L}.pt"
+        saved = torch.load(str(path), weights_only=True)
+        assert saved.shape == (T, L) and (saved[0] == 0).all()
+        assert (saved - recorded).abs().max() < 2e-5
+        # a fresh process would now find the file
+        rmod.destroy_redundancy_map()
+        rm = rmod.init_redundancy_map(cfg, quiet=True)
+        div, _ = od.generate_divider_map(saved.numpy(), N, pct, dv)
+        refined, _ = od.refine_divider_map(div)
+        assert np.array_equal(rm.divider_map.numpy(), refined)
+        assert (refined[3:T - 2] > 1).any(), "the toy map should leave something to reuse"
+        # the cached pass follows the state-machine oracle call by call
+        oracles = [RingOracle(N) for _ in range(L)]
+
+        def check(t, l, layer, out, step):
+            qb, kb, vb = step
+            curr, nxt = od.curr_stride(refined, N, t, l), od.next_stride(refined, N, t, l)
+            traces = oracles[l].call(t, curr, nxt)
+            tr = traces[1]
+            assert list(layer.last_plan.computed) == list(tr.computed), (t, l)
+
+        generate("a", seeds, check=check)
+    finally:
+        rmod.destroy_redundancy_map()
+        parallel_state.destroy_local_groups()
+        update_timestep(0)
