@@ -53,7 +53,6 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kWaves = 8;
 constexpr int kThreads = kWaves * 64;
@@ -65,18 +64,6 @@ constexpr int kNumVBuf = 3;
 #ifndef DT_RING
 #define DT_RING 4
 #endif
-// true: two groups of 4 wavefronts run one phase apart with a barrier after every phase;
-// false: all wavefronts in the same phase, one barrier per tile.
-#ifndef DT_STAGGER
-#define DT_STAGGER 1
-#endif
-constexpr bool kStagger = DT_STAGGER;
-
-template <int N> struct VecOf;
-template <> struct VecOf<4> { typedef u32x4 type; };
-template <> struct VecOf<2> { typedef u32x2 type; };
-template <> struct VecOf<1> { typedef uint32_t type; };
-
 // Row permutation of the K operand: MFMA row i -> key (within a 32-key half tile).
 __device__ __forceinline__ int key_of_row(int i) {
   return (i & 19) | ((i & 4) << 1) | ((i & 8) >> 1);
@@ -108,15 +95,7 @@ __device__ __forceinline__ void phase_barrier_after_vector(V (&p)[2][2]) {
 template <typename V, int NO>
 __device__ __forceinline__ void phase_barrier_after_matrix(V (&sa)[2], V (&oa)[NO]) {
   __builtin_amdgcn_sched_barrier(0);
-  if constexpr (!kStagger) {
-    // no barrier between a wavefront's matrix phase and its next vector phase: the buffers the
-    // next fill overwrites were last read one iteration earlier
-    if constexpr (NO == 4) {
-      asm volatile("" : "+v"(sa[0]), "+v"(sa[1]), "+v"(oa[0]), "+v"(oa[1]), "+v"(oa[2]), "+v"(oa[3]));
-    } else {
-      asm volatile("" : "+v"(sa[0]), "+v"(sa[1]), "+v"(oa[0]), "+v"(oa[1]));
-    }
-  } else if constexpr (NO == 4) {
+  if constexpr (NO == 4) {
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier"
                  : "+v"(sa[0]), "+v"(sa[1]), "+v"(oa[0]), "+v"(oa[1]), "+v"(oa[2]), "+v"(oa[3])
                  :
@@ -216,7 +195,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: keeps group/buffer arithmetic scalar
-  const int group = kStagger ? (wave >> 2) : 0;  // 0: leads, 1: runs one phase behind
+  const int group = wave >> 2;  // 0: leads, 1: runs one phase behind
   const int col = lane & 31;    // query column (B operand) / operand row (A operand)
   const int hh = lane >> 5;     // which half of the contraction dimension this lane feeds
   const int q0 = q_begin + qt * kBQ + wave * 32;
@@ -558,7 +537,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     iteration(t + 1, Set1{});
   }
   // the leading group waits out the phase it is ahead
-  if (kStagger && group == 0) phase_barrier();
+  if (group == 0) phase_barrier();
 
   // ---- epilogue -------------------------------------------------------------------------
   const float l_tot = l_run + __shfl_xor(l_run, 32);

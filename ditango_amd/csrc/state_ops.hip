@@ -295,7 +295,7 @@ __global__ __launch_bounds__(kThreads) void state_copy_kernel(const CopyArgs a) 
 }
 
 // One wavefront per (t, l) row: ballot + prefix popcount compaction.
-__global__ __launch_bounds__(64) void build_schedule_kernel(const uint8_t* mask, int T, int L, int C, int row0,
+__global__ __launch_bounds__(64) void build_schedule_kernel(const uint8_t* mask, int /*T*/, int /*L*/, int C, int row0,
                                                             int diag, int32_t* compute_ids, int32_t* reuse_ids,
                                                             int32_t* counts) {
   const int row = row0 + blockIdx.x;          // t*L + l
