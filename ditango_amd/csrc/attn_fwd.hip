@@ -11,8 +11,8 @@
 //   * The 8 wavefronts form two groups of 4 that run the same loop ONE PHASE
 //     APART ("ping-pong"): while group A issues the MFMAs of a tile
 //     (O^T += V^T P^T of the previous tile, then S^T = K Q^T of this one), group B
-//     runs the VALU half (online softmax of its tile, transposing and storing the
-//     next K/V tile into LDS), and vice versa; a workgroup barrier separates the
+//     runs the VALU half (online softmax of its tile, copying the next K/V tile
+//     from registers into LDS), and vice versa; a workgroup barrier separates the
 //     phases.  Each SIMD holds one wavefront of either group, so its matrix pipe
 //     and its vector ALU are busy at the same time instead of taking turns.
 //   * KV is consumed in tiles of 64 keys, staged in LDS as they come, [key][d]:
