@@ -52,3 +52,33 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert rc == -2 and b"head dim" in lib.dt_last_error()
     rc = lib.dt_build_schedule(None, 1, 1, 1, 0, 0, -1, None, None, None, None)
     assert rc == -1
+
+
+def test_header_is_plain_c_and_links_from_c(tmp_path):
+    """A C translation unit (gcc -std=c99 -pedantic) includes the header, takes the address of every
+    declared function and links against the built library: the boundary has no C++ or torch types."""
+    import shutil
+    import subprocess
+    from ditango_amd import _hip
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    if not _hip.LIB_PATH.exists():
+        from ditango_amd.build import build_lib
+        build_lib()
+    names = _declared()
+    src = tmp_path / "use.c"
+    src.write_text('#include "ditango_hip.h"\n#include <stdio.h>\n'
+                   "int main(void) {\n  void* p[] = {" + ", ".join(f"(void*){n}" for n in names) + "};\n"
+                   "  int rc = dt_merge_states(0, 0, 0, 0, 0, 0, DT_BF16, 0, DT_LSE_BHS, 1, 1, 1, 128, 0);\n"
+                   '  printf("%d %d %d %s\\n", dt_version(), (int)(sizeof(p) / sizeof(p[0])), rc, dt_last_error());\n'
+                   "  return rc == DT_ERR_INVALID ? 0 : 1;\n}\n")
+    exe = tmp_path / "use"
+    libdir = str(_hip.LIB_PATH.parent)
+    # -pedantic flags the function-pointer casts only; everything else must be clean
+    r = subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe),
+                        "-L", libdir, "-lditango_hip", f"-Wl,-rpath,{libdir}"], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    r = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    ver, n, rc, *msg = r.stdout.split()
+    assert int(ver) >= 100 and int(n) == len(names) and int(rc) == -1 and msg
