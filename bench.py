@@ -108,6 +108,53 @@ def cpu_baseline(B, H, D, Sq, lens, mean_computed, n_chunks, norm, budget_s=20.0
     }
 
 
+def bench_stride_schedule(args):
+    """One full pass of the reference's stride schedule: 50 steps x ``--layers`` layers (default 12) of
+    ``proAttention.attn`` at the HunyuanVideo per-rank shape as ring rank 0 of 8, with the divider map
+    generated from the redundancy map the reference ships for HunyuanVideo (percentiles [0,40,90],
+    dividers [8,4,2,1], configs/hunyuanvideo/config.yaml).  Every call is timed, the full-stride
+    steps included."""
+    from ditango_amd.core import config, parallel_state, redundancy_map as rmod
+    from ditango_amd.core.attention import proAttention
+    from ditango_amd.utils import update_timestep
+    label, B, H, D, Sq, lens, T, L, _, _, norm = WORKLOADS["hunyuanvideo"]
+    N, rank = len(lens), 0
+    L_run = min(L, args.layers or 12)
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    parallel_state.init_local_groups(N, rank)
+    cfg = config.init_config(None, num_inference_steps=T, num_layers=L, stride_percentiles=[0, 40, 90],
+                             stride_dividers=[8, 4, 2, 1])
+    rmod.destroy_redundancy_map()
+    rm = rmod.init_redundancy_map(cfg, redun_map_path=os.path.join(ROOT, "tests", "golden", "redundancy_map_50_60.pt"),
+                                  quiet=True)
+    q, ks, vs = make_inputs(B, H, D, Sq, lens, norm, dev)
+    group = parallel_state.get_usp_group()
+    group.set_kv_chunks(ks, vs)
+    layers = [proAttention(l, group) for l in range(L_run)]
+    computed = 0
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for t in range(T):
+        update_timestep(t)
+        for l in range(L_run):
+            layers[l].attn(q, ks[rank], vs[rank])
+            computed += len(layers[l].last_plan.computed)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    calls = T * L_run
+    flops = 4.0 * B * H * Sq * lens[0] * D * computed
+    print(json.dumps({
+        "metric": "ms/layer", "value": round(1e3 * elapsed / calls, 4), "unit": "ms", "n_gpus": 1, "steps": calls, "warmup": 0,
+        "ms_per_step": round(1e3 * elapsed / calls, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": label + ", stride schedule of the shipped redundancy map, ring rank 0 of 8", "B": B, "H": H,
+                   "D": D, "Sq": Sq, "kv_chunks": N, "Sk": lens[0], "layers_instantiated": L_run, "steps_per_layer": T,
+                   "mean_chunks_computed_per_call": round(computed / calls, 3)},
+        "layer_attn_tflops": round(flops / elapsed / 1e12, 1),
+    }), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -118,6 +165,9 @@ def main():
     ap.add_argument("--reuse", type=float, default=None, help="override the mask's reuse probability")
     ap.add_argument("--kernel-reps", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--schedule", default="mask", choices=["mask", "stride"],
+                    help="mask: the seeded Bernoulli reuse mask (the headline metric); stride: the reference's own stride "
+                         "schedule from the HunyuanVideo redundancy map it ships (a separate, shorter report)")
     ap.add_argument("--kernels-only", action="store_true",
                     help="run only the per-kernel roofline launches (short; for rocprofv3 counter passes)")
     args = ap.parse_args()
@@ -135,6 +185,8 @@ def main():
     from ditango_amd.utils import update_timestep
     _hip.load_library()
 
+    if args.schedule == "stride":
+        return bench_stride_schedule(args)
     label, B, H, D, Sq, lens, T, L, p, diag, norm = WORKLOADS[args.workload]
     if args.reuse is not None:
         p = args.reuse
