@@ -85,7 +85,7 @@ def cpu_baseline(B, H, D, Sq, lens, mean_computed, n_chunks, norm, budget_s=20.0
         om.chunk_attention(q, k, v)
         n_done += 1
         el = time.perf_counter() - t0
-        if el > budget_s * 0.7 or n_done >= 8:
+        if el > budget_s * 0.7 or n_done >= 32:
             break
     per_head_chunk = el / n_done
     # merge of n_chunks states on 1/8 of the rows, literal reference fold
