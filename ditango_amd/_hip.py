@@ -24,6 +24,7 @@ DT_MAX_CHUNKS = 40
 DT_MAX_JOBS = 40
 DT_MAX_JOB_ENTRIES = 64
 DT_MAX_MERGE = 40
+DT_MAX_SEGMENTS = 8
 
 c_i32, c_i64, c_f32, c_vp = ctypes.c_int32, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
 _P = ctypes.POINTER
@@ -44,6 +45,10 @@ _SIGNATURES = {
                                          c_i32, _P(c_vp), _P(c_vp), _P(c_i32), _P(c_i64), c_i64, c_i64,
                                          c_vp, c_vp, c_i32, c_vp, c_i64, c_vp, c_i64, c_i32, c_vp, c_vp,
                                          c_f32, c_vp]),
+    "dt_attn_sched_seg_fwd": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i64, c_i64, c_i64,
+                                             c_i32, _P(c_vp), _P(c_vp), _P(c_i32), _P(c_i64), c_i64, c_i64,
+                                             c_vp, c_vp, c_i32, c_vp, c_i64, c_vp, c_i64, c_i32, c_vp, c_vp,
+                                             c_i32, _P(c_i32), _P(c_i32), _P(c_i32), _P(c_i32), c_f32, c_vp]),
     "dt_merge_states": (ctypes.c_int, [c_i32, _P(c_vp), _P(c_vp), _P(c_i32), _P(c_i32), c_vp, c_i32, c_vp, c_i32,
                                        c_i32, c_i32, c_i32, c_i32, c_vp]),
     "dt_cache_store": (ctypes.c_int, [c_vp, c_i32, c_vp, c_i32, c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_vp]),
@@ -252,9 +257,13 @@ def attn_jobs_fwd(q: torch.Tensor, table: ChunkTable, jobs: Sequence[Sequence[in
 def attn_sched_fwd(q: torch.Tensor, table: ChunkTable, dev_compute_ids: torch.Tensor, dev_count: torch.Tensor,
                    max_jobs: int, slot_out: torch.Tensor, slot_lse: torch.Tensor, diag: int,
                    diag_out: Optional[torch.Tensor], diag_lse: Optional[torch.Tensor],
-                   softmax_scale: float = 0.0) -> None:
+                   softmax_scale: float = 0.0, seg_q: Optional[Sequence[Tuple[int, int]]] = None,
+                   seg_kv: Optional[Sequence[Sequence[Tuple[int, int]]]] = None) -> None:
     """Device-scheduled launch: chunk ids come from ``dev_compute_ids[:dev_count]`` in device memory and
-    each state lands in its slot of the arena (``slot_out [C,B,Sq,H,D]`` bf16, ``slot_lse [C,B,H,Sq]`` fp32)."""
+    each state lands in its slot of the arena (``slot_out [C,B,Sq,H,D]`` bf16, ``slot_lse [C,B,H,Sq]`` fp32).
+
+    On a packed variable-length batch, ``seg_q[s] = (begin, length)`` are the query rows of segment s and
+    ``seg_kv[c][s] = (begin, length)`` its keys inside chunk c; every scheduled chunk then runs once per segment."""
     lib = load_library()
     _check_qkv(q, "q")
     B, Sq, H, D = q.shape
@@ -270,14 +279,25 @@ def attn_sched_fwd(q: torch.Tensor, table: ChunkTable, dev_compute_ids: torch.Te
         _require(diag_out is not None and diag_lse is not None, "a diag chunk needs (diag_out, diag_lse)")
         _require(diag_out.dtype == torch.bfloat16 and diag_out.is_contiguous() and tuple(diag_out.shape) == (B, Sq, H, D), "diag_out must be contiguous bf16 [B,Sq,H,D]")
         _require(diag_lse.dtype == torch.float32 and diag_lse.is_contiguous() and tuple(diag_lse.shape) == (B, H, Sq), "diag_lse must be contiguous fp32 [B,H,Sq]")
-    rc = lib.dt_attn_sched_fwd(q.data_ptr(), B, Sq, H, D, q.stride(0), q.stride(1), q.stride(2),
-                               table.n, table.k_ptrs, table.v_ptrs, table.lens, table.sb, table.ss, table.sh,
-                               dev_compute_ids.data_ptr(), dev_count.data_ptr(), int(max_jobs),
-                               slot_out.data_ptr(), slot_out.stride(0), slot_lse.data_ptr(), slot_lse.stride(0),
-                               int(diag), diag_out.data_ptr() if diag_out is not None else None,
-                               diag_lse.data_ptr() if diag_lse is not None else None,
-                               float(softmax_scale), _stream())
-    _check(rc, "dt_attn_sched_fwd")
+    n_seg, a_qb, a_ql, a_kb, a_kl = 0, None, None, None, None
+    if seg_q is not None:
+        n_seg = len(seg_q)
+        _require(seg_kv is not None and len(seg_kv) == table.n and all(len(r) == n_seg for r in seg_kv),
+                 "seg_kv needs one (begin, length) per chunk and segment")
+        _require(0 < n_seg <= DT_MAX_SEGMENTS and n_seg * table.n <= DT_MAX_JOB_ENTRIES,
+                 f"need 1..{DT_MAX_SEGMENTS} segments and at most {DT_MAX_JOB_ENTRIES} (chunk, segment) pairs")
+        a_qb = (c_i32 * n_seg)(*[int(b) for b, _ in seg_q])
+        a_ql = (c_i32 * n_seg)(*[int(n) for _, n in seg_q])
+        a_kb = (c_i32 * (n_seg * table.n))(*[int(b) for row in seg_kv for b, _ in row])
+        a_kl = (c_i32 * (n_seg * table.n))(*[int(n) for row in seg_kv for _, n in row])
+    rc = lib.dt_attn_sched_seg_fwd(q.data_ptr(), B, Sq, H, D, q.stride(0), q.stride(1), q.stride(2),
+                                   table.n, table.k_ptrs, table.v_ptrs, table.lens, table.sb, table.ss, table.sh,
+                                   dev_compute_ids.data_ptr(), dev_count.data_ptr(), int(max_jobs),
+                                   slot_out.data_ptr(), slot_out.stride(0), slot_lse.data_ptr(), slot_lse.stride(0),
+                                   int(diag), diag_out.data_ptr() if diag_out is not None else None,
+                                   diag_lse.data_ptr() if diag_lse is not None else None,
+                                   n_seg, a_qb, a_ql, a_kb, a_kl, float(softmax_scale), _stream())
+    _check(rc, "dt_attn_sched_seg_fwd")
 
 
 # ---------------------------------------------------------------------------------------------

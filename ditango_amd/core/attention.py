@@ -329,8 +329,16 @@ class proAttention:
                 raise RuntimeError(f"T{t}L{l}: mask asks to reuse chunk {c} but no state was ever stored for it")
         n_comp = int(rm.sched_counts_host[t, l, 0])
         table = _hip.ChunkTable(ks, vs)
+        seg_q = seg_kv = None
+        if self._segments is not None:
+            # packed variable-length batch: every scheduled chunk runs once per segment
+            cu_q, cu_kv_of = self._segments
+            seg_q = [(cu_q[i], cu_q[i + 1] - cu_q[i]) for i in range(len(cu_q) - 1)]
+            seg_kv = [[(cu_kv_of(c)[i], cu_kv_of(c)[i + 1] - cu_kv_of(c)[i]) for i in range(len(cu_q) - 1)]
+                      for c in range(C)]
         _hip.attn_sched_fwd(query, table, rm.sched_compute_ids[t, l], rm.sched_counts[t, l, 0:1], n_comp,
-                            cache.arena_out, cache.arena_lse, diag, cache.diag_out, cache.diag_lse)
+                            cache.arena_out, cache.arena_lse, diag, cache.diag_out, cache.diag_lse,
+                            seg_q=seg_q, seg_kv=seg_kv)
         outs, lses = [], []
         for c in range(C):
             if c == diag:
@@ -358,13 +366,11 @@ class proAttention:
         the others come with the chunks: ``LocalRingGroup.set_kv_chunks(..., cu_seqlens_kv=...)``).
         Returns fp32 ``[total, H, D]``.  Without sequence lengths it is ``attn`` (:252-254).
         Each segment runs as attention jobs on row/key sub-ranges of one launch
-        (``dt_attn_seg_jobs_fwd``); schedule, cache and merge are those of ``attn``."""
+        (``dt_attn_seg_jobs_fwd``, or ``dt_attn_sched_seg_fwd`` under a per-chunk reuse mask); schedule,
+        cache and merge are those of ``attn``."""
         if cu_seqlens_q is None and cu_seqlens_kv is None and max_seqlen_q is None and max_seqlen_kv is None:
             logger.warning("cu_seqlens_q not provided, using normal attention instead.")
             return self.attn(query, key, value)
-        rm = get_redundancy_map()
-        if rm is not None and rm.chunk_mask is not None:
-            raise NotImplementedError("the per-chunk mask mode takes dense [B,S,H,D] inputs")
         total_q, H, D = query.shape
         cu_q = [int(x) for x in (cu_seqlens_q.tolist() if hasattr(cu_seqlens_q, "tolist") else cu_seqlens_q)]
         local_cu = [int(x) for x in (cu_seqlens_kv.tolist() if hasattr(cu_seqlens_kv, "tolist") else cu_seqlens_kv)]

@@ -166,9 +166,15 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   int q_begin = 0, q_end = a.Sq;   // query rows of this job
   __bf16* out_ptr;
   float* lse_ptr;
+  int vseg = -1;  // segment of a packed variable-length batch (device-listed jobs only)
   if (a.dev_ids != nullptr) {
-    if (job >= *a.dev_count) return;
-    single = __builtin_amdgcn_readfirstlane(a.dev_ids[job]);  // uniform by construction; tell the compiler
+    int slot = job;
+    if (a.n_seg > 0) {
+      slot = job / a.n_seg;
+      vseg = job - slot * a.n_seg;
+    }
+    if (slot >= *a.dev_count) return;
+    single = __builtin_amdgcn_readfirstlane(a.dev_ids[slot]);  // uniform by construction; tell the compiler
     if (single < 0 || single >= a.n_chunks) return;  // never index the tables with a bad id
     seg_begin = 0;
     seg_end = 1;
@@ -178,6 +184,11 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     } else {
       out_ptr = a.slot_out + (int64_t)single * a.slot_out_stride;
       lse_ptr = a.slot_lse + (int64_t)single * a.slot_lse_stride;
+    }
+    if (vseg >= 0) {
+      q_begin = a.seg_q_begin[vseg];
+      q_end = q_begin + a.seg_q_len[vseg];
+      if (qt * kBQ >= q_end - q_begin) return;  // the grid is sized for the longest segment
     }
   } else {
     seg_begin = a.job_begin[job];
@@ -189,8 +200,14 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     if (qt * kBQ >= q_end - q_begin) return;  // the grid is sized for the longest job
   }
   auto chunk_of = [&](int seg) -> int { return single >= 0 ? single : a.job_chunks[seg]; };
-  auto kv_begin_of = [&](int seg) -> int { return single >= 0 ? 0 : a.entry_kv_begin[seg]; };
-  auto kv_len_of = [&](int seg) -> int { return single >= 0 ? a.kv_len[single] : a.entry_kv_len[seg]; };
+  auto kv_begin_of = [&](int seg) -> int {
+    if (single < 0) return a.entry_kv_begin[seg];
+    return vseg >= 0 ? a.entry_kv_begin[single * a.n_seg + vseg] : 0;
+  };
+  auto kv_len_of = [&](int seg) -> int {
+    if (single < 0) return a.entry_kv_len[seg];
+    return vseg >= 0 ? a.entry_kv_len[single * a.n_seg + vseg] : a.kv_len[single];
+  };
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;

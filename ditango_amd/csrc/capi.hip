@@ -195,12 +195,15 @@ extern "C" int dt_attn_chunk_fwd(const void* q, const void* k, const void* v, vo
                           lses, softmax_scale, stream);
 }
 
-extern "C" int dt_attn_sched_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D, int64_t q_sb, int64_t q_ss,
-                                 int64_t q_sh, int32_t n_chunks, const void* const* k_ptrs, const void* const* v_ptrs,
-                                 const int32_t* kv_lens, const int64_t* kv_sb, int64_t kv_ss, int64_t kv_sh,
-                                 const int32_t* dev_compute_ids, const int32_t* dev_count, int32_t max_jobs,
-                                 void* slot_out, int64_t slot_out_stride, float* slot_lse, int64_t slot_lse_stride,
-                                 int32_t diag, void* diag_out, float* diag_lse, float softmax_scale, void* stream) {
+extern "C" int dt_attn_sched_seg_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D, int64_t q_sb,
+                                     int64_t q_ss, int64_t q_sh, int32_t n_chunks, const void* const* k_ptrs,
+                                     const void* const* v_ptrs, const int32_t* kv_lens, const int64_t* kv_sb,
+                                     int64_t kv_ss, int64_t kv_sh, const int32_t* dev_compute_ids,
+                                     const int32_t* dev_count, int32_t max_jobs, void* slot_out,
+                                     int64_t slot_out_stride, float* slot_lse, int64_t slot_lse_stride, int32_t diag,
+                                     void* diag_out, float* diag_lse, int32_t n_seg, const int32_t* seg_q_begin,
+                                     const int32_t* seg_q_len, const int32_t* seg_kv_begin,
+                                     const int32_t* seg_kv_len, float softmax_scale, void* stream) {
   AttnArgs a{};
   if (int rc = fill_common(a, q, B, Sq, H, D, q_sb, q_ss, q_sh, n_chunks, k_ptrs, v_ptrs, kv_lens, kv_sb, kv_ss, kv_sh,
                            softmax_scale))
@@ -224,6 +227,46 @@ extern "C" int dt_attn_sched_fwd(const void* q, int32_t B, int32_t Sq, int32_t H
     set_error("diag chunk %d needs a destination outside the cache", diag);
     return DT_ERR_INVALID;
   }
+  int32_t jobs = max_jobs;
+  if (n_seg != 0) {
+    if (n_seg < 0 || n_seg > DT_MAX_SEGMENTS || (int64_t)n_seg * n_chunks > DT_MAX_JOB_ENTRIES) {
+      set_error("%d segments x %d chunks: need 1..%d segments and at most %d (chunk, segment) pairs", n_seg, n_chunks,
+                DT_MAX_SEGMENTS, DT_MAX_JOB_ENTRIES);
+      return DT_ERR_INVALID;
+    }
+    if (!seg_q_begin || !seg_q_len || !seg_kv_begin || !seg_kv_len) {
+      set_error("null segment range array");
+      return DT_ERR_INVALID;
+    }
+    int32_t longest = 0;
+    for (int s = 0; s < n_seg; ++s) {
+      const int32_t qb = seg_q_begin[s], ql = seg_q_len[s];
+      if (qb < 0 || ql < 0 || (int64_t)qb + ql > Sq) {
+        set_error("segment %d: query rows [%d, %d) outside [0, %d)", s, qb, qb + ql, Sq);
+        return DT_ERR_INVALID;
+      }
+      a.seg_q_begin[s] = qb;
+      a.seg_q_len[s] = ql;
+      longest = ql > longest ? ql : longest;
+    }
+    for (int c = 0; c < n_chunks; ++c)
+      for (int s = 0; s < n_seg; ++s) {
+        const int e = c * n_seg + s;
+        const int32_t kb = seg_kv_begin[e], kl = seg_kv_len[e];
+        if (kb < 0 || kl < 0 || (int64_t)kb + kl > kv_lens[c]) {
+          set_error("segment %d: keys [%d, %d) outside chunk %d of length %d", s, kb, kb + kl, c, kv_lens[c]);
+          return DT_ERR_INVALID;
+        }
+        a.entry_kv_begin[e] = kb;
+        a.entry_kv_len[e] = kl;
+      }
+    a.n_seg = n_seg;
+    // size the grid for the longest segment; shorter ones leave their surplus workgroups at once
+    a.nqt = (longest + 255) / 256;
+    a.total = B * H * a.nqt;
+    a.per_xcd = (a.total + 7) / 8;
+    jobs = max_jobs * n_seg;
+  }
   a.dev_ids = dev_compute_ids;
   a.dev_count = dev_count;
   a.slot_out = static_cast<__bf16*>(slot_out);
@@ -233,5 +276,17 @@ extern "C" int dt_attn_sched_fwd(const void* q, int32_t B, int32_t Sq, int32_t H
   a.diag = diag;
   a.diag_out = static_cast<__bf16*>(diag_out);
   a.diag_lse = diag_lse;
-  return launch_attn(a, D, max_jobs, (hipStream_t)stream);
+  return launch_attn(a, D, jobs, (hipStream_t)stream);
+}
+
+extern "C" int dt_attn_sched_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D, int64_t q_sb, int64_t q_ss,
+                                 int64_t q_sh, int32_t n_chunks, const void* const* k_ptrs, const void* const* v_ptrs,
+                                 const int32_t* kv_lens, const int64_t* kv_sb, int64_t kv_ss, int64_t kv_sh,
+                                 const int32_t* dev_compute_ids, const int32_t* dev_count, int32_t max_jobs,
+                                 void* slot_out, int64_t slot_out_stride, float* slot_lse, int64_t slot_lse_stride,
+                                 int32_t diag, void* diag_out, float* diag_lse, float softmax_scale, void* stream) {
+  return dt_attn_sched_seg_fwd(q, B, Sq, H, D, q_sb, q_ss, q_sh, n_chunks, k_ptrs, v_ptrs, kv_lens, kv_sb, kv_ss, kv_sh,
+                               dev_compute_ids, dev_count, max_jobs, slot_out, slot_out_stride, slot_lse,
+                               slot_lse_stride, diag, diag_out, diag_lse, 0, nullptr, nullptr, nullptr, nullptr,
+                               softmax_scale, stream);
 }

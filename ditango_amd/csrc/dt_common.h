@@ -47,6 +47,12 @@ struct AttnArgs {
   int32_t diag;
   __bf16* diag_out;
   float* diag_lse;
+  // device-listed jobs on a packed variable-length batch (n_seg > 0): launch job j is segment
+  // j % n_seg of the chunk listed at j / n_seg; the keys of segment s inside chunk c are
+  // entry_kv_begin/len[c * n_seg + s]
+  int32_t n_seg;
+  int32_t seg_q_begin[DT_MAX_SEGMENTS];
+  int32_t seg_q_len[DT_MAX_SEGMENTS];
 };
 
 int launch_attn(const AttnArgs& a, int D, int n_jobs, hipStream_t stream);

@@ -55,6 +55,7 @@ extern "C" {
 #define DT_MAX_JOBS 40         /* attention states one launch can produce */
 #define DT_MAX_JOB_ENTRIES 64  /* total chunk references over all jobs of a launch */
 #define DT_MAX_MERGE 40        /* states one merge launch can combine */
+#define DT_MAX_SEGMENTS 8      /* segments of a packed batch in one device-scheduled launch */
 
 int dt_version(void);
 const char* dt_last_error(void);
@@ -136,6 +137,28 @@ int dt_attn_sched_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D
                       void* slot_out, int64_t slot_out_stride, float* slot_lse, int64_t slot_lse_stride,
                       int32_t diag, void* diag_out, float* diag_lse,
                       float softmax_scale, void* stream);
+
+/*
+ * The device-scheduled launch on a packed variable-length batch (q [1, total, H, D], the layout of
+ * flash_attn_varlen_func as called at core/attention.py:314-324): segment s covers the query
+ * rows [seg_q_begin[s], + seg_q_len[s]) and, inside chunk c, the keys
+ * [seg_kv_begin[c * n_seg + s], + seg_kv_len[c * n_seg + s]).  Every scheduled chunk runs once
+ * per segment and writes that segment's rows of its slot; rows outside every segment are left
+ * untouched.  n_seg <= DT_MAX_SEGMENTS, n_chunks * n_seg <= DT_MAX_JOB_ENTRIES; the four
+ * range arrays are HOST arrays.  With n_seg = 1 covering all rows and keys it is
+ * dt_attn_sched_fwd.  No counterpart in the reference (its varlen path has no mask mode).
+ */
+int dt_attn_sched_seg_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D,
+                          int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
+                          int32_t n_chunks, const void* const* k_ptrs, const void* const* v_ptrs,
+                          const int32_t* kv_lens, const int64_t* kv_stride_b,
+                          int64_t kv_stride_s, int64_t kv_stride_h,
+                          const int32_t* dev_compute_ids, const int32_t* dev_count, int32_t max_jobs,
+                          void* slot_out, int64_t slot_out_stride, float* slot_lse, int64_t slot_lse_stride,
+                          int32_t diag, void* diag_out, float* diag_lse,
+                          int32_t n_seg, const int32_t* seg_q_begin, const int32_t* seg_q_len,
+                          const int32_t* seg_kv_begin, const int32_t* seg_kv_len,
+                          float softmax_scale, void* stream);
 
 /*
  * N-way LSE merge: lse = logsumexp_i lse_i, out = sum_i exp(lse_i - lse) out_i.

@@ -139,3 +139,80 @@ def test_varlen_stride_mode_matches_numeric_oracle(env, hip):
         q = q + 0.01 * torch.randn(q.shape, generator=g)
         ks = [k + 0.01 * torch.randn(k.shape, generator=g) for k in ks]
         vs = [v + 0.01 * torch.randn(v.shape, generator=g) for v in vs]
+
+
+def test_varlen_mask_mode_matches_numeric_oracle(env, hip):
+    """The packed entry under a per-chunk reuse mask: every scheduled chunk runs once per segment
+    (dt_attn_sched_seg_fwd) into its cache slot; a trailing pad region belongs to no segment."""
+    import numpy as np
+    from oracle import mask_schedule as ms
+    from ditango_amd.core.attention import proAttention
+    from ditango_amd.core.parallel_state import get_usp_group
+    from ditango_amd.utils import update_timestep
+    C, diag, H, D, T = 5, 1, 2, 128, 5
+    rm = env(C, diag, T, 1)
+    mask = ms.seeded_mask(T, 1, C, 0.5, seed=3, diag=diag)
+    rm.set_chunk_mask(mask, diag=diag)
+    total_q = 300
+    cu_q = [0, 260, 290]                # rows 290..299 belong to no segment
+    lens = [270, 300, 64, 129, 200]
+    cu_k = [[0, 200, 270], [0, 260, 300], [0, 64, 64], [0, 100, 129], [0, 0, 200]]   # empty segments included
+    g = torch.Generator().manual_seed(41)
+    q = torch.randn(total_q, H, D, generator=g)
+    ks = [torch.randn(n, H, D, generator=g) for n in lens]
+    vs = [torch.randn(n, H, D, generator=g) for n in lens]
+    oracle = ms.MaskCacheOracle(C, diag)
+    group = get_usp_group()
+    attn = proAttention(0, group)
+    for t in range(T):
+        qb, kb, vb = q.bfloat16(), [k.bfloat16() for k in ks], [v.bfloat16() for v in vs]
+        (ref_out, ref_lse), c_ids, r_ids = oracle.call(
+            mask[t, 0], lambda c: om.varlen_chunk_attention(qb, kb[c], vb[c], cu_q, cu_k[c]),
+            lambda sts: tuple(x[0] for x in om.merge_states_closed_form([s[0][None] for s in sts], [s[1][None] for s in sts])),
+            lambda s: (om.bf16_round(s[0]), s[1]))
+        print(f"case varlen mask t={t} computes {c_ids} reuses {r_ids}", flush=True)
+        update_timestep(t)
+        dk, dv = [k.cuda() for k in kb], [v.cuda() for v in vb]
+        group.set_kv_chunks(dk, dv, cu_seqlens_kv=[torch.tensor(c, dtype=torch.int32) for c in cu_k])
+        out = attn.varlen_attn(qb.cuda(), dk[diag], dv[diag], torch.tensor(cu_q, dtype=torch.int32),
+                               torch.tensor(cu_k[diag], dtype=torch.int32), 260, 300)
+        torch.cuda.synchronize()
+        n = int(rm.sched_counts_host[t, 0, 0])
+        assert rm.sched_compute_ids[t, 0, :n].tolist() == list(c_ids)
+        out = out.cpu()
+        assert (out[cu_q[-1]:] == 0).all()
+        err = (out[:cu_q[-1]] - ref_out[:cu_q[-1]]).abs().max().item()
+        lse = attn.last_lse.cpu()[0, :cu_q[-1], :, 0].transpose(0, 1)
+        lerr = (lse - ref_lse[:, :cu_q[-1]]).abs().max().item()
+        print(f"  out max-abs {err:.3e} lse {lerr:.3e}", flush=True)
+        assert err <= OUT_TOL and lerr <= LSE_TOL
+        q = q + 0.01 * torch.randn(q.shape, generator=g)
+        ks = [k + 0.01 * torch.randn(k.shape, generator=g) for k in ks]
+        vs = [v + 0.01 * torch.randn(v.shape, generator=g) for v in vs]
+
+
+def test_sched_seg_with_one_full_segment_is_the_dense_launch(hip):
+    C, B, H, D, Sq = 3, 1, 2, 64, 130
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(B, Sq, H, D, generator=g).bfloat16().cuda()
+    lens = [70, 128, 33]
+    ks = [torch.randn(B, n, H, D, generator=g).bfloat16().cuda() for n in lens]
+    vs = [torch.randn(B, n, H, D, generator=g).bfloat16().cuda() for n in lens]
+    table = hip.ChunkTable(ks, vs)
+    ids = torch.tensor([2, 0, 1], dtype=torch.int32, device="cuda")
+    cnt = torch.tensor([3], dtype=torch.int32, device="cuda")
+
+    def run(**kw):
+        ao = torch.zeros(C, B, Sq, H, D, dtype=torch.bfloat16, device="cuda")
+        al = torch.zeros(C, B, H, Sq, device="cuda")
+        hip.attn_sched_fwd(q, table, ids, cnt, C, ao, al, -1, None, None, **kw)
+        torch.cuda.synchronize()
+        return ao, al
+
+    a0, l0 = run()
+    a1, l1 = run(seg_q=[(0, Sq)], seg_kv=[[(0, n)] for n in lens])
+    assert torch.equal(a0, a1) and torch.equal(l0, l1)
+    with pytest.raises(hip.DitangoHipError):
+        run(seg_q=[(0, Sq + 1)], seg_kv=[[(0, n)] for n in lens])
+    with pytest.raises(hip.DitangoHipError):
+        run(seg_q=[(0, Sq)], seg_kv=[[(5, n)] for n in lens])
