@@ -14,7 +14,6 @@ Prints ONE JSON line: ms per layer call plus
 """
 import argparse
 import json
-import math
 import os
 import sys
 import time

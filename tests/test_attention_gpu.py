@@ -3,8 +3,6 @@ HIP kernels) against the numeric oracle on identical seeded inputs.
 
 Bar: out max-abs <= 2e-2 (bf16 states), lse max-abs <= 1e-3 (fp32), schedule bit-exact.
 """
-import math
-
 import numpy as np
 import pytest
 import torch

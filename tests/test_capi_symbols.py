@@ -1,6 +1,5 @@
 """The built library loads and exports every function include/ditango_hip.h declares
 (no compute calls: this runs without a GPU)."""
-import ctypes
 import os
 import re
 

@@ -2,7 +2,6 @@
 (``configs/*/redundancy_map_50_*.pt`` and the percentiles/dividers of ``configs/*/config.yaml``,
 copied as data under tests/golden/)."""
 import os
-import types
 from collections import Counter
 
 import numpy as np

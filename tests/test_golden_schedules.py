@@ -7,9 +7,6 @@ import numpy as np
 import pytest
 import torch
 
-from oracle import divider_map as od
-from oracle import mask_schedule as ms
-from oracle.state_machine import RingOracle, strides_from_dividers
 
 GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
 _spec = importlib.util.spec_from_file_location("make_schedule_fixtures", os.path.join(GOLDEN, "make_schedule_fixtures.py"))

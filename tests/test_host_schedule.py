@@ -1,9 +1,7 @@
 """The product's host-side schedule (closed-form ring delivery, pointer, cache
 bookkeeping) must equal the lock-step ring simulation of the oracle bit for bit."""
 import random
-import types
 
-import numpy as np
 import pytest
 import torch
 
