@@ -206,3 +206,26 @@ def test_size_independent_properties_at_hunyuan_shape(hip):
     back_o, back_l = hip.cache_load(slot_o, slot_l, torch.bfloat16, dst_lse_bsh=False)
     torch.cuda.synchronize()
     assert torch.equal(back_o, outs[3]) and torch.equal(back_l, lses[3])
+
+
+def test_attention_is_deterministic_at_hunyuan_shape(hip):
+    """Five launches over the same inputs at the HunyuanVideo per-rank shape give bit-identical states
+    (an LDS hazard between the two wavefront groups would show up as run-to-run differences)."""
+    B, H, D, Sq, Sk = 1, 24, 128, 14882, 14882
+    g = torch.Generator(device="cuda").manual_seed(12)
+    q = torch.randn(B, Sq, H, D, generator=g, device="cuda").bfloat16()
+    ks = [torch.randn(B, Sk, H, D, generator=g, device="cuda").bfloat16() for _ in range(2)]
+    vs = [torch.randn(B, Sk, H, D, generator=g, device="cuda").bfloat16() for _ in range(2)]
+    table = hip.ChunkTable(ks, vs)
+    ref = None
+    for i in range(5):
+        outs = [torch.empty(B, Sq, H, D, dtype=torch.bfloat16, device="cuda") for _ in range(3)]
+        lses = [torch.empty(B, H, Sq, dtype=torch.float32, device="cuda") for _ in range(3)]
+        hip.attn_jobs_fwd(q, table, [[0], [1], [0, 1]], outs, lses)
+        torch.cuda.synchronize()
+        if ref is None:
+            ref = (outs, lses)
+            assert all(torch.isfinite(l).all() for l in lses)
+        else:
+            for j in range(3):
+                assert torch.equal(outs[j], ref[0][j]) and torch.equal(lses[j], ref[1][j]), f"run {i} job {j}"
