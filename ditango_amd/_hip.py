@@ -41,6 +41,16 @@ _SIGNATURES = {
                                             c_i32, _P(c_vp), _P(c_vp), _P(c_i32), _P(c_i64), c_i64, c_i64,
                                             c_i32, _P(c_i32), _P(c_i32), _P(c_i32), _P(c_i32), _P(c_i32), _P(c_i32),
                                             _P(c_vp), _P(c_vp), c_f32, c_vp]),
+    "dt_attn_workspace_bytes": (ctypes.c_int64, []),
+    "dt_attn_seg_jobs_ws_fwd": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i64, c_i64, c_i64,
+                                               c_i32, _P(c_vp), _P(c_vp), _P(c_i32), _P(c_i64), c_i64, c_i64,
+                                               c_i32, _P(c_i32), _P(c_i32), _P(c_i32), _P(c_i32), _P(c_i32), _P(c_i32),
+                                               _P(c_vp), _P(c_vp), c_f32, c_vp, c_i64, c_vp]),
+    "dt_attn_sched_seg_ws_fwd": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i64, c_i64, c_i64,
+                                                c_i32, _P(c_vp), _P(c_vp), _P(c_i32), _P(c_i64), c_i64, c_i64,
+                                                c_vp, c_vp, c_i32, c_vp, c_i64, c_vp, c_i64, c_i32, c_vp, c_vp,
+                                                c_i32, _P(c_i32), _P(c_i32), _P(c_i32), _P(c_i32), c_f32,
+                                                c_vp, c_i64, c_vp]),
     "dt_attn_sched_fwd": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i64, c_i64, c_i64,
                                          c_i32, _P(c_vp), _P(c_vp), _P(c_i32), _P(c_i64), c_i64, c_i64,
                                          c_vp, c_vp, c_i32, c_vp, c_i64, c_vp, c_i64, c_i32, c_vp, c_vp,
@@ -162,6 +172,21 @@ def attn_chunk_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_sc
     return out, lse
 
 
+_workspaces = {}
+
+
+def attn_workspace(device) -> torch.Tensor:
+    """The per-device workspace of the attention launches (allocated once, ``dt_attn_workspace_bytes()``
+    bytes).  Launches that share it must be ordered on one stream, which is how ``proAttention`` runs."""
+    dev = torch.device(device)
+    key = (dev.type, dev.index if dev.index is not None else torch.cuda.current_device())
+    ws = _workspaces.get(key)
+    if ws is None:
+        ws = torch.empty(int(load_library().dt_attn_workspace_bytes()), dtype=torch.uint8, device=dev)
+        _workspaces[key] = ws
+    return ws
+
+
 class ChunkTable:
     """Host-side table of the KV chunks one layer call can touch (pointers, lengths, strides)."""
 
@@ -195,14 +220,16 @@ class ChunkTable:
 def attn_jobs_fwd(q: torch.Tensor, table: ChunkTable, jobs: Sequence[Sequence[int]],
                   outs: Sequence[torch.Tensor], lses: Sequence[torch.Tensor], softmax_scale: float = 0.0,
                   q_ranges: Optional[Sequence[Tuple[int, int]]] = None,
-                  kv_ranges: Optional[Sequence[Sequence[Tuple[int, int]]]] = None) -> None:
+                  kv_ranges: Optional[Sequence[Sequence[Tuple[int, int]]]] = None,
+                  workspace: Optional[torch.Tensor] = None) -> None:
     """One launch; job j attends q to the concatenation of chunks ``jobs[j]`` and writes (outs[j], lses[j]).
 
     ``q_ranges[j] = (begin, length)`` restricts job j to those query rows (the rest of its
     destination is left untouched); ``kv_ranges[j][i] = (begin, length)`` restricts the i-th chunk
     of job j to those keys.  Several jobs may share one destination if their rows are disjoint
     (the segments of a packed variable-length batch).  Launches are split to respect the limits
-    of one launch."""
+    of one launch.  With a ``workspace`` (``attn_workspace(device)``) the last, partly filled round of
+    workgroups of a launch is split along the keys and folded back (tail balancing)."""
     lib = load_library()
     _check_qkv(q, "q")
     B, Sq, H, D = q.shape
@@ -246,11 +273,13 @@ def attn_jobs_fwd(q: torch.Tensor, table: ChunkTable, jobs: Sequence[Sequence[in
         a_ql = (c_i32 * n)(*[int(q_ranges[start + jj][1]) for jj in range(n)]) if q_ranges is not None else None
         out_ptrs = (c_vp * n)(*[outs[start + jj].data_ptr() for jj in range(n)])
         lse_ptrs = (c_vp * n)(*[lses[start + jj].data_ptr() for jj in range(n)])
-        rc = lib.dt_attn_seg_jobs_fwd(q.data_ptr(), B, Sq, H, D, q.stride(0), q.stride(1), q.stride(2),
-                                      table.n, table.k_ptrs, table.v_ptrs, table.lens, table.sb, table.ss, table.sh,
-                                      n, begin, chunks, a_kvb, a_kvl, a_qb, a_ql, out_ptrs, lse_ptrs,
-                                      float(softmax_scale), _stream())
-        _check(rc, "dt_attn_seg_jobs_fwd")
+        rc = lib.dt_attn_seg_jobs_ws_fwd(q.data_ptr(), B, Sq, H, D, q.stride(0), q.stride(1), q.stride(2),
+                                         table.n, table.k_ptrs, table.v_ptrs, table.lens, table.sb, table.ss, table.sh,
+                                         n, begin, chunks, a_kvb, a_kvl, a_qb, a_ql, out_ptrs, lse_ptrs,
+                                         float(softmax_scale), workspace.data_ptr() if workspace is not None else None,
+                                         workspace.numel() * workspace.element_size() if workspace is not None else 0,
+                                         _stream())
+        _check(rc, "dt_attn_seg_jobs_ws_fwd")
         start = end
 
 
@@ -258,7 +287,8 @@ def attn_sched_fwd(q: torch.Tensor, table: ChunkTable, dev_compute_ids: torch.Te
                    max_jobs: int, slot_out: torch.Tensor, slot_lse: torch.Tensor, diag: int,
                    diag_out: Optional[torch.Tensor], diag_lse: Optional[torch.Tensor],
                    softmax_scale: float = 0.0, seg_q: Optional[Sequence[Tuple[int, int]]] = None,
-                   seg_kv: Optional[Sequence[Sequence[Tuple[int, int]]]] = None) -> None:
+                   seg_kv: Optional[Sequence[Sequence[Tuple[int, int]]]] = None,
+                   workspace: Optional[torch.Tensor] = None) -> None:
     """Device-scheduled launch: chunk ids come from ``dev_compute_ids[:dev_count]`` in device memory and
     each state lands in its slot of the arena (``slot_out [C,B,Sq,H,D]`` bf16, ``slot_lse [C,B,H,Sq]`` fp32).
 
@@ -290,14 +320,16 @@ def attn_sched_fwd(q: torch.Tensor, table: ChunkTable, dev_compute_ids: torch.Te
         a_ql = (c_i32 * n_seg)(*[int(n) for _, n in seg_q])
         a_kb = (c_i32 * (n_seg * table.n))(*[int(b) for row in seg_kv for b, _ in row])
         a_kl = (c_i32 * (n_seg * table.n))(*[int(n) for row in seg_kv for _, n in row])
-    rc = lib.dt_attn_sched_seg_fwd(q.data_ptr(), B, Sq, H, D, q.stride(0), q.stride(1), q.stride(2),
+    rc = lib.dt_attn_sched_seg_ws_fwd(q.data_ptr(), B, Sq, H, D, q.stride(0), q.stride(1), q.stride(2),
                                    table.n, table.k_ptrs, table.v_ptrs, table.lens, table.sb, table.ss, table.sh,
                                    dev_compute_ids.data_ptr(), dev_count.data_ptr(), int(max_jobs),
                                    slot_out.data_ptr(), slot_out.stride(0), slot_lse.data_ptr(), slot_lse.stride(0),
                                    int(diag), diag_out.data_ptr() if diag_out is not None else None,
                                    diag_lse.data_ptr() if diag_lse is not None else None,
-                                   n_seg, a_qb, a_ql, a_kb, a_kl, float(softmax_scale), _stream())
-    _check(rc, "dt_attn_sched_seg_fwd")
+                                   n_seg, a_qb, a_ql, a_kb, a_kl, float(softmax_scale),
+                                   workspace.data_ptr() if workspace is not None else None,
+                                   workspace.numel() * workspace.element_size() if workspace is not None else 0, _stream())
+    _check(rc, "dt_attn_sched_seg_ws_fwd")
 
 
 # ---------------------------------------------------------------------------------------------

@@ -298,7 +298,7 @@ class proAttention:
         if job_lists:
             table = _hip.ChunkTable(ks, vs)
             _hip.attn_jobs_fwd(query, table, job_lists, [d[0] for d in dests], [d[1] for d in dests],
-                               q_ranges=q_ranges, kv_ranges=kv_ranges)
+                               q_ranges=q_ranges, kv_ranges=kv_ranges, workspace=_hip.attn_workspace(dev))
         for job, (o, l) in zip(plan.jobs, states):
             if job.store_slot is not None:
                 self.cache.store_block(job.store_slot, o, l)  # :207-211
@@ -338,7 +338,7 @@ class proAttention:
                       for c in range(C)]
         _hip.attn_sched_fwd(query, table, rm.sched_compute_ids[t, l], rm.sched_counts[t, l, 0:1], n_comp,
                             cache.arena_out, cache.arena_lse, diag, cache.diag_out, cache.diag_lse,
-                            seg_q=seg_q, seg_kv=seg_kv)
+                            seg_q=seg_q, seg_kv=seg_kv, workspace=_hip.attn_workspace(query.device))
         outs, lses = [], []
         for c in range(C):
             if c == diag:

@@ -41,6 +41,7 @@
 //   * Workgroups are mapped to (head, query tile) so that the 8 XCDs each work
 //     through a contiguous range of heads: the workgroups that share an XCD's
 //     L2 stream the same K/V.
+#include <algorithm>
 #include <type_traits>
 
 #include "dt_common.h"
@@ -152,9 +153,23 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
   // ---- which (job, batch, head, query tile) ------------------------------------------
-  const int job = blockIdx.y;
+  int job = blockIdx.y;
   const int xcd = blockIdx.x & (kXcds - 1);
-  const int idx = blockIdx.x >> 3;
+  int idx = blockIdx.x >> 3;
+  int part = 0;          // which of the part_ways key-tile ranges of a tail item
+  bool is_part = false;  // this workgroup computes one part of a tail item
+  if (job >= a.n_jobs) {
+    // planes behind the jobs hold the parts of the tail items, in dispatch order
+    const int pi = (job - a.n_jobs) * (int)(gridDim.x >> 3) + idx;
+    if (pi >= a.tail_items * a.part_ways) return;
+    job = a.tail_job;
+    const int u = pi / a.part_ways;
+    part = pi - u * a.part_ways;
+    idx = a.tail_idx0 + u;
+    is_part = true;
+  } else if (job == a.tail_job && idx >= a.tail_idx0) {
+    return;  // runs as parts
+  }
   const int item = xcd * a.per_xcd + idx;
   if (idx >= a.per_xcd || item >= a.total) return;
   const int bh = item / a.nqt;
@@ -261,6 +276,36 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   };
   ld_next_chunk();
   cp_next_chunk();
+  if (is_part) {
+    // this workgroup covers key tiles [t0, t1) of the item: walk both cursors to t0
+    const int t0 = (int)((int64_t)n_tiles * part / a.part_ways);
+    const int t1 = (int)((int64_t)n_tiles * (part + 1) / a.part_ways);
+    int skip = t0;
+    while (skip > 0 && ld_seg < seg_end) {
+      const int in_chunk = (ld_left + kBK - 1) / kBK;
+      if (skip >= in_chunk) {
+        skip -= in_chunk;
+        ld_next_chunk();
+      } else {
+        ld_k += (int64_t)skip * kBK * ((int64_t)a.kv_ss * 2);
+        ld_v += (int64_t)skip * kBK * ((int64_t)a.kv_ss * 2);
+        ld_left -= skip * kBK;
+        skip = 0;
+      }
+    }
+    skip = t0;
+    while (skip > 0 && cp_seg < seg_end) {
+      const int in_chunk = (cp_left + kBK - 1) / kBK;
+      if (skip >= in_chunk) {
+        skip -= in_chunk;
+        cp_next_chunk();
+      } else {
+        cp_left -= skip * kBK;
+        skip = 0;
+      }
+    }
+    n_tiles = t1 - t0;
+  }
 
   // thread -> tile elements, the same for K and V: 16-byte chunk kc of rows kr0 + i*kRowStep
   const int kc = tid % T::kChunks;
@@ -541,7 +586,9 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     __builtin_amdgcn_s_setprio(0);
     load_tile(set_tag);
     matrix_phase(t);
-    cp_valid = cp_left;
+    // the tile after the last one of this workgroup's range has no keys for it (it is the
+    // padding of an odd tile count, or belongs to the next part of a split item)
+    cp_valid = t + 1 < n_tiles ? cp_left : 0;
     cp_left -= kBK;
     if (cp_left <= 0) cp_next_chunk();
     phase_barrier_after_matrix(s_acc, o_acc);
@@ -561,7 +608,13 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   const float lse = l_tot > 0.f ? (m_ref * c + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f : -INFINITY;
   const int qrow = q0 + col;
-  if (hh == 0 && qrow < q_end) lse_ptr[((int64_t)b * a.H + h) * a.Sq + qrow] = lse;
+  // tail launch: the partial state goes to this workgroup's workspace slot, [256 queries][D] + [256]
+  const int64_t ws_slot = (((int64_t)(idx - a.tail_idx0) * kXcds + xcd) * a.part_ways + part);
+  if (is_part) {
+    if (hh == 0) a.ws_lse[ws_slot * kBQ + wave * 32 + col] = lse;
+  } else if (hh == 0 && qrow < q_end) {
+    lse_ptr[((int64_t)b * a.H + h) * a.Sq + qrow] = lse;
+  }
 
   // O^T (registers, [d][query]) -> LDS [query][d] bf16 -> coalesced 16-byte stores.
   phase_barrier();  // every wavefront is done with the tile buffers
@@ -592,10 +645,81 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     const int row = p * kRowsPerPass + rr;
     const int qg = q0 + row;
     const u32x4 val = *reinterpret_cast<const u32x4*>(ol + row * T::kPitchO + cc * 16);
-    if (qg < q_end) {
+    if (is_part) {
+      __bf16* dst = a.ws_out + (ws_slot * kBQ + wave * 32 + row) * D + cc * 8;
+      *reinterpret_cast<u32x4*>(dst) = val;
+    } else if (qg < q_end) {
       __bf16* dst = out_ptr + (((int64_t)b * a.Sq + qg) * a.H + h) * D + cc * 8;
       *reinterpret_cast<u32x4*>(dst) = val;
     }
+  }
+}
+
+// Folds the part_ways partial states of every tail item into the item's rows of its destination.
+// One workgroup per item; a group of D/8 lanes owns a row.
+template <int D>
+__global__ __launch_bounds__(256) void attn_tail_fold_kernel(const AttnArgs a) {
+  const int xcd = blockIdx.x & (kXcds - 1);
+  const int u = blockIdx.x >> 3;
+  const int idx = a.tail_idx0 + u;
+  const int item = xcd * a.per_xcd + idx;
+  if (idx >= a.per_xcd || item >= a.total) return;
+  const int bh = item / a.nqt;
+  const int qt = item - bh * a.nqt;
+  const int b = bh / a.H;
+  const int h = bh - b * a.H;
+  const int job = a.tail_job;
+  __bf16* out_ptr;
+  float* lse_ptr;
+  if (a.dev_ids != nullptr) {
+    if (job >= *a.dev_count) return;
+    const int single = a.dev_ids[job];
+    if (single < 0 || single >= a.n_chunks) return;
+    out_ptr = single == a.diag ? a.diag_out : a.slot_out + (int64_t)single * a.slot_out_stride;
+    lse_ptr = single == a.diag ? a.diag_lse : a.slot_lse + (int64_t)single * a.slot_lse_stride;
+  } else {
+    out_ptr = a.job_out[job];
+    lse_ptr = a.job_lse[job];
+  }
+  constexpr int kLanes = D / 8;
+  constexpr int kRows = 256 / kLanes;
+  const int rr = threadIdx.x / kLanes;
+  const int cc = threadIdx.x % kLanes;
+  const int64_t slot0 = ((int64_t)u * kXcds + xcd) * a.part_ways;
+  for (int r0 = 0; r0 < kBQ; r0 += kRows) {
+    const int row = r0 + rr;
+    const int qg = qt * kBQ + row;
+    if (qg >= a.Sq) continue;
+    float m = -INFINITY;
+    for (int p = 0; p < a.part_ways; ++p) m = fmaxf(m, a.ws_lse[(slot0 + p) * kBQ + row]);
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    float den = 0.f;
+    if (m > -INFINITY) {
+      for (int p = 0; p < a.part_ways; ++p) {
+        const float w = __expf(a.ws_lse[(slot0 + p) * kBQ + row] - m);
+        const u32x4 v = *reinterpret_cast<const u32x4*>(a.ws_out + ((slot0 + p) * kBQ + row) * D + cc * 8);
+        const uint32_t e[4] = {v.x, v.y, v.z, v.w};
+        den += w;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          acc[2 * k] = __builtin_fmaf(w, __builtin_bit_cast(float, e[k] << 16), acc[2 * k]);
+          acc[2 * k + 1] = __builtin_fmaf(w, __builtin_bit_cast(float, e[k] & 0xffff0000u), acc[2 * k + 1]);
+        }
+      }
+    }
+    const float inv = den > 0.f ? 1.f / den : 0.f;
+    u32x4 o;
+    uint32_t pk[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      f32x2 f;
+      f.x = acc[2 * k] * inv;
+      f.y = acc[2 * k + 1] * inv;
+      pk[k] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+    }
+    o.x = pk[0]; o.y = pk[1]; o.z = pk[2]; o.w = pk[3];
+    *reinterpret_cast<u32x4*>(out_ptr + (((int64_t)b * a.Sq + qg) * a.H + h) * D + cc * 8) = o;
+    if (cc == 0) lse_ptr[((int64_t)b * a.H + h) * a.Sq + qg] = den > 0.f ? m + __logf(den) : -INFINITY;
   }
 }
 
@@ -616,13 +740,89 @@ static int launch_one(const AttnArgs& a, dim3 grid, hipStream_t stream) {
   return hip_fail(hipGetLastError(), "attn_fwd launch");
 }
 
-int launch_attn(const AttnArgs& a, int D, int n_jobs, hipStream_t stream) {
-  if (n_jobs <= 0 || a.total <= 0) return DT_OK;
-  dim3 grid((unsigned)(a.per_xcd * kXcds), (unsigned)n_jobs, 1);
+static int launch_dim(const AttnArgs& a, int D, dim3 grid, hipStream_t stream) {
   if (D == 128) return launch_one<128>(a, grid, stream);
-  if (D == 64) return launch_one<64>(a, grid, stream);
-  set_error("head dim %d not built (64 and 128 are)", D);
-  return DT_ERR_UNSUPPORTED;
+  return launch_one<64>(a, grid, stream);
+}
+
+// Number of CUs of the current device (one workgroup of the attention kernel per CU at a time).
+static int cu_count() {
+  static thread_local int cached_dev = -1, cached = 0;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  if (dev != cached_dev) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+    cached = n;
+    cached_dev = dev;
+  }
+  return cached;
+}
+
+int launch_attn(const AttnArgs& a_in, int D, int n_jobs, hipStream_t stream, void* workspace,
+                int64_t workspace_bytes, bool balance) {
+  if (n_jobs <= 0 || a_in.total <= 0) return DT_OK;
+  if (D != 128 && D != 64) {
+    set_error("head dim %d not built (64 and 128 are)", D);
+    return DT_ERR_UNSUPPORTED;
+  }
+  AttnArgs a = a_in;
+  a.n_jobs = n_jobs;
+  a.tail_job = -1;
+  a.tail_idx0 = 0;
+  a.tail_items = 0;
+  a.part_ways = 0;
+  const int slots_per_job = a.per_xcd * kXcds;
+  // ---- tail balancing: is the last round of workgroups worth splitting? -------------------
+  // Time is counted in key tiles.  Unsplit, the launch takes ceil(n / cus) rounds of one item
+  // (n_tiles tiles each).  With the last `rem` items cut into w parts, the parts are handed to
+  // CUs as they come free (same launch, no barrier in between), so the tail takes
+  // ceil(rem * w / cus) rounds of (n_tiles / w + kPartOverhead) tiles plus the fold kernel.
+  int tail = 0, ways = 0;
+  const int cus = balance && workspace ? cu_count() : 0;
+  const int64_t slot_bytes = (int64_t)kBQ * D * 2 + (int64_t)kBQ * 4;
+  if (cus >= 64 && cus % kXcds == 0 && a.total == slots_per_job) {
+    int n_tiles = 0;  // key tiles of one item of the last job (device-listed jobs: of the longest chunk)
+    if (a.dev_ids != nullptr) {
+      for (int c = 0; c < a.n_chunks; ++c) n_tiles = std::max(n_tiles, (a.kv_len[c] + kBK - 1) / kBK);
+    } else {
+      for (int e = a.job_begin[n_jobs - 1]; e < a.job_begin[n_jobs]; ++e) n_tiles += (a.entry_kv_len[e] + kBK - 1) / kBK;
+    }
+    // Measured on the HunyuanVideo and Step-Video shares: a part costs about 10 tiles on top of its
+    // own (start-up, epilogue, partial state), so many small parts only pay when they all run at once.
+    constexpr double kPartOverhead = 10.0;
+    constexpr double kFoldOverhead = 4.0;  // the fold kernel's launch
+    const int64_t n = (int64_t)n_jobs * slots_per_job;
+    const int rem = (int)(n % cus);
+    const int64_t cap = std::min<int64_t>(workspace_bytes / slot_bytes, kMaxTailSlots);
+    if (rem > 0 && rem <= slots_per_job && rem < n && n_tiles >= 16) {
+      double best = 0.2 * n_tiles;  // least gain worth the extra kernel
+      for (int w = 2; w <= 16; ++w) {
+        if ((int64_t)rem * w > cap || n_tiles / w < 6) break;
+        const double split = (double)(((int64_t)rem * w + cus - 1) / cus) * ((double)n_tiles / w + kPartOverhead) + kFoldOverhead;
+        if (n_tiles - split > best) {
+          best = n_tiles - split;
+          tail = rem;
+          ways = w;
+        }
+      }
+    }
+  }
+  if (tail == 0) return launch_dim(a, D, dim3((unsigned)slots_per_job, (unsigned)n_jobs, 1), stream);
+  a.tail_job = n_jobs - 1;
+  a.tail_idx0 = a.per_xcd - tail / kXcds;
+  a.tail_items = tail / kXcds;
+  a.part_ways = ways;
+  a.ws_out = static_cast<__bf16*>(workspace);
+  a.ws_lse = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + (int64_t)tail * ways * kBQ * D * 2);
+  // parts per XCD lane of the grid: tail / 8 items x ways parts, spread over extra planes of per_xcd entries
+  const int part_planes = (a.tail_items * ways + a.per_xcd - 1) / a.per_xcd;
+  if (int rc = launch_dim(a, D, dim3((unsigned)slots_per_job, (unsigned)(n_jobs + part_planes), 1), stream)) return rc;
+  if (D == 128)
+    hipLaunchKernelGGL(attn_tail_fold_kernel<128>, dim3((unsigned)tail), dim3(256), 0, stream, a);
+  else
+    hipLaunchKernelGGL(attn_tail_fold_kernel<64>, dim3((unsigned)tail), dim3(256), 0, stream, a);
+  return hip_fail(hipGetLastError(), "attn tail fold launch");
 }
 
 }  // namespace dt

@@ -98,14 +98,25 @@ static int fill_common(AttnArgs& a, const void* q, int32_t B, int32_t Sq, int32_
   return DT_OK;
 }
 
-extern "C" int dt_attn_seg_jobs_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D, int64_t q_sb,
-                                    int64_t q_ss, int64_t q_sh, int32_t n_chunks, const void* const* k_ptrs,
-                                    const void* const* v_ptrs, const int32_t* kv_lens, const int64_t* kv_sb,
-                                    int64_t kv_ss, int64_t kv_sh, int32_t n_jobs, const int32_t* job_begin,
-                                    const int32_t* job_chunks, const int32_t* entry_kv_begin,
-                                    const int32_t* entry_kv_len, const int32_t* job_q_begin,
-                                    const int32_t* job_q_len, void* const* out_ptrs, float* const* lse_ptrs,
-                                    float softmax_scale, void* stream) {
+extern "C" int64_t dt_attn_workspace_bytes(void) { return kMaxTailSlots * (256 * 128 * 2 + 256 * 4); }
+
+static int check_workspace(const void* workspace, int64_t workspace_bytes) {
+  if (workspace && (!aligned16(workspace) || workspace_bytes < 0)) {
+    set_error("workspace must be 16-byte aligned with a non-negative size");
+    return DT_ERR_INVALID;
+  }
+  return DT_OK;
+}
+
+extern "C" int dt_attn_seg_jobs_ws_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D, int64_t q_sb,
+                                       int64_t q_ss, int64_t q_sh, int32_t n_chunks, const void* const* k_ptrs,
+                                       const void* const* v_ptrs, const int32_t* kv_lens, const int64_t* kv_sb,
+                                       int64_t kv_ss, int64_t kv_sh, int32_t n_jobs, const int32_t* job_begin,
+                                       const int32_t* job_chunks, const int32_t* entry_kv_begin,
+                                       const int32_t* entry_kv_len, const int32_t* job_q_begin,
+                                       const int32_t* job_q_len, void* const* out_ptrs, float* const* lse_ptrs,
+                                       float softmax_scale, void* workspace, int64_t workspace_bytes, void* stream) {
+  if (int rc = check_workspace(workspace, workspace_bytes)) return rc;
   AttnArgs a{};
   if (int rc = fill_common(a, q, B, Sq, H, D, q_sb, q_ss, q_sh, n_chunks, k_ptrs, v_ptrs, kv_lens, kv_sb, kv_ss, kv_sh,
                            softmax_scale))
@@ -167,7 +178,21 @@ extern "C" int dt_attn_seg_jobs_fwd(const void* q, int32_t B, int32_t Sq, int32_
   a.nqt = (longest + 255) / 256;
   a.total = B * H * a.nqt;
   a.per_xcd = (a.total + 7) / 8;
-  return launch_attn(a, D, n_jobs, (hipStream_t)stream);
+  // the tail of the launch is only split when every job covers all query rows
+  return launch_attn(a, D, n_jobs, (hipStream_t)stream, workspace, workspace_bytes, job_q_begin == nullptr);
+}
+
+extern "C" int dt_attn_seg_jobs_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D, int64_t q_sb,
+                                    int64_t q_ss, int64_t q_sh, int32_t n_chunks, const void* const* k_ptrs,
+                                    const void* const* v_ptrs, const int32_t* kv_lens, const int64_t* kv_sb,
+                                    int64_t kv_ss, int64_t kv_sh, int32_t n_jobs, const int32_t* job_begin,
+                                    const int32_t* job_chunks, const int32_t* entry_kv_begin,
+                                    const int32_t* entry_kv_len, const int32_t* job_q_begin,
+                                    const int32_t* job_q_len, void* const* out_ptrs, float* const* lse_ptrs,
+                                    float softmax_scale, void* stream) {
+  return dt_attn_seg_jobs_ws_fwd(q, B, Sq, H, D, q_sb, q_ss, q_sh, n_chunks, k_ptrs, v_ptrs, kv_lens, kv_sb, kv_ss, kv_sh,
+                                 n_jobs, job_begin, job_chunks, entry_kv_begin, entry_kv_len, job_q_begin, job_q_len,
+                                 out_ptrs, lse_ptrs, softmax_scale, nullptr, 0, stream);
 }
 
 extern "C" int dt_attn_jobs_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D, int64_t q_sb, int64_t q_ss,
@@ -195,15 +220,17 @@ extern "C" int dt_attn_chunk_fwd(const void* q, const void* k, const void* v, vo
                           lses, softmax_scale, stream);
 }
 
-extern "C" int dt_attn_sched_seg_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D, int64_t q_sb,
-                                     int64_t q_ss, int64_t q_sh, int32_t n_chunks, const void* const* k_ptrs,
-                                     const void* const* v_ptrs, const int32_t* kv_lens, const int64_t* kv_sb,
-                                     int64_t kv_ss, int64_t kv_sh, const int32_t* dev_compute_ids,
-                                     const int32_t* dev_count, int32_t max_jobs, void* slot_out,
-                                     int64_t slot_out_stride, float* slot_lse, int64_t slot_lse_stride, int32_t diag,
-                                     void* diag_out, float* diag_lse, int32_t n_seg, const int32_t* seg_q_begin,
-                                     const int32_t* seg_q_len, const int32_t* seg_kv_begin,
-                                     const int32_t* seg_kv_len, float softmax_scale, void* stream) {
+extern "C" int dt_attn_sched_seg_ws_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D, int64_t q_sb,
+                                        int64_t q_ss, int64_t q_sh, int32_t n_chunks, const void* const* k_ptrs,
+                                        const void* const* v_ptrs, const int32_t* kv_lens, const int64_t* kv_sb,
+                                        int64_t kv_ss, int64_t kv_sh, const int32_t* dev_compute_ids,
+                                        const int32_t* dev_count, int32_t max_jobs, void* slot_out,
+                                        int64_t slot_out_stride, float* slot_lse, int64_t slot_lse_stride,
+                                        int32_t diag, void* diag_out, float* diag_lse, int32_t n_seg,
+                                        const int32_t* seg_q_begin, const int32_t* seg_q_len,
+                                        const int32_t* seg_kv_begin, const int32_t* seg_kv_len, float softmax_scale,
+                                        void* workspace, int64_t workspace_bytes, void* stream) {
+  if (int rc = check_workspace(workspace, workspace_bytes)) return rc;
   AttnArgs a{};
   if (int rc = fill_common(a, q, B, Sq, H, D, q_sb, q_ss, q_sh, n_chunks, k_ptrs, v_ptrs, kv_lens, kv_sb, kv_ss, kv_sh,
                            softmax_scale))
@@ -276,7 +303,22 @@ extern "C" int dt_attn_sched_seg_fwd(const void* q, int32_t B, int32_t Sq, int32
   a.diag = diag;
   a.diag_out = static_cast<__bf16*>(diag_out);
   a.diag_lse = diag_lse;
-  return launch_attn(a, D, jobs, (hipStream_t)stream);
+  return launch_attn(a, D, jobs, (hipStream_t)stream, workspace, workspace_bytes, n_seg == 0);
+}
+
+extern "C" int dt_attn_sched_seg_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D, int64_t q_sb,
+                                     int64_t q_ss, int64_t q_sh, int32_t n_chunks, const void* const* k_ptrs,
+                                     const void* const* v_ptrs, const int32_t* kv_lens, const int64_t* kv_sb,
+                                     int64_t kv_ss, int64_t kv_sh, const int32_t* dev_compute_ids,
+                                     const int32_t* dev_count, int32_t max_jobs, void* slot_out,
+                                     int64_t slot_out_stride, float* slot_lse, int64_t slot_lse_stride, int32_t diag,
+                                     void* diag_out, float* diag_lse, int32_t n_seg, const int32_t* seg_q_begin,
+                                     const int32_t* seg_q_len, const int32_t* seg_kv_begin,
+                                     const int32_t* seg_kv_len, float softmax_scale, void* stream) {
+  return dt_attn_sched_seg_ws_fwd(q, B, Sq, H, D, q_sb, q_ss, q_sh, n_chunks, k_ptrs, v_ptrs, kv_lens, kv_sb, kv_ss,
+                                  kv_sh, dev_compute_ids, dev_count, max_jobs, slot_out, slot_out_stride, slot_lse,
+                                  slot_lse_stride, diag, diag_out, diag_lse, n_seg, seg_q_begin, seg_q_len,
+                                  seg_kv_begin, seg_kv_len, softmax_scale, nullptr, 0, stream);
 }
 
 extern "C" int dt_attn_sched_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D, int64_t q_sb, int64_t q_ss,

@@ -53,8 +53,26 @@ struct AttnArgs {
   int32_t n_seg;
   int32_t seg_q_begin[DT_MAX_SEGMENTS];
   int32_t seg_q_len[DT_MAX_SEGMENTS];
+  // Tail balancing (workspace launches only).  The workgroups of a launch are equal pieces of
+  // work, so its last round usually fills only part of the chip.  The main launch then leaves
+  // the work items with index >= tail_idx0 of job tail_job alone (tail_job < 0: nothing is left);
+  // extra grid planes behind the jobs run each of them as part_ways workgroups over disjoint
+  // ranges of key tiles that write partial states into the workspace (same launch, so a part
+  // starts as soon as a CU is free), and a small second kernel folds the parts into the
+  // destination.
+  int32_t n_jobs;      // grid planes (blockIdx.y) that are jobs; planes behind them hold tail parts
+  int32_t tail_job;
+  int32_t tail_idx0;
+  int32_t tail_items;  // tail items per XCD lane of the grid (= tail workgroup slots / 8)
+  int32_t part_ways;
+  __bf16* ws_out;   // [slot][256 queries][D]
+  float* ws_lse;    // [slot][256]
 };
 
-int launch_attn(const AttnArgs& a, int D, int n_jobs, hipStream_t stream);
+// Workspace bytes the tail balancing can use at most (what dt_attn_workspace_bytes reports).
+constexpr int64_t kMaxTailSlots = 1536;
+
+int launch_attn(const AttnArgs& a, int D, int n_jobs, hipStream_t stream, void* workspace = nullptr,
+                int64_t workspace_bytes = 0, bool balance = false);
 
 }  // namespace dt

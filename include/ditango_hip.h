@@ -161,6 +161,39 @@ int dt_attn_sched_seg_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32
                           float softmax_scale, void* stream);
 
 /*
+ * The two launches above with a workspace (device memory, 16-byte aligned, at most
+ * dt_attn_workspace_bytes() are used; NULL or too small: plain launch).  All workgroups of an
+ * attention launch are equal pieces of work, so its last round usually fills only part of the
+ * chip; with a workspace the work items of that round are each cut into several ranges of key
+ * tiles that run side by side and write partial states into the workspace, and a small kernel
+ * folds them into the destination -- 2 to 8 % off a launch.  Used only when every job covers all
+ * query rows.  Calls that share a workspace must not overlap (same stream, or disjoint
+ * workspaces).  No counterpart in the reference.
+ */
+int64_t dt_attn_workspace_bytes(void);
+int dt_attn_seg_jobs_ws_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D,
+                            int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
+                            int32_t n_chunks, const void* const* k_ptrs, const void* const* v_ptrs,
+                            const int32_t* kv_lens, const int64_t* kv_stride_b,
+                            int64_t kv_stride_s, int64_t kv_stride_h,
+                            int32_t n_jobs, const int32_t* job_begin, const int32_t* job_chunks,
+                            const int32_t* entry_kv_begin, const int32_t* entry_kv_len,
+                            const int32_t* job_q_begin, const int32_t* job_q_len,
+                            void* const* out_ptrs, float* const* lse_ptrs,
+                            float softmax_scale, void* workspace, int64_t workspace_bytes, void* stream);
+int dt_attn_sched_seg_ws_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D,
+                             int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
+                             int32_t n_chunks, const void* const* k_ptrs, const void* const* v_ptrs,
+                             const int32_t* kv_lens, const int64_t* kv_stride_b,
+                             int64_t kv_stride_s, int64_t kv_stride_h,
+                             const int32_t* dev_compute_ids, const int32_t* dev_count, int32_t max_jobs,
+                             void* slot_out, int64_t slot_out_stride, float* slot_lse, int64_t slot_lse_stride,
+                             int32_t diag, void* diag_out, float* diag_lse,
+                             int32_t n_seg, const int32_t* seg_q_begin, const int32_t* seg_q_len,
+                             const int32_t* seg_kv_begin, const int32_t* seg_kv_len,
+                             float softmax_scale, void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
  * N-way LSE merge: lse = logsumexp_i lse_i, out = sum_i exp(lse_i - lse) out_i.
  * Replaces the chain of update_out_and_lse / _update_out_and_lse calls
  * (utils.py:24-84; called at core/attention.py:116,144,194,196,213 and

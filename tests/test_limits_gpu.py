@@ -111,3 +111,76 @@ def test_c_abi_rejects_without_launching(hip):
     torch.cuda.synchronize()
     assert (out.float() == 7.0).all()                                                # nothing ran
     assert call(q.data_ptr()) == 0
+
+
+@pytest.mark.parametrize("D,H,nq,lens,jobs", [
+    (128, 8, 40, [2610], [[0]]),                       # 320 items: 64 left over -> cut in parts; odd part sizes
+    (64, 8, 36, [2600, 2500], [[0], [1]]),             # two jobs of 288 items, 64 left over in the last
+    (128, 8, 43, [2000, 0, 1900], [[0, 1, 2]]),        # one job over several chunks (an empty one among them)
+    (128, 8, 33, [2000], [[0]]),                       # 264 items: 8 left over
+])
+def test_tail_balancing_matches_plain_launch_and_oracle(hip, D, H, nq, lens, jobs):
+    """With a workspace the last round of workgroups runs as key-range parts folded by a second
+    kernel: same states as the plain launch up to the extra bf16 rounding of the parts."""
+    B, Sq = 1, 256 * nq - 19
+    g = torch.Generator().manual_seed(D + nq)
+    q = (torch.randn(B, Sq, H, D, generator=g) * 1.3).bfloat16()
+    ks = [torch.randn(B, n, H, D, generator=g).bfloat16() for n in lens]
+    vs = [torch.randn(B, n, H, D, generator=g).bfloat16() for n in lens]
+    live = [c for c, n in enumerate(lens) if n > 0]
+    table = hip.ChunkTable([k.cuda() for k in ks], [v.cuda() for v in vs])
+    ws = hip.attn_workspace("cuda")
+    dq = q.cuda()
+
+    def run(workspace):
+        outs = [torch.zeros(B, Sq, H, D, dtype=torch.bfloat16, device="cuda") for _ in jobs]
+        lses = [torch.zeros(B, H, Sq, dtype=torch.float32, device="cuda") for _ in jobs]
+        hip.attn_jobs_fwd(dq, table, jobs, outs, lses, workspace=workspace)
+        torch.cuda.synchronize()
+        return outs, lses
+
+    po, pl = run(None)
+    bo, bl = run(ws)
+    changed = 0
+    for j in range(len(jobs)):
+        changed += int((po[j] != bo[j]).any())
+        assert (po[j].float() - bo[j].float()).abs().max() <= 2.0 ** -7 * po[j].float().abs().max()
+        assert (pl[j] - bl[j]).abs().max() <= 1e-5
+    assert changed > 0, "the balanced launch was expected to take the split path for this shape"
+    # a sample of query rows, the tail items (last rows of the last heads) included, against the oracle
+    rows = torch.cat([torch.arange(0, 64), torch.arange(Sq - 300, Sq)])
+    for j, chunks in enumerate(jobs):
+        cs = [c for c in chunks if c in live]
+        ref_out, ref_lse = om.full_attention(q[:, rows], [ks[c] for c in cs], [vs[c] for c in cs])
+        _check(bo[j][:, rows.cuda()], bl[j][:, :, rows.cuda()], ref_out, ref_lse, f"balanced job {j}")
+
+
+def test_tail_balancing_in_the_device_scheduled_launch(hip):
+    B, H, D, C = 1, 8, 128, 3
+    Sq = 256 * 36
+    g = torch.Generator().manual_seed(77)
+    q = torch.randn(B, Sq, H, D, generator=g).bfloat16().cuda()
+    ks = [torch.randn(B, 4000, H, D, generator=g).bfloat16().cuda() for _ in range(C)]
+    vs = [torch.randn(B, 4000, H, D, generator=g).bfloat16().cuda() for _ in range(C)]
+    table = hip.ChunkTable(ks, vs)
+    ids = torch.tensor([1, 2, 0], dtype=torch.int32, device="cuda")
+    cnt = torch.tensor([2], dtype=torch.int32, device="cuda")
+
+    def run(workspace, max_jobs):
+        ao = torch.zeros(C, B, Sq, H, D, dtype=torch.bfloat16, device="cuda")
+        al = torch.zeros(C, B, H, Sq, device="cuda")
+        do = torch.zeros(B, Sq, H, D, dtype=torch.bfloat16, device="cuda")
+        dl = torch.zeros(B, H, Sq, device="cuda")
+        hip.attn_sched_fwd(q, table, ids, cnt, max_jobs, ao, al, 2, do, dl, workspace=workspace)
+        torch.cuda.synchronize()
+        return ao, al, do, dl
+
+    plain = run(None, 2)
+    for max_jobs in (2, 3):   # 3: the tail belongs to a job the device list leaves idle
+        bal = run(hip.attn_workspace("cuda"), max_jobs)
+        for p, b in zip(plain, bal):
+            assert (p.float() - b.float()).abs().max() <= max(1e-5, 2.0 ** -7 * float(p.float().abs().max()))
+        assert (bal[0][0] == 0).all()      # chunk 0 was not scheduled
+        if max_jobs == 2:
+            # 2 x 288 items leave 64 for the last round: the split path ran (its parts round differently)
+            assert any(bool((p != b).any()) for p, b in zip(plain, bal))
