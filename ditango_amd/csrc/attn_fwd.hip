@@ -656,11 +656,14 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
 }
 
 // Folds the part_ways partial states of every tail item into the item's rows of its destination.
-// One workgroup per item; a group of D/8 lanes owns a row.
+// One workgroup per item and slice of 256 / (D/8) rows; a group of D/8 lanes owns a row.
 template <int D>
 __global__ __launch_bounds__(256) void attn_tail_fold_kernel(const AttnArgs a) {
-  const int xcd = blockIdx.x & (kXcds - 1);
-  const int u = blockIdx.x >> 3;
+  constexpr int kSlices = kBQ / (256 / (D / 8));
+  const int slot_id = blockIdx.x / kSlices;
+  const int slice = blockIdx.x - slot_id * kSlices;
+  const int xcd = slot_id & (kXcds - 1);
+  const int u = slot_id >> 3;
   const int idx = a.tail_idx0 + u;
   const int item = xcd * a.per_xcd + idx;
   if (idx >= a.per_xcd || item >= a.total) return;
@@ -686,10 +689,10 @@ __global__ __launch_bounds__(256) void attn_tail_fold_kernel(const AttnArgs a) {
   const int rr = threadIdx.x / kLanes;
   const int cc = threadIdx.x % kLanes;
   const int64_t slot0 = ((int64_t)u * kXcds + xcd) * a.part_ways;
-  for (int r0 = 0; r0 < kBQ; r0 += kRows) {
-    const int row = r0 + rr;
+  {
+    const int row = slice * kRows + rr;
     const int qg = qt * kBQ + row;
-    if (qg >= a.Sq) continue;
+    if (qg >= a.Sq) return;
     float m = -INFINITY;
     for (int p = 0; p < a.part_ways; ++p) m = fmaxf(m, a.ws_lse[(slot0 + p) * kBQ + row]);
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -819,9 +822,9 @@ int launch_attn(const AttnArgs& a_in, int D, int n_jobs, hipStream_t stream, voi
   const int part_planes = (a.tail_items * ways + a.per_xcd - 1) / a.per_xcd;
   if (int rc = launch_dim(a, D, dim3((unsigned)slots_per_job, (unsigned)(n_jobs + part_planes), 1), stream)) return rc;
   if (D == 128)
-    hipLaunchKernelGGL(attn_tail_fold_kernel<128>, dim3((unsigned)tail), dim3(256), 0, stream, a);
+    hipLaunchKernelGGL(attn_tail_fold_kernel<128>, dim3((unsigned)tail * 16), dim3(256), 0, stream, a);
   else
-    hipLaunchKernelGGL(attn_tail_fold_kernel<64>, dim3((unsigned)tail), dim3(256), 0, stream, a);
+    hipLaunchKernelGGL(attn_tail_fold_kernel<64>, dim3((unsigned)tail * 8), dim3(256), 0, stream, a);
   return hip_fail(hipGetLastError(), "attn tail fold launch");
 }
 
