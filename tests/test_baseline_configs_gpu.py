@@ -217,15 +217,16 @@ def test_attention_is_deterministic_at_hunyuan_shape(hip):
     ks = [torch.randn(B, Sk, H, D, generator=g, device="cuda").bfloat16() for _ in range(2)]
     vs = [torch.randn(B, Sk, H, D, generator=g, device="cuda").bfloat16() for _ in range(2)]
     table = hip.ChunkTable(ks, vs)
-    ref = None
-    for i in range(5):
-        outs = [torch.empty(B, Sq, H, D, dtype=torch.bfloat16, device="cuda") for _ in range(3)]
-        lses = [torch.empty(B, H, Sq, dtype=torch.float32, device="cuda") for _ in range(3)]
-        hip.attn_jobs_fwd(q, table, [[0], [1], [0, 1]], outs, lses)
-        torch.cuda.synchronize()
-        if ref is None:
-            ref = (outs, lses)
-            assert all(torch.isfinite(l).all() for l in lses)
-        else:
-            for j in range(3):
-                assert torch.equal(outs[j], ref[0][j]) and torch.equal(lses[j], ref[1][j]), f"run {i} job {j}"
+    for ws in (None, hip.attn_workspace("cuda")):   # plain launch, and with the tail of the launch run as parts
+        ref = None
+        for i in range(5):
+            outs = [torch.empty(B, Sq, H, D, dtype=torch.bfloat16, device="cuda") for _ in range(3)]
+            lses = [torch.empty(B, H, Sq, dtype=torch.float32, device="cuda") for _ in range(3)]
+            hip.attn_jobs_fwd(q, table, [[0], [1], [0, 1]], outs, lses, workspace=ws)
+            torch.cuda.synchronize()
+            if ref is None:
+                ref = (outs, lses)
+                assert all(torch.isfinite(l).all() for l in lses)
+            else:
+                for j in range(3):
+                    assert torch.equal(outs[j], ref[0][j]) and torch.equal(lses[j], ref[1][j]), f"run {i} job {j}"
