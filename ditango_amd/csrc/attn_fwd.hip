@@ -791,18 +791,20 @@ int launch_attn(const AttnArgs& a_in, int D, int n_jobs, hipStream_t stream, voi
     } else {
       for (int e = a.job_begin[n_jobs - 1]; e < a.job_begin[n_jobs]; ++e) n_tiles += (a.entry_kv_len[e] + kBK - 1) / kBK;
     }
-    // Measured on the HunyuanVideo and Step-Video shares: a part costs about 10 tiles on top of its
-    // own (start-up, epilogue, partial state), so many small parts only pay when they all run at once.
-    constexpr double kPartOverhead = 10.0;
+    // Measured on the HunyuanVideo, Step-Video and CogVideoX shares: a part costs about 6 tiles on
+    // top of its own (start-up, epilogue, partial state) when all parts run at once and about 10
+    // when they take several rounds, so many small parts only pay in the first case.
+    constexpr double kPartOverheadOneRound = 6.0, kPartOverheadRounds = 10.0;
     constexpr double kFoldOverhead = 4.0;  // the fold kernel's launch
     const int64_t n = (int64_t)n_jobs * slots_per_job;
     const int rem = (int)(n % cus);
     const int64_t cap = std::min<int64_t>(workspace_bytes / slot_bytes, kMaxTailSlots);
     if (rem > 0 && rem <= slots_per_job && rem < n && n_tiles >= 16) {
-      double best = 0.2 * n_tiles;  // least gain worth the extra kernel
+      double best = 0.1 * n_tiles;  // least gain worth the extra kernel
       for (int w = 2; w <= 16; ++w) {
         if ((int64_t)rem * w > cap || n_tiles / w < 6) break;
-        const double split = (double)(((int64_t)rem * w + cus - 1) / cus) * ((double)n_tiles / w + kPartOverhead) + kFoldOverhead;
+        const int rounds = (int)(((int64_t)rem * w + cus - 1) / cus);
+        const double split = rounds * ((double)n_tiles / w + (rounds == 1 ? kPartOverheadOneRound : kPartOverheadRounds)) + kFoldOverhead;
         if (n_tiles - split > best) {
           best = n_tiles - split;
           tail = rem;
