@@ -184,3 +184,35 @@ def test_tail_balancing_in_the_device_scheduled_launch(hip):
         if max_jobs == 2:
             # 2 x 288 items leave 64 for the last round: the split path ran (its parts round differently)
             assert any(bool((p != b).any()) for p, b in zip(plain, bal))
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_tail_balancing_random_launches_match_plain(hip, seed):
+    """Random launches big enough to leave a partial last round: balanced == plain up to the parts' rounding."""
+    import random
+    rng = random.Random(seed)
+    D = rng.choice([64, 128])
+    H = rng.choice([8, 16])
+    nq = rng.randrange(17, 49) if H == 16 else rng.randrange(33, 60)
+    B, Sq = 1, 256 * nq - rng.randrange(0, 200)
+    C = rng.choice([1, 2, 3])
+    lens = [rng.randrange(1200, 3500) for _ in range(C)]
+    jobs = [[c] for c in range(C)] if rng.random() < 0.5 else [list(range(C))] + [[rng.randrange(C)]]
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    q = torch.randn(B, Sq, H, D, generator=g, device="cuda").bfloat16()
+    ks = [torch.randn(B, n, H, D, generator=g, device="cuda").bfloat16() for n in lens]
+    vs = [torch.randn(B, n, H, D, generator=g, device="cuda").bfloat16() for n in lens]
+    table = hip.ChunkTable(ks, vs)
+    print(f"case seed={seed} D={D} H={H} Sq={Sq} lens={lens} jobs={jobs} items={H * nq}", flush=True)
+    res = []
+    for ws in (None, hip.attn_workspace("cuda")):
+        outs = [torch.zeros(B, Sq, H, D, dtype=torch.bfloat16, device="cuda") for _ in jobs]
+        lses = [torch.zeros(B, H, Sq, dtype=torch.float32, device="cuda") for _ in jobs]
+        hip.attn_jobs_fwd(q, table, jobs, outs, lses, workspace=ws)
+        torch.cuda.synchronize()
+        res.append((outs, lses))
+    for j in range(len(jobs)):
+        po, bo = res[0][0][j].float(), res[1][0][j].float()
+        assert torch.isfinite(bo).all()
+        assert (po - bo).abs().max() <= 2.0 ** -7 * po.abs().max()
+        assert (res[0][1][j] - res[1][1][j]).abs().max() <= 1e-5
