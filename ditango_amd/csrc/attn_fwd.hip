@@ -60,8 +60,7 @@ constexpr int kThreads = kWaves * 64;
 constexpr int kBQ = kWaves * 32;  // queries per workgroup
 constexpr int kBK = 64;           // keys per tile
 constexpr int kXcds = 8;
-constexpr int kNumKBuf = 2;
-constexpr int kNumVBuf = 3;
+constexpr int kNumBuf = 4;        // LDS buffers per operand; a tile uses buffer (tile & 3)
 #ifndef DT_RING
 #define DT_RING 4
 #endif
@@ -84,13 +83,29 @@ __device__ __forceinline__ void phase_barrier() {
 // operands.  Register-only code may otherwise migrate across an asm statement; tied to it,
 // the phase's work stays on its own side (the vector phase produces P^T, the matrix phase
 // produces S^T and updates O^T).
-template <typename V>
+// After a vector phase the wavefront also waits for the direct-to-LDS tile loads it issued two
+// vector phases ago (all but the kInFlight newest): behind the barrier they are visible to
+// every wavefront.
+template <int kInFlight, typename V>
 __device__ __forceinline__ void phase_barrier_after_vector(V (&p)[2][2]) {
   __builtin_amdgcn_sched_barrier(0);
-  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier"
-               : "+v"(p[0][0]), "+v"(p[0][1]), "+v"(p[1][0]), "+v"(p[1][1])
-               :
-               : "memory");
+  if constexpr (kInFlight == 8) {
+    asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier"
+                 : "+v"(p[0][0]), "+v"(p[0][1]), "+v"(p[1][0]), "+v"(p[1][1])
+                 :
+                 : "memory");
+  } else if constexpr (kInFlight == 4) {
+    asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier"
+                 : "+v"(p[0][0]), "+v"(p[0][1]), "+v"(p[1][0]), "+v"(p[1][1])
+                 :
+                 : "memory");
+  } else {
+    static_assert(kInFlight == 2, "loads in flight across the barrier: 2, 4 or 8");
+    asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)\n\ts_barrier"
+                 : "+v"(p[0][0]), "+v"(p[0][1]), "+v"(p[1][0]), "+v"(p[1][1])
+                 :
+                 : "memory");
+  }
   __builtin_amdgcn_sched_barrier(0);
 }
 template <typename V, int NO>
@@ -117,24 +132,34 @@ constexpr float kSumLimit = 4096.0f;
 
 template <int D>
 struct Tile {
-  // Both tiles sit in LDS as [key][d] rows, padded instead of swizzled: every operand read is
-  // then "lane base + compile-time constant" (immediate offsets, no address arithmetic in the
-  // loop).  K rows are padded by 16 bytes: the 16 lanes of a ds_read_b128 pass read 16 different
-  // rows at the same column and land in 16 distinct 16-byte bank groups.  V rows are padded by
-  // 64 bytes: a transposing 8-byte read pass touches 4 rows x 2 column groups, which 64-byte
-  // row shifts spread over all banks.
-  static constexpr int kPitchK = D * 2 + 16;
-  static constexpr int kPitchV = D * 2 + 64;
+  // Both tiles sit in LDS as [key][d] rows WITHOUT padding: a tile arrives through direct-to-LDS
+  // buffer loads, and one such instruction writes 1 KB of consecutive LDS bytes (lane L -> bytes
+  // 16 L .. 16 L + 15), so rows cannot be padded.  Bank conflicts are avoided by swizzling instead:
+  // which 16 bytes of global memory a lane fetches is free, so a row's 16-byte chunks (K) or
+  // 64-byte segments (V) are stored XOR-permuted by a function of the row.
+  //   K: chunk c of row r sits at chunk position c ^ swz_k(r); the 16 lanes of a ds_read_b128 pass
+  //      read 16 rows at the same c and land in 16 distinct 16-byte bank groups.
+  //   V: segment g of row r sits at segment position g ^ swz_v(r); a transposing 8-byte read pass
+  //      touches 4 rows x one 64-byte segment, which land in the four quarters of the banks.
+  // swz_v only depends on row bits that the immediate row steps of the operand reads (multiples
+  // of 4 rows) leave alone; the per-lane part of the swizzle is folded into a few precomputed
+  // address registers (one per k-step for K, one per 32 columns for V).
+  static constexpr int kRowBytes = D * 2;
   static constexpr int kChunks = D / 8;               // 16-byte chunks per row
-  static constexpr int kBytesK = kBK * kPitchK;
-  static constexpr int kBytesV = kBK * kPitchV;
-  static constexpr int kOffV = kNumKBuf * kBytesK;    // V buffers follow the K buffers
-  static constexpr int kLoads = kBK * kChunks / kThreads;  // 16-byte loads per thread and tile (2 or 1)
-  static constexpr int kRowStep = kThreads / kChunks;
+  static constexpr int kSegs = D / 32;                // 64-byte segments per row
+  static constexpr int kBytesK = kBK * kRowBytes;
+  static constexpr int kBytesV = kBK * kRowBytes;
+  static constexpr int kOffV = kNumBuf * kBytesK;     // V buffers follow the K buffers
+  static constexpr int kBlocks = kBytesK / 1024;      // direct-load instructions per tile and operand
+  static constexpr int kLoads = kBlocks / kWaves;     // ... per wavefront (2 or 1)
+  static constexpr int kRowsPerBlock = 1024 / kRowBytes;
   static constexpr int kPitchO = D * 2 + 16;          // epilogue row pitch
-  static constexpr int kLdsTiles = kNumKBuf * kBytesK + kNumVBuf * kBytesV;
+  static constexpr int kLdsTiles = kNumBuf * (kBytesK + kBytesV);
   static constexpr int kLdsEpilogue = kWaves * 32 * kPitchO;
   static constexpr int kLdsBytes = kLdsTiles > kLdsEpilogue ? kLdsTiles : kLdsEpilogue;
+  static_assert(D == 128 || D == 64, "swizzles are written for these two head dimensions");
+  __device__ static constexpr int swz_k(int row) { return D == 128 ? (row & 15) : ((row >> 1) & 7); }
+  __device__ static constexpr int swz_v(int row) { return D == 128 ? (row & 3) : ((row >> 1) & 1); }
 };
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -307,65 +332,60 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     n_tiles = t1 - t0;
   }
 
-  // thread -> tile elements, the same for K and V: 16-byte chunk kc of rows kr0 + i*kRowStep
-  const int kc = tid % T::kChunks;
-  const int kr0 = tid / T::kChunks;
+  // ---- tile loads: global memory -> LDS without passing through registers ---------------
+  // A wavefront brings in kLoads 1 KB blocks of every K tile and of every V tile (block
+  // wave + 8 i = rows kRowsPerBlock * (wave + 8 i) ...).  Lane L of a load lands at LDS bytes
+  // 16 L .. 16 L + 15 of the block, i.e. at row L / kChunks, chunk position L % kChunks; it
+  // therefore fetches the chunk of global memory that the swizzle assigns to that position.
+  // Raw buffer loads: the descriptor (base of the tile's first key for this batch and head,
+  // number of valid bytes) lives in scalar registers, and rows past the end of the chunk fail
+  // the hardware bounds check and arrive as zeros (their scores are masked to -inf; zero V rows
+  // add nothing).
   const uint32_t row_bytes = (uint32_t)a.kv_ss * 2u;
-  // byte offsets from the tile's first key, loop invariant
-  uint32_t koff[T::kLoads];
-#pragma unroll
-  for (int i = 0; i < T::kLoads; ++i) koff[i] = (uint32_t)(kr0 + i * T::kRowStep) * row_bytes + 16u * kc;
-
-  // Two register sets: the loads of a tile are issued TWO iterations before its LDS fill, so
-  // that a first-touch miss all the way to HBM (the workgroup that leads on its XCD takes one
-  // on every tile) is still hidden.  Tile X of a group uses set (X - pf) & 1.
-  u32x4 kreg[2][T::kLoads];
-  u32x4 vreg[2][T::kLoads];
-
+  uint32_t k_goff, v_goff;  // this lane's byte offset from the tile's first key, loop invariant
+  {
+    const int lrow = T::kRowsPerBlock * wave + lane / T::kChunks;  // + 8 * kRowsPerBlock * i
+    const int pos = lane % T::kChunks;
+    k_goff = (uint32_t)lrow * row_bytes + 16u * (uint32_t)(pos ^ T::swz_k(lrow));
+    v_goff = (uint32_t)lrow * row_bytes + 16u * (uint32_t)((((pos >> 2) ^ T::swz_v(lrow)) << 2) | (pos & 3));
+  }
+  static_assert((8 * T::kRowsPerBlock) % 16 == 0, "the swizzle must not depend on the load index");
   const int64_t tile_bytes = (int64_t)kBK * row_bytes;
-  // Loads this thread's share of the tile under the load cursor into registers and moves the
-  // cursor on.  Raw buffer loads: the descriptor (base of the tile's first key for this batch
-  // and head, number of valid bytes) lives in scalar registers, and rows past the end of the
-  // chunk fail the hardware bounds check and come back as zeros (their scores are masked to
-  // -inf; zero V rows add nothing).
-  auto load_tile = [&](auto set_tag) {
-    constexpr int kSet = decltype(set_tag)::value;
-    // Past the last tile the loads are still issued, against an empty descriptor (they return
-    // zeros without touching memory): with the same number of loads in every iteration the
-    // counter the LDS fill waits on is static, and a fill waits for ITS tile only, not for the
-    // loads issued one iteration later.
+  typedef __attribute__((address_space(3))) uint8_t* lds_ptr_t;
+  // Issues this wavefront's loads of K of the tile under the load cursor (tile X, into K buffer
+  // X & 3) and of V of the tile before it (V is needed two phases later than K, so its loads run
+  // one tile behind and reuse the descriptor the previous call made for K), and moves the cursor
+  // on.  Past the last tile the loads are still issued, against an empty descriptor (they store
+  // zeros without touching memory): with the same number of loads in every iteration the counter
+  // the barrier waits on is static.
+  const uint8_t* prev_v = nullptr;  // V of the tile the previous call loaded K of
+  uint32_t prev_valid = 0u;
+  auto load_tile = [&](int kbuf) {
     const bool have = __builtin_expect(ld_seg < seg_end, 1);
     const uint32_t valid = have ? (uint32_t)(ld_left - 1) * row_bytes + (uint32_t)(D * 2) : 0u;
     const __amdgpu_buffer_rsrc_t rk =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(ld_k), 0, (int)valid, kRsrcFlags);
     const __amdgpu_buffer_rsrc_t rv =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(ld_v), 0, (int)valid, kRsrcFlags);
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(prev_v), 0, (int)prev_valid, kRsrcFlags);
+    prev_v = ld_v;
+    prev_valid = valid;
+    const int vbuf = (kbuf + kNumBuf - 1) & (kNumBuf - 1);
+    lds_ptr_t kdst = (lds_ptr_t)lds + kbuf * T::kBytesK + wave * 1024;
+    lds_ptr_t vdst = (lds_ptr_t)lds + T::kOffV + vbuf * T::kBytesV + wave * 1024;
 #pragma unroll
-    for (int i = 0; i < T::kLoads; ++i) kreg[kSet][i] = __builtin_amdgcn_raw_buffer_load_b128(rk, (int)koff[i], 0, 0);
+    for (int i = 0; i < T::kLoads; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, kdst + i * 8192, 16, (int)k_goff,
+                                               (int)(i * 8 * T::kRowsPerBlock * row_bytes), 0, 0);
 #pragma unroll
-    for (int i = 0; i < T::kLoads; ++i) vreg[kSet][i] = __builtin_amdgcn_raw_buffer_load_b128(rv, (int)koff[i], 0, 0);
+    for (int i = 0; i < T::kLoads; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, vdst + i * 8192, 16, (int)v_goff,
+                                               (int)(i * 8 * T::kRowsPerBlock * row_bytes), 0, 0);
     if (have) {
       ld_left -= kBK;
       ld_k += tile_bytes;
       ld_v += tile_bytes;
       if (__builtin_expect(ld_left <= 0, 0)) ld_next_chunk();
     }
-  };
-
-  // LDS write addresses of this thread within a K / V buffer (V is stored as it comes, [key][d];
-  // the transposition the second MFMA needs is done by the transposing LDS read)
-  const int kst = kr0 * T::kPitchK + 16 * kc;
-  const int vst = kr0 * T::kPitchV + 16 * kc;
-  auto store_tile = [&](int tile, auto set_tag) {
-    constexpr int kSet = decltype(set_tag)::value;
-    uint8_t* kbuf = lds + (tile % kNumKBuf) * T::kBytesK;
-    uint8_t* vbuf = lds + T::kOffV + (tile % kNumVBuf) * T::kBytesV;
-#pragma unroll
-    for (int i = 0; i < T::kLoads; ++i)
-      *reinterpret_cast<u32x4*>(kbuf + kst + i * T::kRowStep * T::kPitchK) = kreg[kSet][i];
-#pragma unroll
-    for (int i = 0; i < T::kLoads; ++i)
-      *reinterpret_cast<u32x4*>(vbuf + vst + i * T::kRowStep * T::kPitchV) = vreg[kSet][i];
   };
 
   // ---- accumulators ---------------------------------------------------------------------
@@ -378,26 +398,36 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   float l_run = 0.f;        // running sum over THIS lane's keys (halves combined at the end)
   const float c = a.scale_log2;
 
-  // operand read addresses of this lane within a K / V buffer
-  const int kld = key_of_row(col) * T::kPitchK + 16 * hh;
+  // operand read addresses of this lane within a K / V buffer (the lane's part of the swizzle)
+  uint32_t kld[D / 16];  // K fragment of k-step s: row key_of_row(col) (+32 for the second half tile)
+  {
+    const int krow = key_of_row(col);
+#pragma unroll
+    for (int s = 0; s < D / 16; ++s) kld[s] = krow * T::kRowBytes + 16 * ((2 * s + hh) ^ T::swz_k(krow));
+  }
   // V operand: this lane is source lane 4j+m of its 16-lane block and supplies keys 8*hh + j,
-  // d columns 16*(block parity) + 4m .. +3 of the fragment
-  const int vld = T::kOffV + (8 * hh + ((lane & 15) >> 2)) * T::kPitchV + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+  // d columns 16*(block parity) + 4m .. +3 of the fragment's 32-column segment
+  uint32_t vld[T::kSegs];
+  {
+    const int vrow = 8 * hh + ((lane & 15) >> 2);
+#pragma unroll
+    for (int g = 0; g < T::kSegs; ++g)
+      vld[g] = T::kOffV + vrow * T::kRowBytes + 64 * (g ^ T::swz_v(vrow)) + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+  }
 
   f32x16 s_acc[2];       // S^T of the tile whose softmax comes next
   bf16x8 p_frag[2][2];   // P^T of the tile whose P V product comes next
   int cp_valid = 0;      // keys that exist in the tile held in s_acc
 
-  // S^T = K Q^T for tile `tile` only (first matrix phase)
-  auto qk_only = [&](int tile) {
-    const uint8_t* kl = lds + kld + (tile % kNumKBuf) * T::kBytesK;
+  // S^T = K Q^T for tile 0 only (first matrix phase)
+  auto qk_only = [&]() {
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) s_acc[kb][r] = 0.f;
 #pragma unroll
       for (int s = 0; s < D / 16; ++s) {
-        const bf16x8 ka = *reinterpret_cast<const bf16x8*>(kl + kb * 32 * T::kPitchK + 32 * s);
+        const bf16x8 ka = *reinterpret_cast<const bf16x8*>(lds + kld[s] + kb * 32 * T::kRowBytes);
         s_acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[s], s_acc[kb], 0, 0, 0);
       }
     }
@@ -407,37 +437,43 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   // as ONE stream of MFMAs fed by a ring of LDS reads kept kRing fragments ahead, so that the
   // single wavefront of this SIMD that is in its matrix phase never waits for LDS latency.
   // (After the last tile the second half recomputes scores on a stale K buffer; they are unused.)
+  // U = tile & 3 picks the buffers at compile time: all operand reads use immediate offsets.
   constexpr int kPV = D / 32 * 4;       // fragments of the P V product
   constexpr int kQK = 2 * (D / 16);     // fragments of the score product
   constexpr int kFrags = kPV + kQK;
   constexpr int kRing = DT_RING;
+  // Where a wavefront issues its tile loads: at the start of its vector phase, or behind the
+  // MFMAs of its matrix phase (one phase later, and then awaited one call earlier).  At D = 64
+  // the vector phase is the longer one (half the MFMAs per softmax element) and the matrix
+  // phase has the room (measured +16 %); at D = 128 it is the other way round (+1.5 %).
+  constexpr bool kLoadAfterMatrix = D == 64;
   // The operand ring lives across the barrier in front of a matrix phase: its first kRing
   // fragments (V fragments of a tile completed at least a phase ago) are read at the END of the
   // preceding vector phase, so their LDS latency passes while the wavefront waits at the barrier
   // instead of in front of the first MFMA.
   bf16x8 ring[kRing];
-  auto v_frag = [&](const uint8_t* vl, int i) __attribute__((always_inline)) -> bf16x8 {
+  auto v_frag = [&](int vbuf, int i) __attribute__((always_inline)) -> bf16x8 {
     // 8 consecutive keys of one d column = two transposing reads of 4 keys each
     const int db = i >> 2, kb = (i >> 1) & 1, half = i & 1;
-    const uint8_t* p = vl + (32 * kb + 16 * half) * T::kPitchV + db * 64;
+    const uint8_t* p = lds + vld[db] + vbuf * T::kBytesV + (32 * kb + 16 * half) * T::kRowBytes;
     const s16x4 lo = lds_read_tr(p);
-    const s16x4 hi = lds_read_tr(p + 4 * T::kPitchV);
+    const s16x4 hi = lds_read_tr(p + 4 * T::kRowBytes);
     const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
     return __builtin_bit_cast(bf16x8, both);
   };
-  auto ring_prefill = [&](int tile) __attribute__((always_inline)) {
-    const uint8_t* vl = lds + vld + (tile % kNumVBuf) * T::kBytesV;
+  auto ring_prefill = [&](auto u_tag) __attribute__((always_inline)) {
+    constexpr int kU = decltype(u_tag)::value;
 #pragma unroll
-    for (int i = 0; i < kRing; ++i) ring[i] = v_frag(vl, i);
+    for (int i = 0; i < kRing; ++i) ring[i] = v_frag(kU, i);
   };
-  auto matrix_phase = [&](int tile) {
-    const uint8_t* vl = lds + vld + (tile % kNumVBuf) * T::kBytesV;
-    const uint8_t* kl = lds + kld + ((tile + 1) % kNumKBuf) * T::kBytesK;
+  auto matrix_phase = [&](auto u_tag) {
+    constexpr int kU = decltype(u_tag)::value;         // V buffer of this tile
+    constexpr int kUK = (kU + 1) & (kNumBuf - 1);      // K buffer of the next tile
     auto frag = [&](int i) -> bf16x8 {
-      if (i < kPV) return v_frag(vl, i);
+      if (i < kPV) return v_frag(kU, i);
       const int j = i - kPV;
       const int kb = j / (D / 16), sidx = j % (D / 16);
-      return *reinterpret_cast<const bf16x8*>(kl + kb * 32 * T::kPitchK + 32 * sidx);
+      return *reinterpret_cast<const bf16x8*>(lds + kld[sidx] + kUK * T::kBytesK + kb * 32 * T::kRowBytes);
     };
 #pragma unroll
     for (int i = 0; i < kFrags; ++i) {
@@ -475,42 +511,58 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     __builtin_amdgcn_sched_group_barrier(0x008, kRing, 0);
   };
 
-  // ---- prologue: tile 0 from everybody; the trailing group also brings its share of tile 1
-  //      and then waits one phase, which is what staggers the two groups ---------------------
-  using Set0 = std::integral_constant<int, 0>;
-  using Set1 = std::integral_constant<int, 1>;
-  const int pf = 1 + group;  // how many tiles ahead of its softmax a group fills LDS
-  load_tile(Set0{});
-  store_tile(0, Set0{});
-  if (group == 1) load_tile(Set0{});
-  phase_barrier();
-  if (group == 1) {
-    store_tile(1, Set0{});
-    phase_barrier();
+  // ---- prologue ---------------------------------------------------------------------------
+  // Schedule of the loads (phases are separated by workgroup barriers; group g runs the vector
+  // phase of tile t in phase 2t + g and its matrix phase in phase 2t + g + 1):
+  //   * in the vector phase of tile t a wavefront of group g issues its blocks of K of tile
+  //     t+3+g and of V of tile t+2+g, and waits for them at the end of the vector phase after
+  //     the next one, four phases later (a first-touch miss all the way to HBM is still hidden);
+  //   * K of tile X is first read in phase 2X-1 (scores, by group 0) and last in phase 2X, V of
+  //     tile X in phases 2X+1 and 2X+2: every block has arrived at least one barrier before its
+  //     first reader, and with four buffers per operand the buffer (X & 3) it overwrites was last
+  //     read (K of tile X-4: phase 2X-8, V of tile X-4: phase 2X-6) before the phase the load is
+  //     issued in (K: 2X-6 or 2X-7, V: 2X-4 or 2X-5).
+  // Here: K of tiles 0..2 and V of tiles 0..1 (group 1: one tile more); the trailing group then
+  // waits one phase, which is what staggers the two groups.  (The V half of
+  // the first call has no tile yet: it stores zeros into a buffer nobody reads.)
+  using U0 = std::integral_constant<int, 0>;
+  using U1 = std::integral_constant<int, 1>;
+  using U2 = std::integral_constant<int, 2>;
+  using U3 = std::integral_constant<int, 3>;
+  load_tile(0);
+  load_tile(1);
+  load_tile(2);
+  if (group == 1) load_tile(3);
+  // only K of tile 0 (the first call) has to be there for the first scores; what the later
+  // phases need is awaited by the barriers of the vector phases before them
+  if (group == 0) {
+    if constexpr (T::kLoads == 2) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+  } else {
+    if constexpr (T::kLoads == 2) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
   }
-  // first matrix phase: fetch two tiles ahead (sets 0 and 1), scores of tile 0
-  load_tile(Set0{});
-  load_tile(Set1{});
+  phase_barrier();
+  if (group == 1) phase_barrier();
+  // first matrix phase: scores of tile 0
   if (n_tiles > 0) {
-    qk_only(0);
+    qk_only();
     cp_valid = cp_left;
     cp_left -= kBK;
     if (cp_left <= 0) cp_next_chunk();
   }
   phase_barrier_after_matrix(s_acc, o_acc);
 
-  // one iteration = vector phase of tile t, then matrix phase (P V of tile t, scores of t+1);
-  // iteration t fills LDS from register set t & 1 and then refills that set from memory
-  auto iteration = [&](int t, auto set_tag) {
-    // ======== vector phase: LDS fill of a fetched tile, online softmax of tile t ========
-    // The fill goes first: its registers were loaded two iterations ago, and the latency of
-    // the LDS writes (which compete with the other group's operand reads) hides behind the softmax.
+  // one iteration = vector phase of tile t, then matrix phase (P V of tile t, scores of t+1)
+  auto iteration = [&](int t, auto u_tag) {
+    constexpr int kU = decltype(u_tag)::value;  // t & 3
+    // ======== vector phase: tile loads for later, online softmax of tile t ========
     // The vector phase runs at raised wave priority: where the two wavefronts of a SIMD compete for
     // the vector issue port, the one doing the softmax goes first.  With equal priorities the older
     // wavefront wins in either role and the phases of the two groups come out unequal (measured
     // 1.43k vs 1.24k cycles of vector work), so every other barrier waits for a squeezed softmax.
     __builtin_amdgcn_s_setprio(1);
-    store_tile(t + pf, set_tag);
+    if constexpr (!kLoadAfterMatrix) load_tile((kU + 3 + group) & (kNumBuf - 1));
     if (__builtin_expect(cp_valid < kBK, 0)) {
       // the empty asm has side effects as far as the compiler knows, which keeps this a real
       // branch: otherwise the selects below are hoisted out and run for every tile
@@ -579,26 +631,28 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
         }
     }
     l_run += rs0 + rs1;
-    ring_prefill(t);
-    phase_barrier_after_vector(p_frag);
+    ring_prefill(u_tag);
+    phase_barrier_after_vector<(kLoadAfterMatrix ? 2 : 4) * T::kLoads>(p_frag);
 
-    // ======== matrix phase: fetch ahead, O^T += V^T P^T (tile t), S^T = K Q^T (tile t+1) ========
+    // ======== matrix phase: O^T += V^T P^T (tile t), S^T = K Q^T (tile t+1) ========
     __builtin_amdgcn_s_setprio(0);
-    load_tile(set_tag);
-    matrix_phase(t);
+    matrix_phase(u_tag);
+    if constexpr (kLoadAfterMatrix) load_tile((kU + 3 + group) & (kNumBuf - 1));
     // the tile after the last one of this workgroup's range has no keys for it (it is the
-    // padding of an odd tile count, or belongs to the next part of a split item)
+    // padding of the tile count, or belongs to the next part of a split item)
     cp_valid = t + 1 < n_tiles ? cp_left : 0;
     cp_left -= kBK;
     if (cp_left <= 0) cp_next_chunk();
     phase_barrier_after_matrix(s_acc, o_acc);
   };
-  // Iterations come in pairs (one per register set); an odd tile count is rounded up with a tile
-  // that has no keys: its loads hit the empty descriptor, its scores are masked, it adds zeros.
-  const int n_iter = (n_tiles + 1) & ~1;
-  for (int t = 0; t < n_iter; t += 2) {
-    iteration(t, Set0{});
-    iteration(t + 1, Set1{});
+  // Iterations come in fours (one per LDS buffer); the tile count is rounded up with tiles that
+  // have no keys: their scores are masked, they add zeros.
+  const int n_iter = (n_tiles + 3) & ~3;
+  for (int t = 0; t < n_iter; t += 4) {
+    iteration(t, U0{});
+    iteration(t + 1, U1{});
+    iteration(t + 2, U2{});
+    iteration(t + 3, U3{});
   }
   // the leading group waits out the phase it is ahead
   if (group == 0) phase_barrier();
