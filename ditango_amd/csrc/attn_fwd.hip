@@ -11,18 +11,23 @@
 //   * The 8 wavefronts form two groups of 4 that run the same loop ONE PHASE
 //     APART ("ping-pong"): while group A issues the MFMAs of a tile
 //     (O^T += V^T P^T of the previous tile, then S^T = K Q^T of this one), group B
-//     runs the VALU half (online softmax of its tile, copying the next K/V tile
-//     from registers into LDS), and vice versa; a workgroup barrier separates the
+//     runs the VALU half (online softmax of its tile, issuing the loads of a later
+//     K/V tile), and vice versa; a workgroup barrier separates the
 //     phases.  Each SIMD holds one wavefront of either group, so its matrix pipe
 //     and its vector ALU are busy at the same time instead of taking turns.
-//   * KV is consumed in tiles of 64 keys, staged in LDS as they come, [key][d]:
-//     K in two buffers, V in three (the P V product of a tile runs one phase
-//     after its scores).  The second MFMA needs V^T; the transposition is done
-//     by the LDS read itself (ds_read_b64_tr_b16), so filling a tile is eight
-//     16-byte copies per thread and no ALU work.  Rows are padded so that all
-//     operand reads are bank-conflict free and use immediate offsets.  Tiles come
-//     in through raw buffer loads: descriptor in scalar registers, loop-invariant
-//     lane offsets, and rows past the end of a chunk read as zeros.
+//   * KV is consumed in tiles of 64 keys, staged in LDS as they come, [key][d],
+//     four buffers per operand.  A tile goes from global memory STRAIGHT into
+//     LDS (buffer loads with the LDS as destination: no registers, no LDS write
+//     instructions, no wait for them in the softmax), issued three (K) and two
+//     (V) tiles ahead of their first use.  Staging through registers cost a
+//     fifth of the loop's cycles: the fill's LDS writes queue up in front of the
+//     operand reads of the wavefronts that are issuing MFMAs.  Such a load writes
+//     1 KB of consecutive LDS bytes, so rows are not padded but XOR-swizzled (the
+//     lane picks which 16 bytes of global memory it fetches); operand reads stay
+//     bank-conflict free and use immediate offsets from a few per-lane address
+//     registers.  The second MFMA needs V^T; the transposition is done by the
+//     LDS read itself (ds_read_b64_tr_b16).  The buffer descriptor lives in
+//     scalar registers, and rows past the end of a chunk arrive as zeros.
 //   * Scores are computed TRANSPOSED, S^T = K Q^T, with v_mfma_f32_32x32x16_bf16:
 //     in the accumulator layout a lane then owns ONE query (column lane%32) and
 //     16 of the 32 keys of the tile, so the online-softmax max/sum are
