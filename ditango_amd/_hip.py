@@ -20,6 +20,7 @@ DT_LSE_BHS, DT_LSE_BSH = 0, 1
 DT_NORM_NONE, DT_NORM_RMS, DT_NORM_LAYER = 0, 1, 2
 DT_ROPE_NONE, DT_ROPE_INTERLEAVED, DT_ROPE_HALVES = 0, 1, 2
 DT_ROUND_NORM_BF16, DT_ROUND_ROPE_BF16 = 1, 2
+DT_ATTN_Q_PRESCALED = 1
 DT_MAX_CHUNKS = 40
 DT_MAX_JOBS = 40
 DT_MAX_JOB_ENTRIES = 64
@@ -45,11 +46,11 @@ _SIGNATURES = {
     "dt_attn_seg_jobs_ws_fwd": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i64, c_i64, c_i64,
                                                c_i32, _P(c_vp), _P(c_vp), _P(c_i32), _P(c_i64), c_i64, c_i64,
                                                c_i32, _P(c_i32), _P(c_i32), _P(c_i32), _P(c_i32), _P(c_i32), _P(c_i32),
-                                               _P(c_vp), _P(c_vp), c_f32, c_vp, c_i64, c_vp]),
+                                               _P(c_vp), _P(c_vp), c_f32, c_i32, c_vp, c_i64, c_vp]),
     "dt_attn_sched_seg_ws_fwd": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i64, c_i64, c_i64,
                                                 c_i32, _P(c_vp), _P(c_vp), _P(c_i32), _P(c_i64), c_i64, c_i64,
                                                 c_vp, c_vp, c_i32, c_vp, c_i64, c_vp, c_i64, c_i32, c_vp, c_vp,
-                                                c_i32, _P(c_i32), _P(c_i32), _P(c_i32), _P(c_i32), c_f32,
+                                                c_i32, _P(c_i32), _P(c_i32), _P(c_i32), _P(c_i32), c_f32, c_i32,
                                                 c_vp, c_i64, c_vp]),
     "dt_attn_sched_fwd": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i64, c_i64, c_i64,
                                          c_i32, _P(c_vp), _P(c_vp), _P(c_i32), _P(c_i64), c_i64, c_i64,
@@ -68,7 +69,7 @@ _SIGNATURES = {
     "dt_rel_l1_sums": (ctypes.c_int, [c_vp, c_vp, c_i64, c_vp, c_vp]),
     "dt_qk_norm_rope": (ctypes.c_int, [c_vp, c_i64, c_i64, c_i64, c_vp, c_i32, c_i32, c_i32, c_i32,
                                        c_i32, c_vp, c_vp, c_f32, c_i32, c_vp, c_vp, c_i64, c_i32, c_i32,
-                                       _P(c_i32), c_i32, c_i32, c_vp]),
+                                       _P(c_i32), c_i32, c_i32, c_f32, c_vp]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
@@ -221,7 +222,7 @@ def attn_jobs_fwd(q: torch.Tensor, table: ChunkTable, jobs: Sequence[Sequence[in
                   outs: Sequence[torch.Tensor], lses: Sequence[torch.Tensor], softmax_scale: float = 0.0,
                   q_ranges: Optional[Sequence[Tuple[int, int]]] = None,
                   kv_ranges: Optional[Sequence[Sequence[Tuple[int, int]]]] = None,
-                  workspace: Optional[torch.Tensor] = None) -> None:
+                  workspace: Optional[torch.Tensor] = None, q_prescaled: bool = False) -> None:
     """One launch; job j attends q to the concatenation of chunks ``jobs[j]`` and writes (outs[j], lses[j]).
 
     ``q_ranges[j] = (begin, length)`` restricts job j to those query rows (the rest of its
@@ -229,7 +230,9 @@ def attn_jobs_fwd(q: torch.Tensor, table: ChunkTable, jobs: Sequence[Sequence[in
     of job j to those keys.  Several jobs may share one destination if their rows are disjoint
     (the segments of a packed variable-length batch).  Launches are split to respect the limits
     of one launch.  With a ``workspace`` (``attn_workspace(device)``) the last, partly filled round of
-    workgroups of a launch is split along the keys and folded back (tail balancing)."""
+    workgroups of a launch is split along the keys and folded back (tail balancing).
+    ``q_prescaled``: q already carries ``softmax_scale * log2(e)`` (folded in before its rounding to
+    bf16); ``softmax_scale`` is then ignored and the softmax is that of ``q k^T * ln 2``."""
     lib = load_library()
     _check_qkv(q, "q")
     B, Sq, H, D = q.shape
@@ -276,7 +279,8 @@ def attn_jobs_fwd(q: torch.Tensor, table: ChunkTable, jobs: Sequence[Sequence[in
         rc = lib.dt_attn_seg_jobs_ws_fwd(q.data_ptr(), B, Sq, H, D, q.stride(0), q.stride(1), q.stride(2),
                                          table.n, table.k_ptrs, table.v_ptrs, table.lens, table.sb, table.ss, table.sh,
                                          n, begin, chunks, a_kvb, a_kvl, a_qb, a_ql, out_ptrs, lse_ptrs,
-                                         float(softmax_scale), workspace.data_ptr() if workspace is not None else None,
+                                         float(softmax_scale), DT_ATTN_Q_PRESCALED if q_prescaled else 0,
+                                         workspace.data_ptr() if workspace is not None else None,
                                          workspace.numel() * workspace.element_size() if workspace is not None else 0,
                                          _stream())
         _check(rc, "dt_attn_seg_jobs_ws_fwd")
@@ -288,7 +292,7 @@ def attn_sched_fwd(q: torch.Tensor, table: ChunkTable, dev_compute_ids: torch.Te
                    diag_out: Optional[torch.Tensor], diag_lse: Optional[torch.Tensor],
                    softmax_scale: float = 0.0, seg_q: Optional[Sequence[Tuple[int, int]]] = None,
                    seg_kv: Optional[Sequence[Sequence[Tuple[int, int]]]] = None,
-                   workspace: Optional[torch.Tensor] = None) -> None:
+                   workspace: Optional[torch.Tensor] = None, q_prescaled: bool = False) -> None:
     """Device-scheduled launch: chunk ids come from ``dev_compute_ids[:dev_count]`` in device memory and
     each state lands in its slot of the arena (``slot_out [C,B,Sq,H,D]`` bf16, ``slot_lse [C,B,H,Sq]`` fp32).
 
@@ -327,6 +331,7 @@ def attn_sched_fwd(q: torch.Tensor, table: ChunkTable, dev_compute_ids: torch.Te
                                    int(diag), diag_out.data_ptr() if diag_out is not None else None,
                                    diag_lse.data_ptr() if diag_lse is not None else None,
                                    n_seg, a_qb, a_ql, a_kb, a_kl, float(softmax_scale),
+                                   DT_ATTN_Q_PRESCALED if q_prescaled else 0,
                                    workspace.data_ptr() if workspace is not None else None,
                                    workspace.numel() * workspace.element_size() if workspace is not None else 0, _stream())
     _check(rc, "dt_attn_sched_seg_ws_fwd")
@@ -438,10 +443,11 @@ def qk_norm_rope(x: torch.Tensor, *, norm: int = DT_NORM_NONE, weight: Optional[
                  bias: Optional[torch.Tensor] = None, eps: float = 1e-6, rope: int = DT_ROPE_NONE,
                  cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None,
                  rope_begin: int = 0, rope_end: Optional[int] = None, sections: Sequence[int] = (),
-                 rounding: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                 rounding: int = 0, out: Optional[torch.Tensor] = None, out_scale: float = 1.0) -> torch.Tensor:
     """x bf16 ``[B,S,H,D]`` (any strides with a contiguous last dimension) -> bf16 ``[B,S,H,D]`` contiguous,
     normalised over D and rotated on token rows ``[rope_begin, rope_end)``.  cos/sin are fp32
-    ``[rope_end-rope_begin, D]`` or ``[B, rope_end-rope_begin, D]``."""
+    ``[rope_end-rope_begin, D]`` or ``[B, rope_end-rope_begin, D]``.  ``out_scale`` multiplies the result
+    before its rounding to bf16."""
     lib = load_library()
     _require(x.is_cuda and x.dtype == torch.bfloat16 and x.dim() == 4 and x.stride(3) == 1, "x must be bf16 [B,S,H,D] on the GPU")
     B, S, H, D = x.shape
@@ -470,6 +476,7 @@ def qk_norm_rope(x: torch.Tensor, *, norm: int = DT_NORM_NONE, weight: Optional[
                              int(norm), weight.data_ptr() if weight is not None else None,
                              bias.data_ptr() if bias is not None else None, float(eps), int(rope),
                              cos.data_ptr() if cos is not None else None, sin.data_ptr() if sin is not None else None,
-                             tab_sb, int(rope_begin), int(rope_end), sec, len(sections), int(rounding), _stream())
+                             tab_sb, int(rope_begin), int(rope_end), sec, len(sections), int(rounding), float(out_scale),
+                             _stream())
     _check(rc, "dt_qk_norm_rope")
     return out

@@ -173,6 +173,11 @@ class proAttention:
         # (attention_processor.py:80, step/attentions.py:98); torch.bfloat16 here lets the merge kernel
         # write the bf16 the out-projection consumes: half the result bytes and no separate cast pass.
         self.out_dtype = torch.float32
+        # True: the caller folded softmax_scale * log2(e) into the query before rounding it to bf16
+        # (ditango_amd.producer.prepare_qk(..., fold_softmax_scale=...), or the QK-norm weight): the
+        # kernels then skip the scaling (a quarter of the softmax's vector instructions).  Not what the
+        # reference's callers pass (flash_attn_func scales inside, core/attention.py:137-143).
+        self.q_prescaled = False
         self._segments = None  # (cu_seqlens_q, chunk -> cu_seqlens_kv) while a variable-length call runs
         if self.layer_id == 0:
             logger.info(f"R{self.global_rank}L{layer_id} | cached block attention on HIP kernels (gfx950)")
@@ -298,7 +303,8 @@ class proAttention:
         if job_lists:
             table = _hip.ChunkTable(ks, vs)
             _hip.attn_jobs_fwd(query, table, job_lists, [d[0] for d in dests], [d[1] for d in dests],
-                               q_ranges=q_ranges, kv_ranges=kv_ranges, workspace=_hip.attn_workspace(dev))
+                               q_ranges=q_ranges, kv_ranges=kv_ranges, workspace=_hip.attn_workspace(dev),
+                               q_prescaled=self.q_prescaled)
         for job, (o, l) in zip(plan.jobs, states):
             if job.store_slot is not None:
                 self.cache.store_block(job.store_slot, o, l)  # :207-211
@@ -338,7 +344,8 @@ class proAttention:
                       for c in range(C)]
         _hip.attn_sched_fwd(query, table, rm.sched_compute_ids[t, l], rm.sched_counts[t, l, 0:1], n_comp,
                             cache.arena_out, cache.arena_lse, diag, cache.diag_out, cache.diag_lse,
-                            seg_q=seg_q, seg_kv=seg_kv, workspace=_hip.attn_workspace(query.device))
+                            seg_q=seg_q, seg_kv=seg_kv, workspace=_hip.attn_workspace(query.device),
+                            q_prescaled=self.q_prescaled)
         outs, lses = [], []
         for c in range(C):
             if c == diag:

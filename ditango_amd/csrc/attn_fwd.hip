@@ -134,6 +134,12 @@ __device__ __forceinline__ void phase_barrier_after_matrix(V (&sa)[2], V (&oa)[N
 // exact row maximum.  Below it every probability is at most 2^12: harmless for the bf16
 // operand (same relative precision at any exponent) and for the fp32 accumulators.
 constexpr float kSumLimit = 4096.0f;
+// The same for queries that come with softmax_scale * log2(e) folded in (kPre): rows keep the
+// reference 0 while the maximum of their first tile lies in [kBandLo, kBandHi] (powers of two;
+// 2^-40 .. 2^24 neither underflows nor overflows anything downstream), so a probability is then
+// simply exp2(score), and a tile is redone when its sum exceeds 2^40.
+constexpr float kSumLimitPre = 1099511627776.0f;
+constexpr float kBandLo = -40.f, kBandHi = 24.f;
 
 template <int D>
 struct Tile {
@@ -177,7 +183,7 @@ __device__ __forceinline__ s16x4 lds_read_tr(const uint8_t* p) {
       (s16x4 __attribute__((address_space(3)))*)(p));
 }
 
-template <int D>
+template <int D, bool kPre>
 __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a) {
   using T = Tile<D>;
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -399,9 +405,12 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   for (int i = 0; i < D / 32; ++i)
 #pragma unroll
     for (int r = 0; r < 16; ++r) o_acc[i][r] = 0.f;
-  float m_ref = -INFINITY;  // reference maximum (raw scores) the accumulators are scaled to
+  // reference (raw scores; kPre: log2 units) the accumulators are scaled to
+  float m_ref = kPre ? 0.f : -INFINITY;
+  float rs_bias = kPre ? INFINITY : 0.f;  // kPre: inf until the row has seen a key (forces the exact path)
+  bool any_off = false;                   // kPre: some row of this wavefront has a reference other than 0
   float l_run = 0.f;        // running sum over THIS lane's keys (halves combined at the end)
-  const float c = a.scale_log2;
+  const float c = kPre ? 1.f : a.scale_log2;
 
   // operand read addresses of this lane within a K / V buffer (the lane's part of the swizzle)
   uint32_t kld[D / 16];  // K fragment of k-step s: row key_of_row(col) (+32 for the second half tile)
@@ -568,7 +577,9 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     // 1.43k vs 1.24k cycles of vector work), so every other barrier waits for a squeezed softmax.
     __builtin_amdgcn_s_setprio(1);
     if constexpr (!kLoadAfterMatrix) load_tile((kU + 3 + group) & (kNumBuf - 1));
-    if (__builtin_expect(cp_valid < kBK, 0)) {
+    // (kPre: the same rare branch takes the reference off the scores of a wavefront in which some
+    // row has left the band; everywhere else the reference is 0 and there is nothing to subtract)
+    if (__builtin_expect(cp_valid < kBK || (kPre && any_off), 0)) {
       // the empty asm has side effects as far as the compiler knows, which keeps this a real
       // branch: otherwise the selects below are hoisted out and run for every tile
       asm volatile("" ::: "memory");
@@ -579,6 +590,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
         for (int r = 0; r < 16; ++r) {
           const int key = 32 * kb + 16 * (r >> 3) + 8 * hh + (r & 7);
           if (key >= lim) s_acc[kb][r] = -INFINITY;
+          if constexpr (kPre) s_acc[kb][r] -= m_ref;
         }
     }
     // Probabilities relative to the reference maximum the accumulators are scaled to.  The
@@ -588,29 +600,47 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     // where the reference is -inf and the sum comes out inf or NaN -- the tile is redone below
     // with its exact maximum.
     float mc = m_ref * c;
-    float rs0 = 0.f, rs1 = 0.f;
+    float rs0 = rs_bias, rs1 = 0.f;
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
       for (int r = 0; r < 16; r += 2) {
         f32x2 p;
-        p.x = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[kb][r], c, -mc));
-        p.y = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[kb][r + 1], c, -mc));
+        if constexpr (kPre) {
+          p.x = __builtin_amdgcn_exp2f(s_acc[kb][r]);
+          p.y = __builtin_amdgcn_exp2f(s_acc[kb][r + 1]);
+        } else {
+          p.x = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[kb][r], c, -mc));
+          p.y = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[kb][r + 1], c, -mc));
+        }
         rs0 += p.x;
         rs1 += p.y;
         const bf16x2 pb = __builtin_convertvector(p, bf16x2);
         p_frag[kb][r >> 3][r & 7] = pb.x;
         p_frag[kb][r >> 3][(r & 7) + 1] = pb.y;
       }
-    if (__builtin_expect(__any(!(rs0 + rs1 <= kSumLimit)), 0)) {
+    if (__builtin_expect(__any(!(rs0 + rs1 <= (kPre ? kSumLimitPre : kSumLimit))), 0)) {
       float mx = s_acc[0][0];
 #pragma unroll
       for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s_acc[0][r]);
 #pragma unroll
       for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s_acc[1][r]);
       mx = fmaxf(mx, __shfl_xor(mx, 32));
-      const float m_new = fmaxf(m_ref, mx);
-      const float alpha = m_new > -INFINITY ? __builtin_amdgcn_exp2f((m_ref - m_new) * c) : 1.f;
+      float m_new, alpha;
+      if constexpr (kPre) {
+        float rs_tot = rs0 + rs1;
+        rs_tot += __shfl_xor(rs_tot, 32);
+        const bool first = rs_bias != 0.f;
+        const float mx_true = mx + m_ref;
+        if (first) m_new = (mx_true >= kBandLo && mx_true <= kBandHi) || !(mx_true > -INFINITY) ? 0.f : mx_true;
+        else m_new = !(rs_tot <= kSumLimitPre) ? fmaxf(m_ref, mx_true) : m_ref;
+        alpha = first ? 1.f : __builtin_amdgcn_exp2f(m_ref - m_new);
+        rs_bias = first && !(mx > -INFINITY) ? INFINITY : 0.f;
+        mx = m_new - m_ref;  // what the scores in s_acc still have to lose
+      } else {
+        m_new = fmaxf(m_ref, mx);
+        alpha = m_new > -INFINITY ? __builtin_amdgcn_exp2f((m_ref - m_new) * c) : 1.f;
+      }
       m_ref = m_new;
       l_run *= alpha;
 #pragma unroll
@@ -618,7 +648,8 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
 #pragma unroll
         for (int r = 0; r < 16; ++r) o_acc[i][r] *= alpha;
       // a row whose keys are all masked so far keeps m_ref = -inf: use 0 so that exp2(-inf - 0) = 0
-      mc = m_new > -INFINITY ? m_new * c : 0.f;
+      mc = kPre ? mx : (m_new > -INFINITY ? m_new * c : 0.f);
+      if constexpr (kPre) any_off = any_off || __any(m_ref != 0.f);
       rs0 = 0.f;
       rs1 = 0.f;
 #pragma unroll
@@ -785,26 +816,30 @@ __global__ __launch_bounds__(256) void attn_tail_fold_kernel(const AttnArgs a) {
   }
 }
 
-template <int D>
+template <int D, bool kPre>
 static int launch_one(const AttnArgs& a, dim3 grid, hipStream_t stream) {
   // more than 64 KB of dynamic LDS has to be allowed once per kernel and device
   static thread_local int allowed_dev = -1;
   int dev = 0;
   if (int rc = hip_fail(hipGetDevice(&dev), "hipGetDevice")) return rc;
   if (allowed_dev != dev) {
-    if (int rc = hip_fail(hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_fwd_kernel<D>),
+    if (int rc = hip_fail(hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_fwd_kernel<D, kPre>),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, Tile<D>::kLdsBytes),
                           "hipFuncSetAttribute"))
       return rc;
     allowed_dev = dev;
   }
-  hipLaunchKernelGGL(attn_fwd_kernel<D>, grid, dim3(kThreads), Tile<D>::kLdsBytes, stream, a);
+  hipLaunchKernelGGL((attn_fwd_kernel<D, kPre>), grid, dim3(kThreads), Tile<D>::kLdsBytes, stream, a);
   return hip_fail(hipGetLastError(), "attn_fwd launch");
 }
 
 static int launch_dim(const AttnArgs& a, int D, dim3 grid, hipStream_t stream) {
-  if (D == 128) return launch_one<128>(a, grid, stream);
-  return launch_one<64>(a, grid, stream);
+  if (a.q_prescaled) {
+    if (D == 128) return launch_one<128, true>(a, grid, stream);
+    return launch_one<64, true>(a, grid, stream);
+  }
+  if (D == 128) return launch_one<128, false>(a, grid, stream);
+  return launch_one<64, false>(a, grid, stream);
 }
 
 // Number of CUs of the current device (one workgroup of the attention kernel per CU at a time).

@@ -108,6 +108,15 @@ static int check_workspace(const void* workspace, int64_t workspace_bytes) {
   return DT_OK;
 }
 
+static int apply_flags(AttnArgs& a, int32_t flags) {
+  if (flags & ~DT_ATTN_Q_PRESCALED) {
+    set_error("unknown attention flags 0x%x", (unsigned)flags);
+    return DT_ERR_INVALID;
+  }
+  a.q_prescaled = (flags & DT_ATTN_Q_PRESCALED) ? 1 : 0;
+  return DT_OK;
+}
+
 extern "C" int dt_attn_seg_jobs_ws_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D, int64_t q_sb,
                                        int64_t q_ss, int64_t q_sh, int32_t n_chunks, const void* const* k_ptrs,
                                        const void* const* v_ptrs, const int32_t* kv_lens, const int64_t* kv_sb,
@@ -115,12 +124,14 @@ extern "C" int dt_attn_seg_jobs_ws_fwd(const void* q, int32_t B, int32_t Sq, int
                                        const int32_t* job_chunks, const int32_t* entry_kv_begin,
                                        const int32_t* entry_kv_len, const int32_t* job_q_begin,
                                        const int32_t* job_q_len, void* const* out_ptrs, float* const* lse_ptrs,
-                                       float softmax_scale, void* workspace, int64_t workspace_bytes, void* stream) {
+                                       float softmax_scale, int32_t flags, void* workspace,
+                                       int64_t workspace_bytes, void* stream) {
   if (int rc = check_workspace(workspace, workspace_bytes)) return rc;
   AttnArgs a{};
   if (int rc = fill_common(a, q, B, Sq, H, D, q_sb, q_ss, q_sh, n_chunks, k_ptrs, v_ptrs, kv_lens, kv_sb, kv_ss, kv_sh,
                            softmax_scale))
     return rc;
+  if (int rc = apply_flags(a, flags)) return rc;
   if (n_jobs == 0) return DT_OK;
   if (n_jobs < 0 || n_jobs > DT_MAX_JOBS || !job_begin || !job_chunks || !out_ptrs || !lse_ptrs) {
     set_error("%d jobs: need 0..%d and non-null job tables", n_jobs, DT_MAX_JOBS);
@@ -192,7 +203,7 @@ extern "C" int dt_attn_seg_jobs_fwd(const void* q, int32_t B, int32_t Sq, int32_
                                     float softmax_scale, void* stream) {
   return dt_attn_seg_jobs_ws_fwd(q, B, Sq, H, D, q_sb, q_ss, q_sh, n_chunks, k_ptrs, v_ptrs, kv_lens, kv_sb, kv_ss, kv_sh,
                                  n_jobs, job_begin, job_chunks, entry_kv_begin, entry_kv_len, job_q_begin, job_q_len,
-                                 out_ptrs, lse_ptrs, softmax_scale, nullptr, 0, stream);
+                                 out_ptrs, lse_ptrs, softmax_scale, 0, nullptr, 0, stream);
 }
 
 extern "C" int dt_attn_jobs_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D, int64_t q_sb, int64_t q_ss,
@@ -229,12 +240,13 @@ extern "C" int dt_attn_sched_seg_ws_fwd(const void* q, int32_t B, int32_t Sq, in
                                         int32_t diag, void* diag_out, float* diag_lse, int32_t n_seg,
                                         const int32_t* seg_q_begin, const int32_t* seg_q_len,
                                         const int32_t* seg_kv_begin, const int32_t* seg_kv_len, float softmax_scale,
-                                        void* workspace, int64_t workspace_bytes, void* stream) {
+                                        int32_t flags, void* workspace, int64_t workspace_bytes, void* stream) {
   if (int rc = check_workspace(workspace, workspace_bytes)) return rc;
   AttnArgs a{};
   if (int rc = fill_common(a, q, B, Sq, H, D, q_sb, q_ss, q_sh, n_chunks, k_ptrs, v_ptrs, kv_lens, kv_sb, kv_ss, kv_sh,
                            softmax_scale))
     return rc;
+  if (int rc = apply_flags(a, flags)) return rc;
   if (max_jobs == 0) return DT_OK;
   if (max_jobs < 0 || max_jobs > n_chunks) {
     set_error("max_jobs %d must be in 0..n_chunks (%d)", max_jobs, n_chunks);
@@ -318,7 +330,7 @@ extern "C" int dt_attn_sched_seg_fwd(const void* q, int32_t B, int32_t Sq, int32
   return dt_attn_sched_seg_ws_fwd(q, B, Sq, H, D, q_sb, q_ss, q_sh, n_chunks, k_ptrs, v_ptrs, kv_lens, kv_sb, kv_ss,
                                   kv_sh, dev_compute_ids, dev_count, max_jobs, slot_out, slot_out_stride, slot_lse,
                                   slot_lse_stride, diag, diag_out, diag_lse, n_seg, seg_q_begin, seg_q_len,
-                                  seg_kv_begin, seg_kv_len, softmax_scale, nullptr, 0, stream);
+                                  seg_kv_begin, seg_kv_len, softmax_scale, 0, nullptr, 0, stream);
 }
 
 extern "C" int dt_attn_sched_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D, int64_t q_sb, int64_t q_ss,

@@ -20,6 +20,7 @@ struct AttnArgs {
   int32_t total;      // B*H*nqt work items per job
   int32_t per_xcd;    // work items handed to each of the 8 XCDs
   float scale_log2;   // softmax scale * log2(e)
+  int32_t q_prescaled;  // the caller folded scale_log2 into q: scores are already in log2 units
   // chunk table
   int32_t n_chunks;
   const __bf16* k[DT_MAX_CHUNKS];

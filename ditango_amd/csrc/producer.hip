@@ -30,6 +30,7 @@ struct PrepArgs {
   const float* w;
   const float* bias;
   float eps;
+  float out_scale;  // multiplies the result before its rounding to bf16
   const float* cos;
   const float* sin;
   int64_t tab_sb;
@@ -197,6 +198,10 @@ __global__ __launch_bounds__(kThreads) void qk_norm_rope_kernel(const PrepArgs a
         }
       }
     }
+    if (a.out_scale != 1.0f) {  // uniform
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] *= a.out_scale;
+    }
     u32x4 o;
     o.x = pack2(v[0], v[1]);
     o.y = pack2(v[2], v[3]);
@@ -217,7 +222,8 @@ extern "C" int dt_qk_norm_rope(const void* x, int64_t x_stride_b, int64_t x_stri
                                int32_t B, int32_t S, int32_t H, int32_t D, int32_t norm, const float* weight,
                                const float* bias, float eps, int32_t rope, const float* cos, const float* sin,
                                int64_t table_stride_b, int32_t rope_begin, int32_t rope_end,
-                               const int32_t* sections, int32_t n_sections, int32_t rounding, void* stream) {
+                               const int32_t* sections, int32_t n_sections, int32_t rounding, float out_scale,
+                               void* stream) {
   if (B <= 0 || S <= 0 || H <= 0) {
     set_error("B, S, H must be positive (got %d, %d, %d)", B, S, H);
     return DT_ERR_INVALID;
@@ -235,6 +241,10 @@ extern "C" int dt_qk_norm_rope(const void* x, int64_t x_stride_b, int64_t x_stri
     set_error("bad norm / rope / rounding code (%d, %d, %d)", norm, rope, rounding);
     return DT_ERR_INVALID;
   }
+  if (!(out_scale > 0.0f) || !(out_scale < INFINITY)) {
+    set_error("out_scale must be positive and finite (1 for none)");
+    return DT_ERR_INVALID;
+  }
   if ((weight && !aligned16(weight)) || (bias && !aligned16(bias))) {
     set_error("weight and bias must be 16-byte aligned");
     return DT_ERR_INVALID;
@@ -246,6 +256,7 @@ extern "C" int dt_qk_norm_rope(const void* x, int64_t x_stride_b, int64_t x_stri
   a.B = B; a.S = S; a.H = H;
   a.norm = norm; a.rope = rope; a.rounding = rounding;
   a.w = weight; a.bias = bias; a.eps = eps;
+  a.out_scale = out_scale;
   a.sec_end[0] = a.sec_end[1] = a.sec_end[2] = D;
   if (rope != DT_ROPE_NONE) {
     if (rope_begin < 0 || rope_end > S || rope_begin > rope_end) {

@@ -14,6 +14,7 @@ The reference's executors run these as chains of eager torch ops right before
 """
 from __future__ import annotations
 
+import math
 from typing import Optional, Sequence, Tuple
 
 import torch
@@ -36,7 +37,8 @@ def prepare_qk(x: torch.Tensor, *, norm: Optional[str] = None, weight: Optional[
                bias: Optional[torch.Tensor] = None, eps: float = 1e-6, rope: Optional[str] = None,
                freqs_cis: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, rope_begin: int = 0,
                rope_end: Optional[int] = None, sections: Sequence[int] = (), match_eager_rounding: bool = False,
-               bf16_rope_math: bool = False, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+               bf16_rope_math: bool = False, out: Optional[torch.Tensor] = None,
+               fold_softmax_scale: Optional[float] = None) -> torch.Tensor:
     """x: bf16 ``[B,S,H,D]`` view (e.g. a slice of a fused QKV projection; only the last dimension
     must be contiguous).  Returns bf16 ``[B,S,H,D]`` contiguous.
 
@@ -45,7 +47,13 @@ def prepare_qk(x: torch.Tensor, *, norm: Optional[str] = None, weight: Optional[
     per section of ``sections``) | None; ``freqs_cis = (cos, sin)`` of shape ``[rope_end-rope_begin, D]``
     (or with a leading batch dimension), as the callers already hold them; token ``s`` reads row
     ``s - rope_begin``.  ``match_eager_rounding`` rounds to bf16 where the callers' bf16 norm modules do;
-    ``bf16_rope_math`` additionally rounds both RoPE products (Step-Video computes RoPE in bf16)."""
+    ``bf16_rope_math`` additionally rounds both RoPE products (Step-Video computes RoPE in bf16).
+
+    ``fold_softmax_scale`` (for q only): multiplies the result by ``folded_scale(D, fold_softmax_scale)`` =
+    ``softmax_scale * log2(e)`` before the rounding to bf16 (pass 0 for the default ``D ** -0.5``).  The
+    attention object must then be told with ``proAttention.q_prescaled = True``: its softmax needs a
+    quarter fewer vector instructions.  q differs from the unscaled one by its rounding only, but it is
+    not the tensor the reference would hand to ``attn`` -- an opt-in, not part of the drop-in path."""
     if norm not in _NORMS or rope not in _ROPES:
         raise ValueError(f"unknown norm {norm!r} or rope {rope!r}")
     cos = sin = None
@@ -56,7 +64,15 @@ def prepare_qk(x: torch.Tensor, *, norm: Optional[str] = None, weight: Optional[
     rounding = (_hip.DT_ROUND_NORM_BF16 if match_eager_rounding else 0) | (_hip.DT_ROUND_ROPE_BF16 if bf16_rope_math else 0)
     return _hip.qk_norm_rope(x, norm=_NORMS[norm], weight=_f32(weight, x.device), bias=_f32(bias, x.device), eps=eps,
                              rope=_ROPES[rope], cos=cos, sin=sin, rope_begin=rope_begin, rope_end=rope_end,
-                             sections=sections, rounding=rounding, out=out)
+                             sections=sections, rounding=rounding, out=out,
+                             out_scale=1.0 if fold_softmax_scale is None else folded_scale(x.shape[-1], fold_softmax_scale))
+
+
+def folded_scale(head_dim: int, softmax_scale: float = 0.0) -> float:
+    """``softmax_scale * log2(e)`` (``softmax_scale <= 0``: flash_attn's default ``head_dim ** -0.5``): what a
+    caller multiplies q by (before rounding it to bf16) to run the attention with ``q_prescaled``."""
+    scale = softmax_scale if softmax_scale and softmax_scale > 0 else head_dim ** -0.5
+    return scale * math.log2(math.e)
 
 
 def rope3d_tables(f: int, h: int, w: int, ch_split: Sequence[int] = (64, 32, 32), dtype: torch.dtype = torch.bfloat16,

@@ -100,9 +100,11 @@ def rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, kind: int, secti
 def qk_norm_rope(x: torch.Tensor, norm: int = NORM_NONE, weight: Optional[torch.Tensor] = None,
                  bias: Optional[torch.Tensor] = None, eps: float = 1e-6, rope_kind: int = ROPE_NONE,
                  cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None, rope_begin: int = 0,
-                 rope_end: Optional[int] = None, sections: Sequence[int] = (), rounding: int = 0) -> torch.Tensor:
+                 rope_end: Optional[int] = None, sections: Sequence[int] = (), rounding: int = 0,
+                 out_scale: float = 1.0) -> torch.Tensor:
     """The whole producer step on x bf16 ``[B,S,H,D]``; returns the fp32 value BEFORE the final
-    rounding to bf16 (the caller rounds, so a test can bound the distance to the exact value)."""
+    rounding to bf16 (the caller rounds, so a test can bound the distance to the exact value).
+    ``out_scale`` multiplies the result (fp32) last: a caller's way of folding the softmax scale into q."""
     rn = bool(rounding & ROUND_NORM_BF16)
     if norm == NORM_RMS:
         y = rms_norm(x, weight, eps, rn)
@@ -117,6 +119,8 @@ def qk_norm_rope(x: torch.Tensor, norm: int = NORM_NONE, weight: Optional[torch.
             y = y.clone()
             y[:, rope_begin:rope_end] = rope(y[:, rope_begin:rope_end], cos, sin, rope_kind, sections,
                                              bool(rounding & ROUND_ROPE_BF16))
+    if out_scale != 1.0:
+        y = y * torch.tensor(out_scale, dtype=torch.float32)
     return y
 
 
