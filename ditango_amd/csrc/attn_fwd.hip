@@ -88,29 +88,24 @@ __device__ __forceinline__ void phase_barrier() {
 // operands.  Register-only code may otherwise migrate across an asm statement; tied to it,
 // the phase's work stays on its own side (the vector phase produces P^T, the matrix phase
 // produces S^T and updates O^T).
-// After a vector phase the wavefront also waits for the direct-to-LDS tile loads it issued two
-// vector phases ago (all but the kInFlight newest): behind the barrier they are visible to
-// every wavefront.
+// After a vector phase the wavefront also waits for the direct-to-LDS tile loads it issued earlier,
+// all but the kInFlight newest: behind the barrier they are visible to every wavefront.
 template <int kInFlight, typename V>
 __device__ __forceinline__ void phase_barrier_after_vector(V (&p)[2][2]) {
   __builtin_amdgcn_sched_barrier(0);
-  if constexpr (kInFlight == 8) {
-    asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier"
-                 : "+v"(p[0][0]), "+v"(p[0][1]), "+v"(p[1][0]), "+v"(p[1][1])
-                 :
-                 : "memory");
-  } else if constexpr (kInFlight == 4) {
-    asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier"
-                 : "+v"(p[0][0]), "+v"(p[0][1]), "+v"(p[1][0]), "+v"(p[1][1])
-                 :
-                 : "memory");
-  } else {
-    static_assert(kInFlight == 2, "loads in flight across the barrier: 2, 4 or 8");
-    asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)\n\ts_barrier"
-                 : "+v"(p[0][0]), "+v"(p[0][1]), "+v"(p[1][0]), "+v"(p[1][1])
-                 :
-                 : "memory");
+#define DT_VECTOR_BARRIER(N)                                                      \
+  asm volatile("s_waitcnt vmcnt(" #N ") lgkmcnt(0)\n\ts_barrier"                   \
+               : "+v"(p[0][0]), "+v"(p[0][1]), "+v"(p[1][0]), "+v"(p[1][1])       \
+               :                                                                  \
+               : "memory")
+  if constexpr (kInFlight == 6) DT_VECTOR_BARRIER(6);
+  else if constexpr (kInFlight == 3) DT_VECTOR_BARRIER(3);
+  else if constexpr (kInFlight == 2) DT_VECTOR_BARRIER(2);
+  else {
+    static_assert(kInFlight == 1, "loads in flight across the barrier: 1, 2, 3 or 6");
+    DT_VECTOR_BARRIER(1);
   }
+#undef DT_VECTOR_BARRIER
   __builtin_amdgcn_sched_barrier(0);
 }
 template <typename V, int NO>
@@ -181,6 +176,30 @@ typedef short s16x8 __attribute__((ext_vector_type(8)));
 __device__ __forceinline__ s16x4 lds_read_tr(const uint8_t* p) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
       (s16x4 __attribute__((address_space(3)))*)(p));
+}
+
+// Raw buffer descriptor: base address, stride 0, number of valid bytes, flags.
+__device__ __forceinline__ u32x4 make_rsrc(const void* base, uint32_t valid_bytes) {
+  const uint64_t p = reinterpret_cast<uint64_t>(base);
+  u32x4 r;
+  r.x = (uint32_t)p;
+  r.y = (uint32_t)(p >> 32) & 0xffffu;
+  r.z = valid_bytes;
+  r.w = (uint32_t)kRsrcFlags;
+  return r;
+}
+// One 16-byte-per-lane buffer load whose destination is the LDS: lane L's bytes land at
+// lds_addr + 16 L (lds_addr, through M0, is uniform).  Written as inline assembly on purpose: the
+// compiler, when it sees such a load, makes every later LDS read of the wavefront wait for ALL
+// outstanding loads (it cannot tell that the reads touch other buffers), which turns a prefetch
+// several phases deep into one that must land within the phase.  Here the waits are the explicit
+// vmcnt in front of the barriers.  (Loads the compiler does not know of only make its own vmcnt
+// waits for other loads stricter, never too weak: the counter retires in order.)
+__device__ __forceinline__ void load_block_to_lds(u32x4 rsrc, uint32_t lane_off, uint32_t uniform_off, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds"
+               :
+               : "v"(lane_off), "s"(rsrc), "s"(uniform_off), "s"(lds_addr)
+               : "memory", "m0");
 }
 
 template <int D, bool kPre>
@@ -363,10 +382,11 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   static_assert((8 * T::kRowsPerBlock) % 16 == 0, "the swizzle must not depend on the load index");
   const int64_t tile_bytes = (int64_t)kBK * row_bytes;
   typedef __attribute__((address_space(3))) uint8_t* lds_ptr_t;
-  // Issues this wavefront's loads of K of the tile under the load cursor (tile X, into K buffer
-  // X & 3) and of V of the tile before it (V is needed two phases later than K, so its loads run
-  // one tile behind and reuse the descriptor the previous call made for K), and moves the cursor
-  // on.  Past the last tile the loads are still issued, against an empty descriptor (they store
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
+  // Issues this wavefront's loads of V of the tile before the one under the load cursor and of
+  // K of the tile under it (tile X, into K buffer X & 3; V is needed two phases later than K, so
+  // its loads run one tile behind and reuse the descriptor the previous call made for K), and
+  // moves the cursor on.  Past the last tile the loads are still issued, against an empty descriptor (they store
   // zeros without touching memory): with the same number of loads in every iteration the counter
   // the barrier waits on is static.
   const uint8_t* prev_v = nullptr;  // V of the tile the previous call loaded K of
@@ -374,23 +394,20 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   auto load_tile = [&](int kbuf) {
     const bool have = __builtin_expect(ld_seg < seg_end, 1);
     const uint32_t valid = have ? (uint32_t)(ld_left - 1) * row_bytes + (uint32_t)(D * 2) : 0u;
-    const __amdgpu_buffer_rsrc_t rk =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(ld_k), 0, (int)valid, kRsrcFlags);
-    const __amdgpu_buffer_rsrc_t rv =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(prev_v), 0, (int)prev_valid, kRsrcFlags);
+    const u32x4 rk = make_rsrc(ld_k, valid);
+    const u32x4 rv = make_rsrc(prev_v, prev_valid);
     prev_v = ld_v;
     prev_valid = valid;
     const int vbuf = (kbuf + kNumBuf - 1) & (kNumBuf - 1);
-    lds_ptr_t kdst = (lds_ptr_t)lds + kbuf * T::kBytesK + wave * 1024;
-    lds_ptr_t vdst = (lds_ptr_t)lds + T::kOffV + vbuf * T::kBytesV + wave * 1024;
+    const uint32_t kdst = lds_base + kbuf * T::kBytesK + wave * 1024;
+    const uint32_t vdst = lds_base + T::kOffV + vbuf * T::kBytesV + wave * 1024;
+    // V first: the barrier waits let the K half of a call stay in flight one vector phase longer
 #pragma unroll
     for (int i = 0; i < T::kLoads; ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rk, kdst + i * 8192, 16, (int)k_goff,
-                                               (int)(i * 8 * T::kRowsPerBlock * row_bytes), 0, 0);
+      load_block_to_lds(rv, v_goff, (uint32_t)(i * 8 * T::kRowsPerBlock) * row_bytes, vdst + i * 8192);
 #pragma unroll
     for (int i = 0; i < T::kLoads; ++i)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rv, vdst + i * 8192, 16, (int)v_goff,
-                                               (int)(i * 8 * T::kRowsPerBlock * row_bytes), 0, 0);
+      load_block_to_lds(rk, k_goff, (uint32_t)(i * 8 * T::kRowsPerBlock) * row_bytes, kdst + i * 8192);
     if (have) {
       ld_left -= kBK;
       ld_k += tile_bytes;
@@ -528,17 +545,22 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   // ---- prologue ---------------------------------------------------------------------------
   // Schedule of the loads (phases are separated by workgroup barriers; group g runs the vector
   // phase of tile t in phase 2t + g and its matrix phase in phase 2t + g + 1):
-  //   * in the vector phase of tile t a wavefront of group g issues its blocks of K of tile
-  //     t+3+g and of V of tile t+2+g, and waits for them at the end of the vector phase after
-  //     the next one, four phases later (a first-touch miss all the way to HBM is still hidden);
-  //   * K of tile X is first read in phase 2X-1 (scores, by group 0) and last in phase 2X, V of
-  //     tile X in phases 2X+1 and 2X+2: every block has arrived at least one barrier before its
-  //     first reader, and with four buffers per operand the buffer (X & 3) it overwrites was last
-  //     read (K of tile X-4: phase 2X-8, V of tile X-4: phase 2X-6) before the phase the load is
-  //     issued in (K: 2X-6 or 2X-7, V: 2X-4 or 2X-5).
-  // Here: K of tiles 0..2 and V of tiles 0..1 (group 1: one tile more); the trailing group then
-  // waits one phase, which is what staggers the two groups.  (The V half of
-  // the first call has no tile yet: it stores zeros into a buffer nobody reads.)
+  //   * K of tile X is read in phases 2X-1 and 2X (scores, matrix phases of tile X-1), V of tile X
+  //     at the end of phases 2X and 2X+1 (the operand ring's prefill) and in phases 2X+1 and 2X+2.
+  //   * A call of load_tile issues V of tile Y-1 and then K of tile Y.  In the vector phase of
+  //     tile t a wavefront of group g makes the call Y = t+3+g: with four buffers per operand the
+  //     slot a load overwrites (K of tile Y-4: last read in phase 2Y-8; V of tile Y-5: phase 2Y-8)
+  //     is free since the barrier before the phase the load is issued in (2Y-6 or 2Y-7).
+  //   * The barrier that ends a vector phase waits for all of the wavefront's loads but the newest
+  //     call and the K half of the call before: V of tile t+1+g and K of tile t+1+g are then in
+  //     the LDS for everybody, i.e. V one barrier before its first reader (the prefill in phase
+  //     2(t+1) + g at the earliest) after three phases in flight, K after five.
+  //   * At D = 64 the calls are made behind the MFMAs of the matrix phase instead (see
+  //     kLoadAfterMatrix); the barrier of the next vector phase then lets only the K half of the
+  //     newest call stay in flight.
+  // Here: the calls Y = 0..2 (group 1: ..3) -- the V half of the first has no tile, it stores
+  // zeros into a buffer nobody reads -- of which K of tile 0 (first scores) and V of tile 0 (first
+  // prefill) are awaited; the trailing group then waits one phase, which staggers the two groups.
   using U0 = std::integral_constant<int, 0>;
   using U1 = std::integral_constant<int, 1>;
   using U2 = std::integral_constant<int, 2>;
@@ -547,14 +569,13 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   load_tile(1);
   load_tile(2);
   if (group == 1) load_tile(3);
-  // only K of tile 0 (the first call) has to be there for the first scores; what the later
-  // phases need is awaited by the barriers of the vector phases before them
+  // in flight behind this wait: K of tile 1 and the calls after it (kLoads + 2 kLoads (1 + g) loads)
   if (group == 0) {
-    if constexpr (T::kLoads == 2) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    if constexpr (T::kLoads == 2) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
   } else {
-    if constexpr (T::kLoads == 2) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+    if constexpr (T::kLoads == 2) asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
   }
   phase_barrier();
   if (group == 1) phase_barrier();
@@ -668,7 +689,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     }
     l_run += rs0 + rs1;
     ring_prefill(u_tag);
-    phase_barrier_after_vector<(kLoadAfterMatrix ? 2 : 4) * T::kLoads>(p_frag);
+    phase_barrier_after_vector<(kLoadAfterMatrix ? 1 : 3) * T::kLoads>(p_frag);
 
     // ======== matrix phase: O^T += V^T P^T (tile t), S^T = K Q^T (tile t+1) ========
     __builtin_amdgcn_s_setprio(0);
@@ -690,6 +711,9 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     iteration(t + 2, U2{});
     iteration(t + 3, U3{});
   }
+  // tile loads issued for tiles past the end are still on their way (they store zeros): let them
+  // land before the epilogue reuses the tile buffers
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   // the leading group waits out the phase it is ahead
   if (group == 0) phase_barrier();
 
