@@ -136,7 +136,8 @@ struct RowAcc {
 constexpr int kMergeRows = 2;
 
 template <int D, int NB, bool ALL_BF16>
-__device__ __forceinline__ void merge_batch(const MergeArgs& a, int i0, int b, int h, const int (&s)[kMergeRows],
+__device__ __forceinline__ void merge_batch(const MergeArgs& a, int i0, const int (&b)[kMergeRows],
+                                            const int (&h)[kMergeRows], const int (&s)[kMergeRows],
                                             const bool (&live)[kMergeRows], const int64_t (&elem)[kMergeRows], int cc,
                                             RowAcc (&ra)[kMergeRows]) {
   float l[kMergeRows][NB];
@@ -151,7 +152,7 @@ __device__ __forceinline__ void merge_batch(const MergeArgs& a, int i0, int b, i
 #pragma unroll
     for (int p = 0; p < kMergeRows; ++p) {
       if (live[p]) {
-        l[p][j] = lp[lse_index(bsh, b, h, s[p], a.H, a.Sq)];
+        l[p][j] = lp[lse_index(bsh, b[p], h[p], s[p], a.H, a.Sq)];
         if (ALL_BF16) {
           const uint16_t* q = reinterpret_cast<const uint16_t*>(op) + elem[p] + 4 * cc;
           const u32x2 g0 = *reinterpret_cast<const u32x2*>(q);
@@ -197,27 +198,46 @@ __device__ __forceinline__ void merge_batch(const MergeArgs& a, int i0, int b, i
   }
 }
 
-// One workgroup = kMergeRows * 256/(D/8) consecutive queries of one (batch, head); a group of
-// D/8 lanes owns kMergeRows rows.  States are consumed in batches of kBatch (the remainder
-// through a fully unrolled smaller batch) and folded with the running-maximum rescale.
-template <int D, bool ALL_BF16>
+// One workgroup = kMergeRows * 256/(D/8) rows; a group of D/8 lanes owns kMergeRows rows.  Two
+// ways of handing rows to workgroups: consecutive queries of one (batch, head), workgroups ordered
+// head-fastest (the lse reads are contiguous, the row reads of concurrently running workgroups
+// are neighbours) -- or, LINEAR, consecutive rows of the [B,Sq,H,D] tensors (every stream a
+// workgroup reads is one contiguous block), which wins once many states are read at a time
+// (measured: 8 states +5 %, 16 states +3 %, 4 states +-3 %, 1-2 states -6 to -12 %).
+// States are consumed in batches of kBatch (the remainder through a fully unrolled smaller
+// batch) and folded with the running-maximum rescale.
+template <int D, bool ALL_BF16, bool LINEAR>
 __global__ __launch_bounds__(kThreads) void merge_states_kernel(const MergeArgs a) {
   constexpr int kLanesPerRow = D / 8;
   constexpr int kRowsPerPass = kThreads / kLanesPerRow;
   constexpr int kRowsPerWg = kRowsPerPass * kMergeRows;
-  int st, b, h;
-  decode_wg(blockIdx.x, a.B, a.H, st, b, h);
+  int st = 0, b0 = 0, h0 = 0;
+  if constexpr (!LINEAR) decode_wg(blockIdx.x, a.B, a.H, st, b0, h0);
   const int rr = threadIdx.x / kLanesPerRow;
   const int cc = threadIdx.x % kLanesPerRow;
-  int s[kMergeRows];
+  int s[kMergeRows], b[kMergeRows], h[kMergeRows];
   bool live[kMergeRows];
   int64_t elem[kMergeRows];
   RowAcc ra[kMergeRows];
+  const int64_t rows_total = (int64_t)a.B * a.Sq * a.H;
 #pragma unroll
   for (int p = 0; p < kMergeRows; ++p) {
-    s[p] = st * kRowsPerWg + p * kRowsPerPass + rr;
-    live[p] = s[p] < a.Sq;
-    elem[p] = (((int64_t)b * a.Sq + s[p]) * a.H + h) * D;
+    if constexpr (LINEAR) {
+      const int64_t row = (int64_t)blockIdx.x * kRowsPerWg + p * kRowsPerPass + rr;
+      live[p] = row < rows_total;
+      const int64_t rc = live[p] ? row : 0;
+      const int64_t bs = rc / a.H;
+      h[p] = (int)(rc - bs * a.H);
+      b[p] = (int)(bs / a.Sq);
+      s[p] = (int)(bs - (int64_t)b[p] * a.Sq);
+      elem[p] = rc * D;
+    } else {
+      b[p] = b0;
+      h[p] = h0;
+      s[p] = st * kRowsPerWg + p * kRowsPerPass + rr;
+      live[p] = s[p] < a.Sq;
+      elem[p] = (((int64_t)b0 * a.Sq + s[p]) * a.H + h0) * D;
+    }
     ra[p].m = -INFINITY;
     ra[p].den = 0.f;
 #pragma unroll
@@ -244,7 +264,7 @@ __global__ __launch_bounds__(kThreads) void merge_states_kernel(const MergeArgs 
     for (int k = 0; k < 8; ++k) o[k] = ra[p].acc[k] * inv;
     store_row8<D>(a.dst_out, a.dst_fp32 != 0, elem[p], cc, o);
     if (cc == 0 && a.dst_lse != nullptr)
-      a.dst_lse[lse_index(a.dst_bsh != 0, b, h, s[p], a.H, a.Sq)] =
+      a.dst_lse[lse_index(a.dst_bsh != 0, b[p], h[p], s[p], a.H, a.Sq)] =
           ra[p].den > 0.f ? ra[p].m + __logf(ra[p].den) : -INFINITY;
   }
 }
@@ -375,26 +395,36 @@ __global__ __launch_bounds__(kThreads) void rel_l1_sums_kernel(const float* a, c
 
 // ---- host-side launchers ---------------------------------------------------------------
 
+constexpr int kLinearFrom = 6;  // states per launch from which rows are handed out in memory order
+
+template <int D>
+static void launch_merge_d(const MergeArgs& a, bool all_bf16, bool linear, unsigned wgs, hipStream_t stream) {
+  if (linear) {
+    if (all_bf16) hipLaunchKernelGGL((merge_states_kernel<D, true, true>), dim3(wgs), dim3(kThreads), 0, stream, a);
+    else hipLaunchKernelGGL((merge_states_kernel<D, false, true>), dim3(wgs), dim3(kThreads), 0, stream, a);
+  } else {
+    if (all_bf16) hipLaunchKernelGGL((merge_states_kernel<D, true, false>), dim3(wgs), dim3(kThreads), 0, stream, a);
+    else hipLaunchKernelGGL((merge_states_kernel<D, false, false>), dim3(wgs), dim3(kThreads), 0, stream, a);
+  }
+}
+
 int launch_merge(const MergeArgs& a, int D, hipStream_t stream) {
+  if (D != 128 && D != 64) {
+    set_error("head dim %d not built (64 and 128 are)", D);
+    return DT_ERR_UNSUPPORTED;
+  }
   const int rows_per_wg = kThreads / (D / 8) * kMergeRows;
+  const bool linear = a.n >= kLinearFrom;
   const int n_st = (a.Sq + rows_per_wg - 1) / rows_per_wg;
-  const int64_t wgs = (int64_t)a.B * a.H * n_st;
+  const int64_t wgs = linear ? ((int64_t)a.B * a.Sq * a.H + rows_per_wg - 1) / rows_per_wg : (int64_t)a.B * a.H * n_st;
   if (wgs <= 0) return DT_OK;
   if (wgs > 0x7fffffffLL) {
     set_error("merge grid too large");
     return DT_ERR_INVALID;
   }
   const bool all_bf16 = (a.fp32_mask == 0);
-  if (D == 128) {
-    if (all_bf16) hipLaunchKernelGGL((merge_states_kernel<128, true>), dim3((unsigned)wgs), dim3(kThreads), 0, stream, a);
-    else hipLaunchKernelGGL((merge_states_kernel<128, false>), dim3((unsigned)wgs), dim3(kThreads), 0, stream, a);
-  } else if (D == 64) {
-    if (all_bf16) hipLaunchKernelGGL((merge_states_kernel<64, true>), dim3((unsigned)wgs), dim3(kThreads), 0, stream, a);
-    else hipLaunchKernelGGL((merge_states_kernel<64, false>), dim3((unsigned)wgs), dim3(kThreads), 0, stream, a);
-  } else {
-    set_error("head dim %d not built (64 and 128 are)", D);
-    return DT_ERR_UNSUPPORTED;
-  }
+  if (D == 128) launch_merge_d<128>(a, all_bf16, linear, (unsigned)wgs, stream);
+  else launch_merge_d<64>(a, all_bf16, linear, (unsigned)wgs, stream);
   return hip_fail(hipGetLastError(), "merge_states launch");
 }
 

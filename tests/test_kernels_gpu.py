@@ -110,7 +110,8 @@ def test_multi_chunk_job_equals_merge_of_chunks(hip):
     assert (outs[2].float() == 0).all()
 
 
-@pytest.mark.parametrize("D,n,src_fp32", [(128, 1, False), (128, 5, False), (64, 8, False), (128, 3, True), (64, 33, False)])
+@pytest.mark.parametrize("D,n,src_fp32", [(128, 1, False), (128, 5, False), (64, 8, False), (128, 3, True), (64, 33, False),
+                                          (128, 6, False), (128, 7, True), (64, 9, True)])
 def test_merge_states_matches_closed_form(hip, D, n, src_fp32):
     B, Sq, H = 2, 150, 3
     g = torch.Generator().manual_seed(n * 7 + D)
@@ -151,6 +152,25 @@ def test_merge_all_empty_and_layouts(hip):
     torch.cuda.synchronize()
     assert r_out.data_ptr() == a_out.data_ptr()
     assert (a_out.float().cpu() - ref_out).abs().max() < 2e-2
+    assert (a_lse.cpu().squeeze(-1).transpose(1, 2) - ref_lse).abs().max() < 1e-5
+
+
+@pytest.mark.parametrize("D", [64, 128])
+def test_merge_many_states_in_place_with_row_layout_lse(hip, D):
+    """Six states and more take the kernel's other row-to-workgroup mapping: in place into the first
+    state (bf16 destination), lse of that state in the running [B,S,H,1] layout, a repeated pointer."""
+    B, Sq, H, n = 2, 77, 5, 7
+    g = torch.Generator().manual_seed(D)
+    outs = [torch.randn(B, Sq, H, D, generator=g).bfloat16() for _ in range(n)]
+    lses = [torch.randn(B, H, Sq, generator=g) * 2 for _ in range(n)]
+    lses[3][:, :, 1::3] = -math.inf
+    ref_out, ref_lse = om.merge_states_closed_form(outs + [outs[2]], lses + [lses[2]])
+    d_outs = [o.cuda() for o in outs]
+    d_lses = [l.cuda() for l in lses]
+    a_lse = lses[0].transpose(1, 2).contiguous().unsqueeze(-1).cuda()
+    hip.merge_states(d_outs + [d_outs[2]], [a_lse] + d_lses[1:] + [d_lses[2]], dst_out=d_outs[0], dst_lse=a_lse)
+    torch.cuda.synchronize()
+    assert (d_outs[0].float().cpu() - ref_out).abs().max() < 2e-2
     assert (a_lse.cpu().squeeze(-1).transpose(1, 2) - ref_lse).abs().max() < 1e-5
 
 
