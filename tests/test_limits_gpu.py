@@ -81,16 +81,18 @@ def test_forty_way_merge_and_its_limit(hip):
         hip.merge_states([x.cuda() for x in outs] + [outs[0].cuda()], [x.cuda() for x in lses] + [lses[0].cuda()])
 
 
-@pytest.mark.parametrize("Sk", [63, 64, 65, 127, 128, 129, 191, 193, 320])
-def test_tile_counts_around_the_iteration_pairs(hip, Sk):
-    """1, 2, 3, 4 and 5 key tiles, full and ragged: odd counts run one key-less tile extra."""
-    B, Sq, H, D = 1, 96, 1, 128
+@pytest.mark.parametrize("Sk", [63, 64, 65, 127, 128, 129, 191, 193, 256, 257, 320, 449, 512, 513, 577])
+@pytest.mark.parametrize("D", [64, 128])
+def test_tile_counts_around_the_unrolled_iterations(hip, Sk, D):
+    """1 to 10 key tiles, full and ragged: the loop runs four tiles per trip (one per LDS buffer), counts
+    that are not multiples of four run key-less tiles extra."""
+    B, Sq, H = 1, 96, 1
     g = torch.Generator().manual_seed(Sk)
     q, k, v = _rand((B, Sq, H, D), g), _rand((B, Sk, H, D), g), _rand((B, Sk, H, D), g)
     ref = om.chunk_attention(q, k, v)
     out, lse = hip.attn_chunk_fwd(q.cuda(), k.cuda(), v.cuda())
     torch.cuda.synchronize()
-    _check(out, lse, *ref, f"Sk={Sk}")
+    _check(out, lse, *ref, f"Sk={Sk} D={D}")
 
 
 def test_c_abi_rejects_without_launching(hip):
