@@ -37,11 +37,12 @@ Pinning status (what fixes each function besides "it restates the source"):
   N in {2,4,8} and random ones for N=16: send/recv pairing of the simulated
   ring, every chunk contributing exactly once per call (except the documented
   double count), constant-input steps reproducing full attention.
-* divider map: pinned on the three redundancy maps the reference ships
-  (``configs/*/redundancy_map_50_*.pt``) by the structural rules of
-  ``_refine_divider_map`` and by the divider histograms an independent
-  restatement produced; a golden map produced by running the reference itself
-  does not exist, so that part is **parity unpinned** beyond those checks.
+* divider map: pinned bit-exact against the REFERENCE'S OWN OUTPUT on the three
+  redundancy maps it ships (``configs/*/redundancy_map_50_*.pt`` with the
+  percentiles and dividers of its ``config.yaml`` files) for ring sizes 2, 4, 8
+  and 16: ``tests/golden/divider_maps.npz``, written by
+  ``tests/golden/make_divider_fixtures.py``, which imports the two functions from
+  the reference tree; and by the structural rules of ``_refine_divider_map``.
 * producer: RMSNorm / LayerNorm pinned against ``torch.nn.functional.rms_norm``
   / ``layer_norm``; interleaved RoPE against complex multiplication
   (``torch.view_as_complex``); rotate-half RoPE against explicit 2x2 rotations,

@@ -141,3 +141,50 @@ def test_divider_generation_edge_cases():
     # base weight not divisible: falls to the smallest listed divider that divides it (:264-271)
     div6, _ = od.generate_divider_map(red, 6, [25, 50, 75], [8, 4, 2, 1])
     assert set(np.unique(div6)) <= {1, 2, 6}
+
+
+# ---- against the reference's own output ---------------------------------------------------------
+# tests/golden/divider_maps.npz holds what the reference's generate_divider_map_from_redundancy +
+# _refine_divider_map (core/redundancy_map.py:199-326) return on the shipped maps for ring sizes
+# 2, 4, 8 and 16 (written by tests/golden/make_divider_fixtures.py, which imports those two
+# functions from the reference tree).  Integer work: bit exact.
+REFERENCE_OUTPUT = np.load(os.path.join(GOLDEN, "divider_maps.npz"))
+
+
+@pytest.mark.parametrize("N", [2, 4, 8, 16])
+@pytest.mark.parametrize("name", list(MODELS))
+def test_oracle_equals_reference_output(name, N):
+    red, pct, dv = _load(name)
+    key = name.replace("-", "_")
+    assert np.array_equal(REFERENCE_OUTPUT[f"{key}.redundancy"], red.numpy())          # same inputs
+    assert list(REFERENCE_OUTPUT[f"{key}.percentiles"]) == pct and list(REFERENCE_OUTPUT[f"{key}.dividers"]) == dv
+    div, thresholds = od.generate_divider_map(red.numpy(), N, pct, dv)
+    assert np.array_equal(np.asarray(thresholds, dtype=np.float64), REFERENCE_OUTPUT[f"{key}.N{N}.thresholds"])
+    assert np.array_equal(div, REFERENCE_OUTPUT[f"{key}.N{N}.generated"])
+    refined, changes = od.refine_divider_map(div)
+    assert np.array_equal(refined, REFERENCE_OUTPUT[f"{key}.N{N}.refined"])
+    assert changes == int(REFERENCE_OUTPUT[f"{key}.N{N}.changes"])
+
+
+@pytest.mark.parametrize("N", [2, 4, 8, 16])
+@pytest.mark.parametrize("name", list(MODELS))
+def test_product_equals_reference_output(name, N):
+    """The host-side RedundancyMap of the package (what init_redundancy_map builds from a .pt file)."""
+    from ditango_amd.core import config, parallel_state, redundancy_map as rmod
+
+    red, pct, dv = _load(name)
+    key = name.replace("-", "_")
+    parallel_state.init_local_groups(N, 0)
+    cfg = config.init_config(None, num_inference_steps=50, num_layers=MODELS[name][1], stride_percentiles=pct,
+                             stride_dividers=dv)
+    rmod.destroy_redundancy_map()
+    try:
+        rm = rmod.RedundancyMap(cfg)
+        rm.redundancy_map = red
+        rm.generate_divider_map_from_redundancy(custom_percentages=pct, custom_dividers=dv)
+        assert np.array_equal(rm.divider_map.numpy(), REFERENCE_OUTPUT[f"{key}.N{N}.generated"])
+        rm._refine_divider_map()
+        assert np.array_equal(rm.divider_map.numpy(), REFERENCE_OUTPUT[f"{key}.N{N}.refined"])
+    finally:
+        rmod.destroy_redundancy_map()
+        parallel_state.destroy_local_groups()
