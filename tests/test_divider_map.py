@@ -188,3 +188,11 @@ def test_product_equals_reference_output(name, N):
     finally:
         rmod.destroy_redundancy_map()
         parallel_state.destroy_local_groups()
+
+
+def test_golden_stride_schedules_start_from_the_reference_dividers():
+    """The committed stride schedules (made from the oracle) were generated from dividers that equal
+    the reference's own refined maps for a ring of 8."""
+    stride = np.load(os.path.join(GOLDEN, "stride_schedules.npz"))
+    for short, key in (("cogvideox", "cogvideox_5b"), ("hunyuanvideo", "hunyuanvideo"), ("stepvideo", "stepvideo")):
+        assert np.array_equal(stride[f"{short}/dividers"], REFERENCE_OUTPUT[f"{key}.N8.refined"])
