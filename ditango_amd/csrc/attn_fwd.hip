@@ -196,9 +196,17 @@ __device__ __forceinline__ u32x4 make_rsrc(const void* base, uint32_t valid_byte
 // vmcnt in front of the barriers.  (Loads the compiler does not know of only make its own vmcnt
 // waits for other loads stricter, never too weak: the counter retires in order.)
 __device__ __forceinline__ void load_block_to_lds(u32x4 rsrc, uint32_t lane_off, uint32_t uniform_off, uint32_t lds_addr) {
+  // (the uniform operands are uniform by construction; say so, or a value the compiler happens to
+  // hold in a vector register ends up in the instruction as one)
+  u32x4 r;
+  r.x = __builtin_amdgcn_readfirstlane(rsrc.x);
+  r.y = __builtin_amdgcn_readfirstlane(rsrc.y);
+  r.z = __builtin_amdgcn_readfirstlane(rsrc.z);
+  r.w = __builtin_amdgcn_readfirstlane(rsrc.w);
   asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds"
                :
-               : "v"(lane_off), "s"(rsrc), "s"(uniform_off), "s"(lds_addr)
+               : "v"(lane_off), "s"(r), "s"(__builtin_amdgcn_readfirstlane(uniform_off)),
+                 "s"(__builtin_amdgcn_readfirstlane(lds_addr))
                : "memory", "m0");
 }
 
@@ -391,7 +399,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   // the barrier waits on is static.
   const uint8_t* prev_v = nullptr;  // V of the tile the previous call loaded K of
   uint32_t prev_valid = 0u;
-  auto load_tile = [&](int kbuf) {
+  auto load_tile = [&](int kbuf) __attribute__((always_inline)) {
     const bool have = __builtin_expect(ld_seg < seg_end, 1);
     const uint32_t valid = have ? (uint32_t)(ld_left - 1) * row_bytes + (uint32_t)(D * 2) : 0u;
     const u32x4 rk = make_rsrc(ld_k, valid);
@@ -451,7 +459,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   int cp_valid = 0;      // keys that exist in the tile held in s_acc
 
   // S^T = K Q^T for tile 0 only (first matrix phase)
-  auto qk_only = [&]() {
+  auto qk_only = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
@@ -497,7 +505,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
 #pragma unroll
     for (int i = 0; i < kRing; ++i) ring[i] = v_frag(kU, i);
   };
-  auto matrix_phase = [&](auto u_tag) {
+  auto matrix_phase = [&](auto u_tag) __attribute__((always_inline)) {
     constexpr int kU = decltype(u_tag)::value;         // V buffer of this tile
     constexpr int kUK = (kU + 1) & (kNumBuf - 1);      // K buffer of the next tile
     auto frag = [&](int i) -> bf16x8 {
@@ -589,7 +597,7 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
   phase_barrier_after_matrix(s_acc, o_acc);
 
   // one iteration = vector phase of tile t, then matrix phase (P V of tile t, scores of t+1)
-  auto iteration = [&](int t, auto u_tag) {
+  auto iteration = [&](int t, auto u_tag) __attribute__((always_inline)) {
     constexpr int kU = decltype(u_tag)::value;  // t & 3
     // ======== vector phase: tile loads for later, online softmax of tile t ========
     // The vector phase runs at raised wave priority: where the two wavefronts of a SIMD compete for
@@ -695,20 +703,23 @@ __global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a)
     __builtin_amdgcn_s_setprio(0);
     matrix_phase(u_tag);
     if constexpr (kLoadAfterMatrix) load_tile((kU + 3 + group) & (kNumBuf - 1));
-    // the tile after the last one of this workgroup's range has no keys for it (it is the
-    // padding of the tile count, or belongs to the next part of a split item)
+    // the tile after the last one of this workgroup's range has no keys for it (its scores are
+    // computed on whatever the buffer holds and never used; it may belong to the next part of a
+    // split item)
     cp_valid = t + 1 < n_tiles ? cp_left : 0;
     cp_left -= kBK;
     if (cp_left <= 0) cp_next_chunk();
     phase_barrier_after_matrix(s_acc, o_acc);
   };
-  // Iterations come in fours (one per LDS buffer); the tile count is rounded up with tiles that
-  // have no keys: their scores are masked, they add zeros.
-  const int n_iter = (n_tiles + 3) & ~3;
-  for (int t = 0; t < n_iter; t += 4) {
+  // Iterations come in fours (one per LDS buffer, so that buffer offsets are immediates); the last
+  // round stops after the last tile.
+  for (int t = 0; t < n_tiles; t += 4) {
     iteration(t, U0{});
+    if (t + 1 >= n_tiles) break;
     iteration(t + 1, U1{});
+    if (t + 2 >= n_tiles) break;
     iteration(t + 2, U2{});
+    if (t + 3 >= n_tiles) break;
     iteration(t + 3, U3{});
   }
   // tile loads issued for tiles past the end are still on their way (they store zeros): let them

@@ -84,8 +84,8 @@ def test_forty_way_merge_and_its_limit(hip):
 @pytest.mark.parametrize("Sk", [63, 64, 65, 127, 128, 129, 191, 193, 256, 257, 320, 449, 512, 513, 577])
 @pytest.mark.parametrize("D", [64, 128])
 def test_tile_counts_around_the_unrolled_iterations(hip, Sk, D):
-    """1 to 10 key tiles, full and ragged: the loop runs four tiles per trip (one per LDS buffer), counts
-    that are not multiples of four run key-less tiles extra."""
+    """1 to 10 key tiles, full and ragged: the loop runs four tiles per trip (one per LDS buffer) and
+    leaves the last trip after the last tile."""
     B, Sq, H = 1, 96, 1
     g = torch.Generator().manual_seed(Sk)
     q, k, v = _rand((B, Sq, H, D), g), _rand((B, Sk, H, D), g), _rand((B, Sk, H, D), g)
