@@ -208,12 +208,18 @@ def test_size_independent_properties_at_hunyuan_shape(hip):
     assert torch.equal(back_o, outs[3]) and torch.equal(back_l, lses[3])
 
 
-def test_attention_is_deterministic_at_hunyuan_shape(hip):
-    """Five launches over the same inputs at the HunyuanVideo per-rank shape give bit-identical states
-    (an LDS hazard between the two wavefront groups would show up as run-to-run differences)."""
-    B, H, D, Sq, Sk = 1, 24, 128, 14882, 14882
+@pytest.mark.parametrize("H,D,Sq,Sk,prescaled", [(24, 128, 14882, 14882, False), (48, 64, 2222, 2222, False),
+                                                  (48, 64, 2222, 2222, True), (24, 128, 3000, 14882, True)])
+def test_attention_is_deterministic_at_full_shapes(hip, H, D, Sq, Sk, prescaled):
+    """Five launches over the same inputs at the HunyuanVideo and CogVideoX per-rank shapes give
+    bit-identical states (a hazard between the tile loads into the LDS, or between the two wavefront
+    groups, would show up as run-to-run differences)."""
+    B = 1
     g = torch.Generator(device="cuda").manual_seed(12)
-    q = torch.randn(B, Sq, H, D, generator=g, device="cuda").bfloat16()
+    q = torch.randn(B, Sq, H, D, generator=g, device="cuda")
+    if prescaled:
+        q = q * (D ** -0.5 * 1.4426950408889634)
+    q = q.bfloat16()
     ks = [torch.randn(B, Sk, H, D, generator=g, device="cuda").bfloat16() for _ in range(2)]
     vs = [torch.randn(B, Sk, H, D, generator=g, device="cuda").bfloat16() for _ in range(2)]
     table = hip.ChunkTable(ks, vs)
@@ -222,7 +228,7 @@ def test_attention_is_deterministic_at_hunyuan_shape(hip):
         for i in range(5):
             outs = [torch.empty(B, Sq, H, D, dtype=torch.bfloat16, device="cuda") for _ in range(3)]
             lses = [torch.empty(B, H, Sq, dtype=torch.float32, device="cuda") for _ in range(3)]
-            hip.attn_jobs_fwd(q, table, [[0], [1], [0, 1]], outs, lses, workspace=ws)
+            hip.attn_jobs_fwd(q, table, [[0], [1], [0, 1]], outs, lses, workspace=ws, q_prescaled=prescaled)
             torch.cuda.synchronize()
             if ref is None:
                 ref = (outs, lses)
