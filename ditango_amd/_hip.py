@@ -24,7 +24,7 @@ DT_ATTN_Q_PRESCALED = 1
 DT_MAX_CHUNKS = 40
 DT_MAX_JOBS = 40
 DT_MAX_JOB_ENTRIES = 64
-DT_MAX_MERGE = 40
+DT_MAX_MERGE = 64
 DT_MAX_SEGMENTS = 8
 
 c_i32, c_i64, c_f32, c_vp = ctypes.c_int32, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
@@ -189,17 +189,19 @@ def attn_workspace(device) -> torch.Tensor:
 
 
 class ChunkTable:
-    """Host-side table of the KV chunks one layer call can touch (pointers, lengths, strides)."""
+    """Host-side table of the KV chunks one layer call can touch (pointers, lengths, strides).  A table
+    may hold more chunks than one launch can address (``DT_MAX_CHUNKS``); the job launches then pass the
+    sub-table of the chunks their jobs reference."""
 
     def __init__(self, k_chunks: Sequence[torch.Tensor], v_chunks: Sequence[torch.Tensor]):
         n = len(k_chunks)
-        _require(0 < n <= DT_MAX_CHUNKS and n == len(v_chunks), f"need 1..{DT_MAX_CHUNKS} KV chunks")
+        _require(n > 0 and n == len(v_chunks), "need at least one KV chunk and as many V as K chunks")
         self.n = n
         self.keep = (list(k_chunks), list(v_chunks))  # keep the tensors alive while pointers are in use
-        self.k_ptrs = (c_vp * n)()
-        self.v_ptrs = (c_vp * n)()
-        self.lens = (c_i32 * n)()
-        self.sb = (c_i64 * n)()
+        self._k: List[int] = []
+        self._v: List[int] = []
+        self._len: List[int] = []
+        self._sb: List[int] = []
         ss = sh = None
         for i, (k, v) in enumerate(zip(k_chunks, v_chunks)):
             _check_qkv(k, f"k[{i}]"); _check_qkv(v, f"v[{i}]")
@@ -210,12 +212,43 @@ class ChunkTable:
                     self.B, self.H, self.D = k.shape[0], k.shape[2], k.shape[3]
                 _require((k.stride(1), k.stride(2)) == (ss, sh), "all chunks must share token/head strides")
                 _require((k.shape[0], k.shape[2], k.shape[3]) == (self.B, self.H, self.D), "chunk B/H/D mismatch")
-            self.k_ptrs[i] = k.data_ptr()
-            self.v_ptrs[i] = v.data_ptr()
-            self.lens[i] = k.shape[1]
-            self.sb[i] = k.stride(0)
+            self._k.append(k.data_ptr())
+            self._v.append(v.data_ptr())
+            self._len.append(k.shape[1])
+            self._sb.append(k.stride(0))
         _require(ss is not None, "all KV chunks are empty")
         self.ss, self.sh = ss, sh
+        self._whole = self.arrays(range(n)) if n <= DT_MAX_CHUNKS else None
+
+    def arrays(self, ids: Sequence[int]):
+        """ctypes arrays (k_ptrs, v_ptrs, lens, batch strides) of the chunks ``ids``, in that order."""
+        ids = list(ids)
+        m = len(ids)
+        _require(0 < m <= DT_MAX_CHUNKS, f"one launch addresses 1..{DT_MAX_CHUNKS} KV chunks, not {m}")
+        return ((c_vp * m)(*[self._k[i] for i in ids]), (c_vp * m)(*[self._v[i] for i in ids]),
+                (c_i32 * m)(*[self._len[i] for i in ids]), (c_i64 * m)(*[self._sb[i] for i in ids]))
+
+    def whole(self):
+        """The arrays of all chunks (tables that fit one launch)."""
+        _require(self._whole is not None, f"the table holds {self.n} chunks, one launch addresses {DT_MAX_CHUNKS}")
+        return self._whole
+
+    # the whole-table arrays under their old names
+    @property
+    def k_ptrs(self):
+        return self.whole()[0]
+
+    @property
+    def v_ptrs(self):
+        return self.whole()[1]
+
+    @property
+    def lens(self):
+        return self.whole()[2]
+
+    @property
+    def sb(self):
+        return self.whole()[3]
 
 
 def attn_jobs_fwd(q: torch.Tensor, table: ChunkTable, jobs: Sequence[Sequence[int]],
@@ -246,14 +279,29 @@ def attn_jobs_fwd(q: torch.Tensor, table: ChunkTable, jobs: Sequence[Sequence[in
         _require(o.dtype == torch.bfloat16 and o.is_contiguous() and tuple(o.shape) == (B, Sq, H, D), f"outs[{j}] must be contiguous bf16 [B,Sq,H,D]")
         _require(l.dtype == torch.float32 and l.is_contiguous() and tuple(l.shape) == (B, H, Sq), f"lses[{j}] must be contiguous fp32 [B,H,Sq]")
         _require(len(jobs[j]) <= DT_MAX_JOB_ENTRIES, f"job {j} references more than {DT_MAX_JOB_ENTRIES} chunks")
-    # split into launches that fit the per-launch limits
+    # split into launches that fit the per-launch limits (jobs, chunk references, distinct chunks)
     start = 0
     while start < nj:
         end, entries = start, 0
+        used = set()
         while end < nj and end - start < DT_MAX_JOBS and entries + len(jobs[end]) <= DT_MAX_JOB_ENTRIES:
+            more = used | {int(c) for c in jobs[end]}
+            if table.n > DT_MAX_CHUNKS and len(more) > DT_MAX_CHUNKS:
+                break
+            used = more
             entries += len(jobs[end])
             end += 1
+        _require(end > start, f"job {start} references more than {DT_MAX_CHUNKS} distinct chunks: split it and merge the parts")
         n = end - start
+        if table.n <= DT_MAX_CHUNKS:
+            t_k, t_v, t_len, t_sb = table.whole()
+            t_n = table.n
+            local = None
+        else:
+            ids = sorted(used) or [0]
+            t_k, t_v, t_len, t_sb = table.arrays(ids)
+            t_n = len(ids)
+            local = {c: i for i, c in enumerate(ids)}
         begin = (c_i32 * (n + 1))()
         flat: List[int] = []
         kvb: List[int] = []
@@ -263,7 +311,8 @@ def attn_jobs_fwd(q: torch.Tensor, table: ChunkTable, jobs: Sequence[Sequence[in
             begin[jj] = len(flat)
             for i, c in enumerate(jobs[j]):
                 c = int(c)
-                flat.append(c)
+                _require(0 <= c < table.n, f"job {j} references chunk {c} outside the table of {table.n}")
+                flat.append(c if local is None else local[c])
                 if kv_ranges is not None:
                     kvb.append(int(kv_ranges[j][i][0]))
                     kvl.append(int(kv_ranges[j][i][1]))
@@ -276,14 +325,15 @@ def attn_jobs_fwd(q: torch.Tensor, table: ChunkTable, jobs: Sequence[Sequence[in
         a_ql = (c_i32 * n)(*[int(q_ranges[start + jj][1]) for jj in range(n)]) if q_ranges is not None else None
         out_ptrs = (c_vp * n)(*[outs[start + jj].data_ptr() for jj in range(n)])
         lse_ptrs = (c_vp * n)(*[lses[start + jj].data_ptr() for jj in range(n)])
-        rc = lib.dt_attn_seg_jobs_ws_fwd(q.data_ptr(), B, Sq, H, D, q.stride(0), q.stride(1), q.stride(2),
-                                         table.n, table.k_ptrs, table.v_ptrs, table.lens, table.sb, table.ss, table.sh,
-                                         n, begin, chunks, a_kvb, a_kvl, a_qb, a_ql, out_ptrs, lse_ptrs,
-                                         float(softmax_scale), DT_ATTN_Q_PRESCALED if q_prescaled else 0,
-                                         workspace.data_ptr() if workspace is not None else None,
-                                         workspace.numel() * workspace.element_size() if workspace is not None else 0,
-                                         _stream())
-        _check(rc, "dt_attn_seg_jobs_ws_fwd")
+        if True:
+            rc = lib.dt_attn_seg_jobs_ws_fwd(q.data_ptr(), B, Sq, H, D, q.stride(0), q.stride(1), q.stride(2),
+                                             t_n, t_k, t_v, t_len, t_sb, table.ss, table.sh,
+                                             n, begin, chunks, a_kvb, a_kvl, a_qb, a_ql, out_ptrs, lse_ptrs,
+                                             float(softmax_scale), DT_ATTN_Q_PRESCALED if q_prescaled else 0,
+                                             workspace.data_ptr() if workspace is not None else None,
+                                             workspace.numel() * workspace.element_size() if workspace is not None else 0,
+                                             _stream())
+            _check(rc, "dt_attn_seg_jobs_ws_fwd")
         start = end
 
 
@@ -341,16 +391,9 @@ def attn_sched_fwd(q: torch.Tensor, table: ChunkTable, dev_compute_ids: torch.Te
 # K2: merge, K3: cache store/load
 # ---------------------------------------------------------------------------------------------
 
-def merge_states(outs: Sequence[torch.Tensor], lses: Sequence[torch.Tensor],
-                 dst_out: Optional[torch.Tensor] = None, dst_lse: Optional[torch.Tensor] = None,
-                 dst_dtype: torch.dtype = torch.float32, dst_lse_bsh: bool = False):
-    """N-way LSE merge in one pass.  outs[i] contiguous [B,Sq,H,D] (bf16 or fp32), lses[i] fp32 in
-    [B,H,Sq] or [B,Sq,H(,1)] storage.  Returns (dst_out, dst_lse)."""
+def _merge_once(outs, lses, dst_out, dst_lse, B, Sq, H, D) -> None:
     lib = load_library()
     n = len(outs)
-    _require(0 < n <= DT_MAX_MERGE and n == len(lses), f"need 1..{DT_MAX_MERGE} states")
-    B, Sq, H, D = outs[0].shape
-    dev = outs[0].device
     out_ptrs = (c_vp * n)()
     lse_ptrs = (c_vp * n)()
     dts = (c_i32 * n)()
@@ -361,15 +404,40 @@ def merge_states(outs: Sequence[torch.Tensor], lses: Sequence[torch.Tensor],
         lse_ptrs[i] = l.data_ptr()
         dts[i] = _dtype_code(o)
         lays[i] = lse_layout_of(l, B, Sq, H)
+    dlay = lse_layout_of(dst_lse, B, Sq, H)
+    rc = lib.dt_merge_states(n, out_ptrs, lse_ptrs, dts, lays, dst_out.data_ptr(), _dtype_code(dst_out),
+                             dst_lse.data_ptr(), dlay, B, Sq, H, D, _stream())
+    _check(rc, "dt_merge_states")
+
+
+def merge_states(outs: Sequence[torch.Tensor], lses: Sequence[torch.Tensor],
+                 dst_out: Optional[torch.Tensor] = None, dst_lse: Optional[torch.Tensor] = None,
+                 dst_dtype: torch.dtype = torch.float32, dst_lse_bsh: bool = False):
+    """N-way LSE merge.  outs[i] contiguous [B,Sq,H,D] (bf16 or fp32), lses[i] fp32 in
+    [B,H,Sq] or [B,Sq,H(,1)] storage.  Returns (dst_out, dst_lse).  Up to ``DT_MAX_MERGE`` states are one
+    pass over HBM; more are folded in rounds through a running fp32 state that is updated in place (the
+    merge is associative; the running state is never rounded below fp32)."""
+    n = len(outs)
+    _require(n > 0 and n == len(lses), "need at least one state and one lse per state")
+    B, Sq, H, D = outs[0].shape
+    dev = outs[0].device
     if dst_out is None:
         dst_out = torch.empty((B, Sq, H, D), dtype=dst_dtype, device=dev)
     if dst_lse is None:
         dst_lse = torch.empty((B, Sq, H, 1) if dst_lse_bsh else (B, H, Sq), dtype=torch.float32, device=dev)
     _require(dst_out.is_contiguous() and tuple(dst_out.shape) == (B, Sq, H, D), "dst_out must be contiguous [B,Sq,H,D]")
-    dlay = lse_layout_of(dst_lse, B, Sq, H)
-    rc = lib.dt_merge_states(n, out_ptrs, lse_ptrs, dts, lays, dst_out.data_ptr(), _dtype_code(dst_out),
-                             dst_lse.data_ptr(), dlay, B, Sq, H, D, _stream())
-    _check(rc, "dt_merge_states")
+    outs, lses = list(outs), list(lses)
+    if n > DT_MAX_MERGE:
+        run_out = torch.empty((B, Sq, H, D), dtype=torch.float32, device=dev)
+        run_lse = torch.empty((B, H, Sq), dtype=torch.float32, device=dev)
+        _merge_once(outs[:DT_MAX_MERGE], lses[:DT_MAX_MERGE], run_out, run_lse, B, Sq, H, D)
+        i = DT_MAX_MERGE
+        while n - i > DT_MAX_MERGE - 1:
+            _merge_once([run_out] + outs[i:i + DT_MAX_MERGE - 1], [run_lse] + lses[i:i + DT_MAX_MERGE - 1],
+                        run_out, run_lse, B, Sq, H, D)
+            i += DT_MAX_MERGE - 1
+        outs, lses = [run_out] + outs[i:], [run_lse] + lses[i:]
+    _merge_once(outs, lses, dst_out, dst_lse, B, Sq, H, D)
     return dst_out, dst_lse
 
 

@@ -146,8 +146,27 @@ def plan_call(N: int, r: int, curr: int, nxt: int, targets: List[int], use_ditan
     return plan, targets
 
 
+_warned_cast = set()
+
+
+def _kernel_input(t: torch.Tensor) -> torch.Tensor:
+    """The kernels read bf16.  fp32 / fp16 inputs (flash_attn_func itself only takes fp16 / bf16; the
+    reference's CPU-runnable case is stated in fp32) are rounded to bf16 here, once, explicitly: the
+    result is then the attention of the ROUNDED inputs, which differs from fp32 attention of the
+    unrounded ones by the input rounding (2^-9 relative per element)."""
+    if t is None or t.dtype == torch.bfloat16:
+        return t
+    if t.dtype not in (torch.float32, torch.float16):
+        raise TypeError(f"attention inputs must be bf16, fp16 or fp32, got {t.dtype}")
+    if t.dtype not in _warned_cast:
+        _warned_cast.add(t.dtype)
+        logger.warning(f"attention inputs of dtype {t.dtype} are rounded to bf16 at the kernel boundary")
+    return t.to(torch.bfloat16)
+
+
 def _as4d(t: torch.Tensor, B: int) -> torch.Tensor:
-    """Packed ``[B*S, H, D]`` (the varlen entry's layout) viewed as ``[B, S, H, D]``."""
+    """Packed ``[B*S, H, D]`` (the varlen entry's layout) viewed as ``[B, S, H, D]``, in the kernels' dtype."""
+    t = _kernel_input(t)
     return t if t.dim() == 4 else t.view(B, t.shape[0] // B, t.shape[1], t.shape[2])
 
 
@@ -182,6 +201,8 @@ class proAttention:
         if self.layer_id == 0:
             logger.info(f"R{self.global_rank}L{layer_id} | cached block attention on HIP kernels (gfx950)")
 
+    _MAX_JOB_CHUNKS = 32  # chunks of one block computed as one job (a launch addresses _hip.DT_MAX_CHUNKS)
+
     # ---- stride mode ------------------------------------------------------------------------------
     def _strides(self, timestep: int) -> Tuple[int, int]:
         rm = get_redundancy_map()
@@ -192,6 +213,8 @@ class proAttention:
         """query ``[B,Sq,H,D]``, key/value ``[B,Sk,H,D]`` = this rank's shard (bf16).
         Returns fp32 ``[B,Sq,H,D]`` (core/attention.py:74-237)."""
         rm = get_redundancy_map()
+        if not self.dry_run:
+            query, key, value = _kernel_input(query), _kernel_input(key), _kernel_input(value)
         if rm is not None and rm.chunk_mask is not None and not self.dry_run:
             return self._attn_masked(query, key, value)
         timestep = get_timestep()
@@ -279,6 +302,7 @@ class proAttention:
         # one launch for all distinct states; a chunk computed twice by the reference
         # (local + own) is computed once and merged twice
         job_lists, dests, seen = [], [], {}
+        pieced = []  # states computed in pieces: [(o, l) of the first piece = destination, the others...]
         q_ranges, kv_ranges = ([], []) if segments is not None else (None, None)
         states = []
         for job in plan.jobs:
@@ -287,9 +311,21 @@ class proAttention:
                 continue
             o = torch.empty((B, Sq, H, D), dtype=torch.bfloat16, device=dev)
             l = torch.empty((B, H, Sq), dtype=torch.float32, device=dev)
+            if len(set(job.chunks)) > self._MAX_JOB_CHUNKS:
+                # a block of more chunks than one launch addresses (rings of 128 positions and more): its
+                # state is computed in pieces that are folded into (o, l) behind the attention launch
+                pieces = [job.chunks[i:i + self._MAX_JOB_CHUNKS] for i in range(0, len(job.chunks), self._MAX_JOB_CHUNKS)]
+                piece_states = [(o, l)] + [(torch.empty_like(o), torch.empty_like(l)) for _ in pieces[1:]]
+                pieced.append(piece_states)
+            else:
+                pieces, piece_states = [job.chunks], [(o, l)]
             if segments is None:
-                job_lists.append([index[c] for c in job.chunks])
-                dests.append((o, l))
+                for piece, st in zip(pieces, piece_states):
+                    job_lists.append([index[c] for c in piece])
+                    dests.append(st)
+            elif len(pieces) > 1:
+                raise NotImplementedError("variable-length calls with blocks of more than "
+                                          f"{self._MAX_JOB_CHUNKS} chunks are not supported")
             else:
                 # one kernel job per segment: its query rows against its key rows of every chunk
                 cu_q, cu_kv_of = segments
@@ -305,6 +341,9 @@ class proAttention:
             _hip.attn_jobs_fwd(query, table, job_lists, [d[0] for d in dests], [d[1] for d in dests],
                                q_ranges=q_ranges, kv_ranges=kv_ranges, workspace=_hip.attn_workspace(dev),
                                q_prescaled=self.q_prescaled)
+        for piece_states in pieced:
+            _hip.merge_states([s[0] for s in piece_states], [s[1] for s in piece_states],
+                              dst_out=piece_states[0][0], dst_lse=piece_states[0][1])
         for job, (o, l) in zip(plan.jobs, states):
             if job.store_slot is not None:
                 self.cache.store_block(job.store_slot, o, l)  # :207-211
@@ -322,7 +361,6 @@ class proAttention:
         diag = rm.mask_diag
         B, Sq, H, D = query.shape
         cache = self.cache
-        cache.ensure_arena(C, B, Sq, H, D, query.device)
         row = rm.chunk_mask[t, l]
         ks, vs = [], []
         for c in range(C):
@@ -330,11 +368,13 @@ class proAttention:
             k_c, v_c = (key, value) if use_local else self.group.kv_chunk(c)
             ks.append(_as4d(k_c, B))
             vs.append(_as4d(v_c, B))
+        if not cache.ensure_arena(C, B, Sq, H, D, query.device):
+            out = self._attn_uncached(query, ks, vs)
+            rm.record_out_redundancy(timestep=t, layer_id=l, curr_out=out)
+            return out
         for c in range(C):
             if c != diag and row[c] != 0 and not cache.arena_valid[c]:
                 raise RuntimeError(f"T{t}L{l}: mask asks to reuse chunk {c} but no state was ever stored for it")
-        n_comp = int(rm.sched_counts_host[t, l, 0])
-        table = _hip.ChunkTable(ks, vs)
         seg_q = seg_kv = None
         if self._segments is not None:
             # packed variable-length batch: every scheduled chunk runs once per segment
@@ -342,10 +382,23 @@ class proAttention:
             seg_q = [(cu_q[i], cu_q[i + 1] - cu_q[i]) for i in range(len(cu_q) - 1)]
             seg_kv = [[(cu_kv_of(c)[i], cu_kv_of(c)[i + 1] - cu_kv_of(c)[i]) for i in range(len(cu_q) - 1)]
                       for c in range(C)]
-        _hip.attn_sched_fwd(query, table, rm.sched_compute_ids[t, l], rm.sched_counts[t, l, 0:1], n_comp,
-                            cache.arena_out, cache.arena_lse, diag, cache.diag_out, cache.diag_lse,
-                            seg_q=seg_q, seg_kv=seg_kv, workspace=_hip.attn_workspace(query.device),
-                            q_prescaled=self.q_prescaled)
+        ws = _hip.attn_workspace(query.device)
+        if not rm.sched_windows:
+            n_comp = int(rm.sched_counts_host[t, l, 0])
+            _hip.attn_sched_fwd(query, _hip.ChunkTable(ks, vs), rm.sched_compute_ids[t, l], rm.sched_counts[t, l, 0:1],
+                                n_comp, cache.arena_out, cache.arena_lse, diag, cache.diag_out, cache.diag_lse,
+                                seg_q=seg_q, seg_kv=seg_kv, workspace=ws, q_prescaled=self.q_prescaled)
+        else:
+            # more chunks than one launch addresses: one launch per window of chunk ids (ordered on the
+            # stream, so they can share the workspace)
+            for w0, w1, d_w, comp_w, cnt_w, cnt_host_w in rm.sched_windows:
+                n_comp = int(cnt_host_w[t, l, 0])
+                if n_comp == 0 or all(k.shape[1] == 0 for k in ks[w0:w1]):
+                    continue
+                _hip.attn_sched_fwd(query, _hip.ChunkTable(ks[w0:w1], vs[w0:w1]), comp_w[t, l], cnt_w[t, l, 0:1],
+                                    n_comp, cache.arena_out[w0:w1], cache.arena_lse[w0:w1], d_w, cache.diag_out,
+                                    cache.diag_lse, seg_q=seg_q, seg_kv=None if seg_kv is None else seg_kv[w0:w1],
+                                    workspace=ws, q_prescaled=self.q_prescaled)
         outs, lses = [], []
         for c in range(C):
             if c == diag:
@@ -359,6 +412,32 @@ class proAttention:
         out, lse = _hip.merge_states(outs, lses, dst_dtype=self.out_dtype, dst_lse_bsh=True)
         self.last_lse = lse
         rm.record_out_redundancy(timestep=t, layer_id=l, curr_out=out)
+        return out
+
+    def _attn_uncached(self, query, ks, vs) -> torch.Tensor:
+        """A layer whose state arena did not fit: attention over all chunks, nothing kept."""
+        B, Sq, H, D = query.shape
+        dev = query.device
+        ids = [c for c in range(len(ks)) if ks[c].shape[1] > 0]
+        pieces = [ids[i:i + self._MAX_JOB_CHUNKS] for i in range(0, len(ids), self._MAX_JOB_CHUNKS)]
+        outs = [torch.empty((B, Sq, H, D), dtype=torch.bfloat16, device=dev) for _ in pieces]
+        lses = [torch.empty((B, H, Sq), dtype=torch.float32, device=dev) for _ in pieces]
+        q_ranges = kv_ranges = None
+        jobs, d_out, d_lse = pieces, outs, lses
+        if self._segments is not None:
+            cu_q, cu_kv_of = self._segments
+            jobs, d_out, d_lse, q_ranges, kv_ranges = [], [], [], [], []
+            for piece, o, l_ in zip(pieces, outs, lses):
+                for i in range(len(cu_q) - 1):
+                    jobs.append(piece)
+                    d_out.append(o)
+                    d_lse.append(l_)
+                    q_ranges.append((cu_q[i], cu_q[i + 1] - cu_q[i]))
+                    kv_ranges.append([(cu_kv_of(c)[i], cu_kv_of(c)[i + 1] - cu_kv_of(c)[i]) for c in piece])
+        _hip.attn_jobs_fwd(query, _hip.ChunkTable(ks, vs), jobs, d_out, d_lse, q_ranges=q_ranges, kv_ranges=kv_ranges,
+                           workspace=_hip.attn_workspace(dev), q_prescaled=self.q_prescaled)
+        out, lse = _hip.merge_states(outs, lses, dst_dtype=self.out_dtype, dst_lse_bsh=True)
+        self.last_lse = lse
         return out
 
     # ---- varlen entry (HunyuanVideo) ---------------------------------------------------------------

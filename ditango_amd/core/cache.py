@@ -45,6 +45,7 @@ class proCache:
         self.diag_out: Optional[torch.Tensor] = None
         self.diag_lse: Optional[torch.Tensor] = None
         self.arena_valid: List[bool] = []
+        self.arena_refused: Optional[tuple] = None  # arena shape the memory guard turned down
 
     # ---- memory guard (cache.py:89-128) -------------------------------------------------------
     @property
@@ -170,21 +171,45 @@ class proCache:
         return _hip.cache_load(o, l, dtype, dst_lse_bsh=True)
 
     def clear(self) -> None:
-        """cache.py:86-87 only logs; this one also drops the states."""
+        """cache.py:86-87: logs and keeps every state, as the reference does."""
         logger.warning("============== Clear oCache =================")
+
+    def release(self) -> None:
+        """Drop every cached state and the mask-mode arena (no counterpart in the reference, whose
+        ``clear`` keeps them): frees the HBM a finished generation holds."""
         self.out_block_cache = [None] * self.curr_block_num
         self.lse_block_cache = [None] * self.curr_block_num
-        self.arena_valid = [False] * len(self.arena_valid)
+        self.arena_out = self.arena_lse = self.diag_out = self.diag_lse = None
+        self.arena_valid = []
+        self.arena_refused = None
 
     # ---- mask-mode arena --------------------------------------------------------------------------
-    def ensure_arena(self, n_chunks: int, B: int, Sq: int, H: int, D: int, device) -> None:
+    def ensure_arena(self, n_chunks: int, B: int, Sq: int, H: int, D: int, device) -> bool:
+        """Make sure the mask-mode arena of this layer exists.  Returns False when it does not fit:
+        the arena (``n_chunks + 1`` states) is only allocated if the current allocation plus its size
+        stays under ``memory_constraint`` -- the same probe and budget as ``pass_memory_check``
+        (cache.py:103-128) -- and a layer without arena recomputes every chunk on every call, which is
+        what the reference's guard falls back to (core/attention.py:97-98: stride forced to N)."""
         shape = (n_chunks, B, Sq, H, D)
-        if self.arena_out is None or tuple(self.arena_out.shape) != shape or self.arena_out.device != device:
-            self.arena_out = torch.empty(shape, dtype=torch.bfloat16, device=device)
-            self.arena_lse = torch.empty((n_chunks, B, H, Sq), dtype=torch.float32, device=device)
-            self.diag_out = torch.empty((B, Sq, H, D), dtype=torch.bfloat16, device=device)
-            self.diag_lse = torch.empty((B, H, Sq), dtype=torch.float32, device=device)
-            self.arena_valid = [False] * n_chunks
+        if self.arena_out is not None and tuple(self.arena_out.shape) == shape and self.arena_out.device == device:
+            return True
+        if self.arena_refused == shape:
+            return False
+        self.arena_out = self.arena_lse = self.diag_out = self.diag_lse = None
+        need_mb = (n_chunks + 1) * B * Sq * H * (2 * D + 4) / (1024 ** 2)
+        now = self.memory_probe()
+        if now + need_mb > self.memory_constraint:
+            logger.warning(f"T{get_timestep()}L{self.layer_id} | Memory check failed: {now + need_mb:.0f} > "
+                           f"{self.memory_constraint:.0f} MB, this layer keeps no state arena and recomputes every chunk")
+            self.arena_refused = shape
+            self.arena_valid = []
+            return False
+        self.arena_out = torch.empty(shape, dtype=torch.bfloat16, device=device)
+        self.arena_lse = torch.empty((n_chunks, B, H, Sq), dtype=torch.float32, device=device)
+        self.diag_out = torch.empty((B, Sq, H, D), dtype=torch.bfloat16, device=device)
+        self.diag_lse = torch.empty((B, H, Sq), dtype=torch.float32, device=device)
+        self.arena_valid = [False] * n_chunks
+        return True
 
     def report_cache_status(self, layer_id: int) -> None:
         """cache.py:131-207, condensed."""

@@ -54,6 +54,7 @@ class RedundancyMap:
         self.sched_reuse_ids: Optional[torch.Tensor] = None
         self.sched_counts: Optional[torch.Tensor] = None  # int32 [T,L,2] device
         self.sched_counts_host: Optional[np.ndarray] = None
+        self.sched_windows: list = []  # (first chunk, end, diag in window, compute ids, counts, counts on host)
 
     # ---- divider map / strides ---------------------------------------------------------------
     def _init_map(self) -> torch.Tensor:
@@ -275,11 +276,22 @@ class RedundancyMap:
         comp, reu, cnt = _hip.build_schedule_table(dmask, self.mask_diag)
         self.sched_compute_ids, self.sched_reuse_ids, self.sched_counts = comp, reu, cnt
         self.sched_counts_host = cnt.cpu().numpy()  # one read-back at install time, none per call
+        # One attention launch addresses at most DT_MAX_CHUNKS chunks: more chunks run as one launch per
+        # window of chunk ids, each with its own compute list (ids relative to the window's first chunk).
+        self.sched_windows = []
+        C = m.shape[2]
+        if C > _hip.DT_MAX_CHUNKS:
+            for w0 in range(0, C, _hip.DT_MAX_CHUNKS):
+                w1 = min(C, w0 + _hip.DT_MAX_CHUNKS)
+                d_w = self.mask_diag - w0 if w0 <= self.mask_diag < w1 else -1
+                c_w, _, n_w = _hip.build_schedule_table(dmask[:, :, w0:w1].contiguous(), d_w)
+                self.sched_windows.append((w0, w1, d_w, c_w, n_w, n_w.cpu().numpy()))
 
     def clear_chunk_mask(self) -> None:
         self.chunk_mask = None
         self.sched_compute_ids = self.sched_reuse_ids = self.sched_counts = None
         self.sched_counts_host = None
+        self.sched_windows = []
 
 
 def make_bernoulli_mask(num_timesteps: int, num_layers: int, num_chunks: int, reuse_prob: float, seed: int,

@@ -28,6 +28,10 @@ def disable_timing() -> None:
     _ENABLED = False
 
 
+def is_timing_enabled() -> bool:
+    return _ENABLED
+
+
 class _Timer(ContextDecorator):
     def __init__(self, name: str):
         self.name = name

@@ -47,6 +47,15 @@ def update_out_and_lse(out: Optional[torch.Tensor], lse: Optional[torch.Tensor],
     return _hip.merge_states([out.contiguous(), block_out], [lse, block_lse], dst_dtype=torch.float32, dst_lse_bsh=True)
 
 
+def _update_out_and_lse(out: torch.Tensor, lse: torch.Tensor, block_out: torch.Tensor, block_lse: torch.Tensor
+                        ) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Drop-in for utils.py:24-40: the two-state merge on an existing running state (fp32 ``out``
+    ``[B,S,H,D]``, fp32 ``lse [B,S,H,1]``; ``block_lse`` in flash-attn's ``[B,H,S]``).  One
+    ``dt_merge_states`` launch with n = 2."""
+    return _hip.merge_states([out.contiguous(), block_out.contiguous()], [lse, block_lse], dst_dtype=torch.float32,
+                             dst_lse_bsh=True)
+
+
 def rel_l1(new, ori) -> float:
     """Drop-in for utils.py:202-267.  Tensor inputs are reduced on the GPU in one
     kernel and read back once (the reference syncs three times)."""

@@ -54,7 +54,7 @@ extern "C" {
 #define DT_MAX_CHUNKS 40       /* KV chunks one launch can address */
 #define DT_MAX_JOBS 40         /* attention states one launch can produce */
 #define DT_MAX_JOB_ENTRIES 64  /* total chunk references over all jobs of a launch */
-#define DT_MAX_MERGE 40        /* states one merge launch can combine */
+#define DT_MAX_MERGE 64        /* states one merge launch can combine */
 #define DT_MAX_SEGMENTS 8      /* segments of a packed batch in one device-scheduled launch */
 
 int dt_version(void);

@@ -64,6 +64,9 @@ def _cmp(out, lse_bsh1, ref_out, ref_lse_bhs, what):
     (4, 1, 128, (1, 1, 1, 2, 2, 2, 1, 4, 2, 2, 1, 1)),     # includes the stride-1 -> 2 misalignment
     (8, 3, 64, (1, 1, 1, 4, 4, 4, 2, 2, 2, 2, 1, 1)),
     (8, 0, 128, (1, 1, 1, 8, 8, 4, 4, 2, 1, 8, 1, 1)),
+    # a ring of 64 positions (strides 64 / 32 / 16 / 8, two-level ring above 8): a full-stride step that
+    # announces stride 8 files 64 fine-grained states, more than one merge launch or chunk table holds
+    (64, 37, 64, (1, 1, 1, 8, 8, 4, 4, 2, 1, 8, 1, 1)),
 ])
 def test_stride_mode_matches_numeric_oracle(env, N, rank, D, col):
     from ditango_amd.core.attention import proAttention
@@ -121,6 +124,8 @@ def test_stride_mode_matches_numeric_oracle(env, N, rank, D, col):
     (8, 0, 128, 0.5, None),
     (8, 5, 64, 0.6, None),
     (6, -1, 128, 0.75, [70, 69, 69, 70, 1, 64]),     # ragged chunks, no local chunk
+    (48, 5, 128, 0.5, None),                         # more chunks than one launch addresses: two windows
+    (70, 43, 64, 0.6, None),                         # local chunk in the second window; 70-way merge
 ])
 def test_mask_mode_matches_numeric_oracle(env, C, diag, D, p, lens):
     from ditango_amd.core.attention import proAttention
@@ -211,6 +216,82 @@ def test_config1_cpu_plumbing_case(env):
     # stale-but-close: the cached result stays near exact attention on the step-t inputs
     exact, _ = om.full_attention(q1.bfloat16(), [k.bfloat16() for k in k1], [v.bfloat16() for v in v1])
     assert (out.cpu() - exact).abs().max() < 5e-2
+
+
+def test_config1_fp32_inputs_as_stated(env):
+    """BASELINE configuration 1 with the fp32 tensors handed over as they are: the driver rounds them
+    to bf16 at the kernel boundary (flash_attn_func itself takes no fp32).  Two comparisons: the strict
+    bar against the oracle on the rounded inputs (same numbers as test_config1_cpu_plumbing_case), and
+    the distance to fp32 attention of the UNROUNDED inputs, which is the price of the bf16 inputs:
+    observed 4e-3 in out and 6e-3 in lse for N(0,1) inputs at D = 64; the test allows 2e-2 / 2e-2."""
+    from ditango_amd.core.attention import proAttention
+    from ditango_amd.core.parallel_state import get_usp_group
+    from ditango_amd.utils import update_timestep
+    B, H, D, Sq, C = 1, 4, 64, 512, 4
+    rm = env(C, 0, 2, 1)
+    mask = np.zeros((2, 1, C), dtype=np.uint8)
+    mask[1, 0, [1, 3]] = 1
+    rm.set_chunk_mask(mask, diag=0)
+    g0 = torch.Generator().manual_seed(0)
+    q1 = torch.randn(B, Sq, H, D, generator=g0)
+    k1 = [torch.randn(B, 512, H, D, generator=g0) for _ in range(C)]
+    v1 = [torch.randn(B, 512, H, D, generator=g0) for _ in range(C)]
+    g1 = torch.Generator().manual_seed(1)
+    q0, k0, v0 = _perturb(q1, g1), [_perturb(k, g1) for k in k1], [_perturb(v, g1) for v in v1]
+    group = get_usp_group()
+    attn = proAttention(0, group)
+    merge = lambda sts: om.merge_states_closed_form([s[0] for s in sts], [s[1] for s in sts])
+    orc_rounded, orc_fp32 = ms.MaskCacheOracle(C, 0), ms.MaskCacheOracle(C, 0)
+    for t, (q, ks, vs) in enumerate([(q0, k0, v0), (q1, k1, v1)]):
+        qb, kb, vb = q.bfloat16(), [k.bfloat16() for k in ks], [v.bfloat16() for v in vs]
+        (ref_out, ref_lse), _, _ = orc_rounded.call(mask[t, 0], lambda c: om.chunk_attention(qb, kb[c], vb[c]), merge,
+                                                    lambda s: (om.bf16_round(s[0]), s[1]))
+        (f_out, f_lse), _, _ = orc_fp32.call(mask[t, 0], lambda c: om.chunk_attention(q, ks[c], vs[c]), merge)
+        update_timestep(t)
+        dk, dv = [k.cuda() for k in ks], [v.cuda() for v in vs]          # fp32 on the device
+        group.set_kv_chunks(dk, dv)
+        out = attn.attn(q.cuda(), dk[0], dv[0])
+        torch.cuda.synchronize()
+        assert out.dtype == torch.float32
+        _cmp(out, attn.last_lse, ref_out, ref_lse, f"config1 fp32 inputs t={t}, oracle on rounded inputs")
+        err = (out.cpu() - f_out).abs().max().item()
+        lerr = (attn.last_lse.cpu().squeeze(-1).transpose(1, 2) - f_lse).abs().max().item()
+        print(f"config1 fp32 inputs t={t}: distance to fp32 attention of the unrounded inputs: out {err:.3e} lse {lerr:.3e}",
+              flush=True)
+        assert err <= 2e-2 and lerr <= 2e-2
+    with pytest.raises(TypeError):
+        attn.attn(q1.double().cuda(), dk[0], dv[0])
+
+
+def test_mask_mode_memory_guard_recomputes_without_arena(env):
+    """A layer whose state arena does not fit under the memory budget keeps no states and computes
+    every chunk on every call (what the reference's guard falls back to, core/attention.py:97-98):
+    the result is full attention whatever the mask says, and no arena is allocated."""
+    from ditango_amd.core.attention import proAttention
+    from ditango_amd.core.parallel_state import get_usp_group
+    from ditango_amd.utils import update_timestep
+    B, H, D, Sq, C, T = 1, 2, 128, 80, 5, 3
+    rm = env(C, 0, T, 2)
+    mask = ms.seeded_mask(T, 2, C, 0.6, seed=3, diag=0)
+    rm.set_chunk_mask(mask, diag=0)
+    q, ks, vs = _inputs(B, Sq, [Sq, 70, 1, 64, 90], H, D, seed=9)
+    group = get_usp_group()
+    tight, roomy = proAttention(0, group), proAttention(1, group)
+    tight.cache.memory_probe = lambda: 1000.0
+    tight.cache.memory_constraint = 1000.2          # the arena (6 states of 80 KB) would not fit
+    g = torch.Generator().manual_seed(2)
+    for t in range(T):
+        update_timestep(t)
+        qb, kb, vb = q.bfloat16(), [k.bfloat16() for k in ks], [v.bfloat16() for v in vs]
+        dk, dv = [k.cuda() for k in kb], [v.cuda() for v in vb]
+        group.set_kv_chunks(dk, dv)
+        out = tight.attn(qb.cuda(), dk[0], dv[0])
+        roomy.attn(qb.cuda(), dk[0], dv[0])
+        torch.cuda.synchronize()
+        ref_out, ref_lse = om.full_attention(qb, kb, vb)
+        _cmp(out, tight.last_lse, ref_out, ref_lse, f"no arena t={t}")
+        q, ks, vs = _perturb(q, g), [_perturb(k, g) for k in ks], [_perturb(v, g) for v in vs]
+    assert tight.cache.arena_out is None and roomy.cache.arena_out is not None
 
 
 def test_update_out_and_lse_dropin(hip):

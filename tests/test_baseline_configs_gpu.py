@@ -176,6 +176,79 @@ def test_reuse_sweep_shape_properties(env, hip):
         assert err <= OUT_TOL and lerr <= LSE_TOL
 
 
+@pytest.mark.parametrize("frac", [0.5, 0.9])
+def test_reuse_sweep_at_full_size(env, hip, frac):
+    """Configuration 5 as it stands: Q and KV are the full 119 056 tokens, KV in 32 chunks of 3721 / 3720
+    keys (the reference's uneven split, utils.py:99-111, without zero padding), H = 24, D = 128, no local
+    chunk.  Step 0 fills the 32-slot arena (23.8 GB), step 1 runs under the committed seeded mask of
+    the given reuse fraction on inputs that drifted by 1 %; the oracle follows on a seeded sample of
+    32 query rows (all heads, all keys), the schedule lists are compared with the committed vectors."""
+    import os
+    from ditango_amd.core.attention import proAttention
+    from ditango_amd.core.parallel_state import get_usp_group
+    from ditango_amd.utils import update_timestep
+    B, H, D, S = 1, 24, 128, 119056
+    lens = [3721] * 16 + [3720] * 16
+    C, T, L = 32, 2, 60
+    assert sum(lens) == S
+    free, _ = torch.cuda.mem_get_info()
+    if free < 40 * 2 ** 30:
+        pytest.skip(f"needs about 32 GB of device memory, {free / 2 ** 30:.0f} GiB are free")
+    print(f"case sweep full size: reuse {frac}, Sq={S}, C={C}", flush=True)
+    gold = np.load(os.path.join(os.path.dirname(__file__), "golden", "mask_schedules.npz"))
+    mask = gold[f"sweep_{frac}/mask"]
+    rm = env(C, 0, T, L)
+    rm.set_chunk_mask(mask, diag=-1)
+    assert np.array_equal(rm.sched_compute_ids.cpu().numpy(), gold[f"sweep_{frac}/compute_ids"].astype(np.int32))
+    assert np.array_equal(rm.sched_reuse_ids.cpu().numpy(), gold[f"sweep_{frac}/reuse_ids"].astype(np.int32))
+    assert np.array_equal(rm.sched_counts.cpu().numpy(), gold[f"sweep_{frac}/counts"].astype(np.int32))
+    layer = int(np.argmin(np.abs(mask[1].mean(axis=1) - frac)))    # the layer whose realised ratio is closest
+    print(f"layer {layer}: {int(mask[1, layer].sum())}/32 chunks reused at step 1", flush=True)
+
+    # inputs are drawn on the GPU (1.1 G normal numbers per step) and copied to the host for the oracle
+    g = torch.Generator(device="cuda").manual_seed(5)
+    cg = torch.Generator().manual_seed(6)
+    rows = torch.sort(torch.randperm(S, generator=cg)[:32]).values
+    drows = rows.cuda()
+
+    def draw(norm):
+        x = torch.randn(B, S, H, D, generator=g, device="cuda")
+        if norm:
+            x = x / x.pow(2).mean(-1, keepdim=True).sqrt()
+        return x
+
+    xs = [draw(True), draw(True), draw(False)]               # fp32 masters of q, k, v
+    group = get_usp_group()
+    attn = proAttention(layer, group)
+    cached = {}
+    for t in range(2):
+        update_timestep(t)
+        dq, dk, dv = (x.bfloat16() for x in xs)
+        dks, dvs = list(torch.split(dk, lens, dim=1)), list(torch.split(dv, lens, dim=1))
+        group.set_kv_chunks(dks, dvs)
+        out = attn.attn(dq, None, None)
+        torch.cuda.synchronize()
+        hk, hv = dk.cpu(), dv.cpu()
+        hq = torch.zeros(B, int(rows.max()) + 1, H, D, dtype=torch.bfloat16)
+        hq[:, rows] = dq[:, drows].cpu()
+        ref_out, ref_lse, cached, compute, reuse = _oracle_rows(
+            hq, list(torch.split(hk, lens, dim=1)), list(torch.split(hv, lens, dim=1)), rows, mask[t, layer], -1, cached)
+        got_out = out[:, drows].cpu()
+        got_lse = attn.last_lse[:, drows].cpu().squeeze(-1).transpose(1, 2)
+        assert torch.isfinite(out).all()
+        err = (got_out - ref_out).abs().max().item()
+        lerr = (got_lse - ref_lse).abs().max().item()
+        rel = (got_out - ref_out).norm().item() / ref_out.norm().item()
+        print(f"sweep {frac} t={t} computed {len(compute)} reused {len(reuse)}: out max-abs {err:.3e} rel-l2 {rel:.3e} "
+              f"lse {lerr:.3e}", flush=True)
+        assert err <= OUT_TOL and lerr <= LSE_TOL and rel <= 1e-2
+        del out, dq, dk, dv, dks, dvs, hk, hv
+        for x in xs:                                          # 1 % drift: reused states are stale but close
+            x.add_(torch.randn(x.shape, generator=g, device="cuda"), alpha=0.01)
+    del attn, xs
+    group.set_kv_chunks([None] * C, [None] * C)
+
+
 def test_size_independent_properties_at_hunyuan_shape(hip):
     """(a) one job over 3 chunks == merge of the 3 single-chunk states; (b) a state written to the
     cache and loaded back is bit-identical; at the full per-rank shape."""

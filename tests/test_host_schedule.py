@@ -112,3 +112,24 @@ def test_memory_guard_falls_back_to_full_refresh(ditango_env):
     assert c.pass_memory_check(1, 0) is False          # 8 blocks * 100 MB + 500 > 1000
     c.out_block_cache = [object()] * 8                 # already holding as many blocks as predicted
     assert c.pass_memory_check(1, 0) is True
+
+
+def test_mask_mode_arena_consults_the_memory_guard(ditango_env):
+    """ensure_arena uses the probe and budget of pass_memory_check (core/cache.py:103-128): an arena
+    that would push the allocation over the budget is refused (once, with a warning), a fitting one is
+    allocated; release() forgets the refusal."""
+    from ditango_amd.core.cache import proCache
+    c = proCache(8, 0)
+    need_mb = 9 * 1 * 64 * 2 * (2 * 64 + 4) / 2 ** 20          # 8 chunks + the local state
+    c.memory_constraint = 100.0
+    c.memory_probe = lambda: 100.0 - need_mb / 2
+    assert c.ensure_arena(8, 1, 64, 2, 64, torch.device("cpu")) is False
+    assert c.arena_out is None and c.arena_refused == (8, 1, 64, 2, 64)
+    c.memory_probe = lambda: 0.0
+    assert c.ensure_arena(8, 1, 64, 2, 64, torch.device("cpu")) is False       # a refusal sticks for that shape
+    c.release()
+    assert c.ensure_arena(8, 1, 64, 2, 64, torch.device("cpu")) is True
+    assert tuple(c.arena_out.shape) == (8, 1, 64, 2, 64) and tuple(c.arena_lse.shape) == (8, 1, 2, 64)
+    assert c.arena_valid == [False] * 8
+    c.clear()                                                                   # the reference's clear() keeps the states
+    assert c.arena_out is not None

@@ -1,5 +1,5 @@
-"""The per-launch limits of the C ABI (40 chunks, 40 states, 64 chunk references, 40-way merge),
-the splitting of larger requests on the host side, tile counts around the pairing of iterations,
+"""The per-launch limits of the C ABI (40 chunks, 40 states, 64 chunk references, 64-way merge),
+the splitting of larger requests on the host side (launch groups, chunk windows, merge rounds), tile counts around the pairing of iterations,
 and the error behaviour at the boundary (return code + message, never a launch)."""
 import ctypes
 
@@ -37,8 +37,38 @@ def test_forty_chunks_in_one_job(hip):
     hip.attn_jobs_fwd(q.cuda(), table, [list(range(C))], [out], [lse])
     torch.cuda.synchronize()
     _check(out, lse, ref_out, ref_lse, "40 chunks, one job")
+    # the C ABI itself turns a 41st chunk down ...
+    big = hip.ChunkTable([k.cuda() for k in ks] + [ks[0].cuda()], [v.cuda() for v in vs] + [vs[0].cuda()])
     with pytest.raises(hip.DitangoHipError):
-        hip.ChunkTable([k.cuda() for k in ks] + [ks[0].cuda()], [v.cuda() for v in vs] + [vs[0].cuda()])
+        big.whole()
+    # ... and so does a single job over 41 distinct chunks (the caller splits such a job and merges)
+    with pytest.raises(hip.DitangoHipError):
+        hip.attn_jobs_fwd(q.cuda(), big, [list(range(C + 1))], [out], [lse])
+
+
+def test_table_of_more_chunks_than_a_launch_addresses(hip):
+    """70 chunks, 70 single-chunk jobs and two jobs of 35 chunks each: the binding groups jobs into
+    launches whose sub-table holds at most 40 distinct chunks."""
+    B, Sq, H, D, C = 1, 40, 2, 64, 70
+    g = torch.Generator().manual_seed(8)
+    lens = [5 + (11 * i) % 40 for i in range(C)]
+    q = _rand((B, Sq, H, D), g)
+    ks = [_rand((B, n, H, D), g) for n in lens]
+    vs = [_rand((B, n, H, D), g) for n in lens]
+    table = hip.ChunkTable([k.cuda() for k in ks], [v.cuda() for v in vs])
+    jobs = [[c] for c in range(C)] + [list(range(0, C, 2)), list(range(1, C, 2))]
+    outs = [torch.empty(B, Sq, H, D, dtype=torch.bfloat16, device="cuda") for _ in jobs]
+    lses = [torch.empty(B, H, Sq, dtype=torch.float32, device="cuda") for _ in jobs]
+    hip.attn_jobs_fwd(q.cuda(), table, jobs, outs, lses)
+    torch.cuda.synchronize()
+    for j, chunks in enumerate(jobs):
+        ref = om.full_attention(q, [ks[c] for c in chunks], [vs[c] for c in chunks])
+        _check(outs[j], lses[j], *ref, f"job {j}")
+    # everything merged = attention over all 70 chunks (a 70-way merge: more than one merge launch holds)
+    o, l = hip.merge_states(outs[:C], lses[:C])
+    torch.cuda.synchronize()
+    ref_out, ref_lse = om.full_attention(q, ks, vs)
+    _check(o, l, ref_out, ref_lse, "70-way merge of the chunk states")
 
 
 def test_more_jobs_than_one_launch_holds(hip):
@@ -67,18 +97,35 @@ def test_more_jobs_than_one_launch_holds(hip):
         _check(outs[j], lses[j], *full, f"full job {j}")
 
 
-def test_forty_way_merge_and_its_limit(hip):
-    B, Sq, H, D, n = 1, 50, 2, 128, hip.DT_MAX_MERGE
-    g = torch.Generator().manual_seed(3)
+@pytest.mark.parametrize("n", [64, 65, 100, 127, 200])
+@pytest.mark.parametrize("D,dst_dtype", [(128, torch.float32), (64, torch.bfloat16)])
+def test_many_way_merge_in_rounds(hip, n, D, dst_dtype):
+    """One launch folds up to 64 states; more go through a running fp32 state in rounds of 63.  Against
+    the closed form, with -inf states, a repeated pointer and mixed dtypes / lse layouts among them."""
+    assert hip.DT_MAX_MERGE == 64
+    B, Sq, H = 1, 50, 3
+    g = torch.Generator().manual_seed(3 + n)
     outs = [_rand((B, Sq, H, D), g) for _ in range(n)]
     lses = [torch.randn(B, H, Sq, generator=g) * 3 for _ in range(n)]
     lses[7].fill_(float("-inf"))
+    lses[n - 2].fill_(float("-inf"))
+    outs[n - 1], lses[n - 1] = outs[3], lses[3]                      # the same state twice
+    d_outs = [x.cuda() for x in outs]
+    d_lses = [x.cuda() for x in lses]
+    d_outs[n // 2] = d_outs[n // 2].float()                          # one fp32 state ...
+    d_lses[n // 3] = d_lses[n // 3].transpose(1, 2).contiguous().unsqueeze(-1)   # ... one lse stored [B,S,H,1]
     ref_out, ref_lse = om.merge_states_closed_form([o.float() for o in outs], lses)
-    o, l = hip.merge_states([x.cuda() for x in outs], [x.cuda() for x in lses])
+    o, l = hip.merge_states(d_outs, d_lses, dst_dtype=dst_dtype)
     torch.cuda.synchronize()
-    assert (o.cpu() - ref_out).abs().max() <= 1e-5 and (l.cpu() - ref_lse).abs().max() <= 1e-5
-    with pytest.raises(hip.DitangoHipError):
-        hip.merge_states([x.cuda() for x in outs] + [outs[0].cuda()], [x.cuda() for x in lses] + [lses[0].cuda()])
+    tol = 1e-5 if dst_dtype == torch.float32 else 2.0 ** -8 * float(ref_out.abs().max())
+    assert o.dtype == dst_dtype
+    assert (o.float().cpu() - ref_out).abs().max() <= tol and (l.cpu() - ref_lse).abs().max() <= 1e-5
+    # in place over the first input (cache coarsening writes over its first member)
+    first_o, first_l = d_outs[0].clone(), d_lses[0].clone()
+    hip.merge_states([first_o] + d_outs[1:], [first_l] + d_lses[1:], dst_out=first_o, dst_lse=first_l)
+    torch.cuda.synchronize()
+    assert (first_o.float().cpu() - ref_out).abs().max() <= 2.0 ** -8 * float(ref_out.abs().max())
+    assert (first_l.cpu() - ref_lse).abs().max() <= 1e-5
 
 
 @pytest.mark.parametrize("Sk", [63, 64, 65, 127, 128, 129, 191, 193, 256, 257, 320, 449, 512, 513, 577])
