@@ -26,6 +26,7 @@ DT_MAX_JOBS = 40
 DT_MAX_JOB_ENTRIES = 64
 DT_MAX_MERGE = 64
 DT_MAX_SEGMENTS = 8
+DT_NOALLOC_TAIL_SLOTS = 512
 
 c_i32, c_i64, c_f32, c_vp = ctypes.c_int32, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
 _P = ctypes.POINTER
@@ -47,6 +48,10 @@ _SIGNATURES = {
                                                c_i32, _P(c_vp), _P(c_vp), _P(c_i32), _P(c_i64), c_i64, c_i64,
                                                c_i32, _P(c_i32), _P(c_i32), _P(c_i32), _P(c_i32), _P(c_i32), _P(c_i32),
                                                _P(c_vp), _P(c_vp), c_f32, c_i32, c_vp, c_i64, c_vp]),
+    "dt_attn_seg_jobs_noalloc_fwd": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i64, c_i64, c_i64,
+                                                    c_i32, _P(c_vp), _P(c_vp), _P(c_i32), _P(c_i64), c_i64, c_i64,
+                                                    c_i32, _P(c_i32), _P(c_i32), _P(c_i32), _P(c_i32), _P(c_i32), _P(c_i32),
+                                                    _P(c_vp), _P(c_vp), c_f32, c_i32, c_vp]),
     "dt_attn_sched_seg_ws_fwd": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i64, c_i64, c_i64,
                                                 c_i32, _P(c_vp), _P(c_vp), _P(c_i32), _P(c_i64), c_i64, c_i64,
                                                 c_vp, c_vp, c_i32, c_vp, c_i64, c_vp, c_i64, c_i32, c_vp, c_vp,
@@ -255,7 +260,8 @@ def attn_jobs_fwd(q: torch.Tensor, table: ChunkTable, jobs: Sequence[Sequence[in
                   outs: Sequence[torch.Tensor], lses: Sequence[torch.Tensor], softmax_scale: float = 0.0,
                   q_ranges: Optional[Sequence[Tuple[int, int]]] = None,
                   kv_ranges: Optional[Sequence[Sequence[Tuple[int, int]]]] = None,
-                  workspace: Optional[torch.Tensor] = None, q_prescaled: bool = False) -> None:
+                  workspace: Optional[torch.Tensor] = None, q_prescaled: bool = False,
+                  no_alloc: bool = False) -> None:
     """One launch; job j attends q to the concatenation of chunks ``jobs[j]`` and writes (outs[j], lses[j]).
 
     ``q_ranges[j] = (begin, length)`` restricts job j to those query rows (the rest of its
@@ -265,11 +271,14 @@ def attn_jobs_fwd(q: torch.Tensor, table: ChunkTable, jobs: Sequence[Sequence[in
     of one launch.  With a ``workspace`` (``attn_workspace(device)``) the last, partly filled round of
     workgroups of a launch is split along the keys and folded back (tail balancing).
     ``q_prescaled``: q already carries ``softmax_scale * log2(e)`` (folded in before its rounding to
-    bf16); ``softmax_scale`` is then ignored and the softmax is that of ``q k^T * ln 2``."""
+    bf16); ``softmax_scale`` is then ignored and the softmax is that of ``q k^T * ln 2``.
+    ``no_alloc``: go through ``dt_attn_seg_jobs_noalloc_fwd``, which splits the tail inside the library's
+    own device array instead of a workspace (for callers that cannot allocate)."""
     lib = load_library()
     _check_qkv(q, "q")
     B, Sq, H, D = q.shape
     _require((B, H, D) == (table.B, table.H, table.D), "q and KV chunks disagree on B/H/D")
+    _require(not (no_alloc and workspace is not None), "no_alloc launches take no workspace")
     nj = len(jobs)
     _require(nj == len(outs) == len(lses), "one destination per job")
     _require(q_ranges is None or len(q_ranges) == nj, "one query range per job")
@@ -325,7 +334,14 @@ def attn_jobs_fwd(q: torch.Tensor, table: ChunkTable, jobs: Sequence[Sequence[in
         a_ql = (c_i32 * n)(*[int(q_ranges[start + jj][1]) for jj in range(n)]) if q_ranges is not None else None
         out_ptrs = (c_vp * n)(*[outs[start + jj].data_ptr() for jj in range(n)])
         lse_ptrs = (c_vp * n)(*[lses[start + jj].data_ptr() for jj in range(n)])
-        if True:
+        if no_alloc:
+            rc = lib.dt_attn_seg_jobs_noalloc_fwd(q.data_ptr(), B, Sq, H, D, q.stride(0), q.stride(1), q.stride(2),
+                                                  t_n, t_k, t_v, t_len, t_sb, table.ss, table.sh,
+                                                  n, begin, chunks, a_kvb, a_kvl, a_qb, a_ql, out_ptrs,
+                                                  lse_ptrs, float(softmax_scale),
+                                                  DT_ATTN_Q_PRESCALED if q_prescaled else 0, _stream())
+            _check(rc, "dt_attn_seg_jobs_noalloc_fwd")
+        else:
             rc = lib.dt_attn_seg_jobs_ws_fwd(q.data_ptr(), B, Sq, H, D, q.stride(0), q.stride(1), q.stride(2),
                                              t_n, t_k, t_v, t_len, t_sb, table.ss, table.sh,
                                              n, begin, chunks, a_kvb, a_kvl, a_qb, a_ql, out_ptrs, lse_ptrs,

@@ -47,6 +47,7 @@
 //     through a contiguous range of heads: the workgroups that share an XCD's
 //     L2 stream the same K/V.
 #include <algorithm>
+#include <mutex>
 #include <type_traits>
 
 #include "dt_common.h"
@@ -891,6 +892,38 @@ static int cu_count() {
   return cached;
 }
 
+// Scratch of the allocation-free entry point: the tail-balancing workspace as a device array that
+// lives as long as the code object (one copy per GPU, at that GPU's own address).  Host code never
+// uses the array's name as an address: static_tail_scratch() asks the runtime for the device
+// address once per device and hands that out.
+static __device__ __align__(256) uint8_t g_tail_scratch[kStaticTailBytes];
+
+int static_tail_scratch(void** ptr, int64_t* bytes) {
+  constexpr int kMaxDevices = 64;
+  static std::mutex mu;
+  static void* addr[kMaxDevices] = {};
+  int dev = 0;
+  if (int rc = hip_fail(hipGetDevice(&dev), "hipGetDevice")) return rc;
+  if (dev < 0 || dev >= kMaxDevices) {
+    set_error("device ordinal %d outside the %d the static scratch table covers", dev, kMaxDevices);
+    return DT_ERR_UNSUPPORTED;
+  }
+  std::lock_guard<std::mutex> lock(mu);
+  if (addr[dev] == nullptr) {
+    void* p = nullptr;
+    if (int rc = hip_fail(hipGetSymbolAddress(&p, HIP_SYMBOL(g_tail_scratch)), "hipGetSymbolAddress(tail scratch)"))
+      return rc;
+    if (p == nullptr || (reinterpret_cast<uintptr_t>(p) & 255) != 0) {
+      set_error("the runtime returned an unusable address for the static tail scratch");
+      return DT_ERR_HIP;
+    }
+    addr[dev] = p;
+  }
+  *ptr = addr[dev];
+  *bytes = kStaticTailBytes;
+  return DT_OK;
+}
+
 int launch_attn(const AttnArgs& a_in, int D, int n_jobs, hipStream_t stream, void* workspace,
                 int64_t workspace_bytes, bool balance) {
   if (n_jobs <= 0 || a_in.total <= 0) return DT_OK;
@@ -943,6 +976,11 @@ int launch_attn(const AttnArgs& a_in, int D, int n_jobs, hipStream_t stream, voi
     }
   }
   if (tail == 0) return launch_dim(a, D, dim3((unsigned)slots_per_job, (unsigned)n_jobs, 1), stream);
+  if ((int64_t)tail * ways * slot_bytes > workspace_bytes) {
+    set_error("tail split of %d items x %d parts needs %lld bytes of scratch, %lld are there", tail, ways,
+              (long long)((int64_t)tail * ways * slot_bytes), (long long)workspace_bytes);
+    return DT_ERR_INVALID;
+  }
   a.tail_job = n_jobs - 1;
   a.tail_idx0 = a.per_xcd - tail / kXcds;
   a.tail_items = tail / kXcds;

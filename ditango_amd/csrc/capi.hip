@@ -193,6 +193,24 @@ extern "C" int dt_attn_seg_jobs_ws_fwd(const void* q, int32_t B, int32_t Sq, int
   return launch_attn(a, D, n_jobs, (hipStream_t)stream, workspace, workspace_bytes, job_q_begin == nullptr);
 }
 
+// The same launch for callers that cannot allocate: the tail is split inside the library's own
+// device array instead of a caller's workspace.
+extern "C" int dt_attn_seg_jobs_noalloc_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D, int64_t q_sb,
+                                            int64_t q_ss, int64_t q_sh, int32_t n_chunks, const void* const* k_ptrs,
+                                            const void* const* v_ptrs, const int32_t* kv_lens, const int64_t* kv_sb,
+                                            int64_t kv_ss, int64_t kv_sh, int32_t n_jobs, const int32_t* job_begin,
+                                            const int32_t* job_chunks, const int32_t* entry_kv_begin,
+                                            const int32_t* entry_kv_len, const int32_t* job_q_begin,
+                                            const int32_t* job_q_len, void* const* out_ptrs, float* const* lse_ptrs,
+                                            float softmax_scale, int32_t flags, void* stream) {
+  void* scratch = nullptr;
+  int64_t scratch_bytes = 0;
+  if (int rc = static_tail_scratch(&scratch, &scratch_bytes)) return rc;
+  return dt_attn_seg_jobs_ws_fwd(q, B, Sq, H, D, q_sb, q_ss, q_sh, n_chunks, k_ptrs, v_ptrs, kv_lens, kv_sb, kv_ss, kv_sh,
+                                 n_jobs, job_begin, job_chunks, entry_kv_begin, entry_kv_len, job_q_begin, job_q_len,
+                                 out_ptrs, lse_ptrs, softmax_scale, flags, scratch, scratch_bytes, stream);
+}
+
 extern "C" int dt_attn_seg_jobs_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D, int64_t q_sb,
                                     int64_t q_ss, int64_t q_sh, int32_t n_chunks, const void* const* k_ptrs,
                                     const void* const* v_ptrs, const int32_t* kv_lens, const int64_t* kv_sb,

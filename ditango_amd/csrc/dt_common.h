@@ -73,6 +73,13 @@ struct AttnArgs {
 // Workspace bytes the tail balancing can use at most (what dt_attn_workspace_bytes reports).
 constexpr int64_t kMaxTailSlots = 1536;
 
+// The allocation-free entry point splits tails inside a device array of this many partial-state
+// slots (sized for D = 128: 256 queries x 128 bf16 + 256 lse values each).
+constexpr int64_t kStaticTailSlots = DT_NOALLOC_TAIL_SLOTS;
+constexpr int64_t kStaticTailBytes = kStaticTailSlots * (256 * 128 * 2 + 256 * 4);
+// Device address and size of that array on the current device (looked up once per device).
+int static_tail_scratch(void** ptr, int64_t* bytes);
+
 int launch_attn(const AttnArgs& a, int D, int n_jobs, hipStream_t stream, void* workspace = nullptr,
                 int64_t workspace_bytes = 0, bool balance = false);
 

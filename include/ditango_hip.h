@@ -203,6 +203,33 @@ int dt_attn_sched_seg_ws_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, in
                              void* stream);
 
 /*
+ * dt_attn_seg_jobs_ws_fwd for callers that cannot allocate device memory (code under HIP graph
+ * capture, serving loops, harnesses that forbid hipMalloc): no workspace argument, the tail of the
+ * launch is split inside a device array that is part of the library (DT_NOALLOC_TAIL_SLOTS partial
+ * states of 256 queries x 128 bf16 + 256 lse values = 34 078 720 bytes, held by every GPU the
+ * library runs on until the process ends).  No counterpart in the reference.  Arguments, limits,
+ * errors and results are those of dt_attn_seg_jobs_ws_fwd called with a workspace of exactly that
+ * size: the split is planned to fit the array (a tail that would need more parts gets fewer), so the
+ * scratch need does not grow with the input and no shape is turned away on its account; a plan
+ * that does not fit is refused with DT_ERR_INVALID instead of being launched.  The call makes no
+ * hipMalloc / hipFree; the array's device address is looked up once per device on the first call
+ * there.  All calls on one GPU share the array: calls that overlap in time on one GPU (different
+ * streams or threads) race on it; order them on one stream.  Nothing in the array has to start at
+ * zero (every partial state that is read was written by the same call).
+ */
+#define DT_NOALLOC_TAIL_SLOTS 512
+int dt_attn_seg_jobs_noalloc_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D,
+                                 int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
+                                 int32_t n_chunks, const void* const* k_ptrs, const void* const* v_ptrs,
+                                 const int32_t* kv_lens, const int64_t* kv_stride_b,
+                                 int64_t kv_stride_s, int64_t kv_stride_h,
+                                 int32_t n_jobs, const int32_t* job_begin, const int32_t* job_chunks,
+                                 const int32_t* entry_kv_begin, const int32_t* entry_kv_len,
+                                 const int32_t* job_q_begin, const int32_t* job_q_len,
+                                 void* const* out_ptrs, float* const* lse_ptrs,
+                                 float softmax_scale, int32_t flags, void* stream);
+
+/*
  * N-way LSE merge: lse = logsumexp_i lse_i, out = sum_i exp(lse_i - lse) out_i.
  * Replaces the chain of update_out_and_lse / _update_out_and_lse calls
  * (utils.py:24-84; called at core/attention.py:116,144,194,196,213 and
