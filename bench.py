@@ -6,17 +6,28 @@ diffusion step) at the HunyuanVideo per-rank shape: local query shard of 14882 t
 KV = 8 chunks of 14882 tokens, H=24, D=128, bf16, under the seeded Bernoulli(0.6) reuse mask
 over 50 steps x 60 layers.  Inputs are resident in HBM before the timed region.
 
+The timed calls are a stratified sample of the schedule's (step, layer) rows: the rows are sorted by
+the number of chunks they recompute and visited with a fixed stride through that order, so any
+number of steps sees the schedule's mix of cheap and expensive rows and ``value`` does not depend
+on ``--steps``.
+
 Prints ONE JSON line: ms per layer call plus
   * ``roofline``        the fresh-chunk attention kernel against the bf16 dense MFMA peak,
   * ``roofline_merge``  the fused LSE-merge kernel against the HBM peak,
   * ``cache_gbs``       cache store / load copies against the HBM peak,
+  * ``other_configs``   compact records of the other single-GPU configurations (CogVideoX share,
+                        Step-Video share, the 32-chunk reuse sweep),
   * ``cpu_baseline``    the torch-math oracle timed on this box's host cores on a bounded sample.
+The HBM-bound kernels are timed over a rotation of distinct buffers of more than 1 GB in total,
+so the figures are those of HBM and not of the 256 MB memory-side cache.
 """
 import argparse
 import json
 import math
 import os
+import subprocess
 import sys
+import threading
 import time
 
 import numpy as np
@@ -27,6 +38,7 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+NOMINAL_CLOCK_MHZ = 2400.0  # the shader clock the bf16 peak is quoted at
 
 WORKLOADS = {
     # name: (label, B, H, D, Sq, chunk lengths, T, L, reuse probability, diag, qk norm)
@@ -38,24 +50,30 @@ WORKLOADS = {
 
 
 def make_inputs(B, H, D, Sq, lens, norm, device, seed=0):
-    g = torch.Generator(device="cpu").manual_seed(seed)
+    """Seeded synthetic q / K chunks / V chunks, drawn on the device (Q and K normalised over D as the model does)."""
+    g = torch.Generator(device=device).manual_seed(seed)
 
     def draw(n, normalise):
-        x = torch.randn(B, n, H, D, generator=g)
+        x = torch.randn(B, n, H, D, generator=g, device=device)
         if normalise == "rms":
             x = x / x.pow(2).mean(-1, keepdim=True).sqrt()
         elif normalise == "layer":
             x = torch.nn.functional.layer_norm(x, (D,))
         return x.bfloat16()
 
-    q = draw(Sq, norm).to(device)
-    ks = [draw(n, norm).to(device) for n in lens]
-    vs = [draw(n, None).to(device) for n in lens]
+    q = draw(Sq, norm)
+    ks = [draw(n, norm) for n in lens]
+    vs = [draw(n, None) for n in lens]
     return q, ks, vs
 
 
-def time_kernel(fn, reps, warm=3):
+PROFILING = False   # --kernels-only: a handful of launches per kernel, no minimum timed duration
+
+
+def time_kernel(fn, reps, warm=3, min_ms=40.0):
     """Average duration in ms of ``fn`` over ``reps`` launches (HIP events on the launch stream)."""
+    if PROFILING:
+        warm, reps, min_ms = 1, 2, 0.0
     for _ in range(warm):
         fn()
     torch.cuda.synchronize()
@@ -66,8 +84,8 @@ def time_kernel(fn, reps, warm=3):
     e1.record()
     torch.cuda.synchronize()
     total = e0.elapsed_time(e1)
-    if total < 40.0:  # short kernels: time at least 40 ms of them, so that clock ramps average out
-        more = int(reps * 40.0 / max(total, 1e-3)) + 1
+    if total < min_ms:  # short kernels: time at least min_ms of them, so that clock ramps average out
+        more = int(reps * min_ms / max(total, 1e-3)) + 1
         e0.record()
         for _ in range(more):
             fn()
@@ -75,6 +93,57 @@ def time_kernel(fn, reps, warm=3):
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / more
     return total / reps
+
+
+class Rotation:
+    """Calls ``fn(i)`` with i cycling through ``n`` argument sets (distinct memory per call)."""
+
+    def __init__(self, fn, n):
+        self.fn, self.n, self.k = fn, max(1, n), 0
+
+    def __call__(self):
+        self.fn(self.k % self.n)
+        self.k += 1
+
+
+def sample_clock_mhz(fn, seconds=2.0):
+    """Shader clock (MHz) read with ``rocm-smi`` while ``fn`` keeps the GPU busy; None if it cannot be read."""
+    samples, stop = [], [False]
+
+    def sampler():
+        while not stop[0]:
+            try:
+                r = subprocess.run(["rocm-smi", "--showclocks", "--json"], capture_output=True, text=True, timeout=10)
+                card = list(json.loads(r.stdout).values())[0]
+                samples.append((time.perf_counter(), float(card["sclk clock speed:"].strip("()Mhz"))))
+            except Exception:
+                pass
+            time.sleep(0.1)
+
+    th = threading.Thread(target=sampler, daemon=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    th.start()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(4):
+            fn()
+        torch.cuda.synchronize()
+    stop[0] = True
+    th.join(timeout=15)
+    vals = [v for ts, v in samples if ts - t0 > 0.5]   # after the ramp
+    return round(sum(vals) / len(vals), 0) if vals else None
+
+
+def stratified_order(counts):
+    """A fixed visiting order of the schedule rows in which every prefix has (nearly) the whole
+    schedule's distribution of ``counts``: rows sorted by count, visited with a stride of about
+    1/golden-ratio of their number (coprime with it)."""
+    order = sorted(range(len(counts)), key=lambda i: (counts[i], i))
+    m = len(order)
+    stride = max(1, int(m * 0.6180339887))
+    while math.gcd(stride, m) != 1:
+        stride += 1
+    return [order[(j * stride) % m] for j in range(m)]
 
 
 def cpu_baseline(B, H, D, Sq, lens, mean_computed, n_chunks, norm, budget_s=20.0):
@@ -135,8 +204,7 @@ def bench_stride_schedule(args):
     cfg = config.init_config(None, num_inference_steps=T, num_layers=L, stride_percentiles=[0, 40, 90],
                              stride_dividers=[8, 4, 2, 1])
     rmod.destroy_redundancy_map()
-    rm = rmod.init_redundancy_map(cfg, redun_map_path=os.path.join(ROOT, "tests", "golden", "redundancy_map_50_60.pt"),
-                                  quiet=True)
+    rmod.init_redundancy_map(cfg, redun_map_path=os.path.join(ROOT, "tests", "golden", "redundancy_map_50_60.pt"), quiet=True)
     q, ks, vs = make_inputs(B, H, D, Sq, lens, norm, dev)
     group = parallel_state.get_usp_group()
     group.set_kv_chunks(ks, vs)
@@ -164,48 +232,32 @@ def bench_stride_schedule(args):
     }), flush=True)
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=120)
-    ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="hunyuanvideo", choices=list(WORKLOADS))
-    ap.add_argument("--layers", type=int, default=None, help="layers to instantiate (default: all of the model)")
-    ap.add_argument("--reuse", type=float, default=None, help="override the mask's reuse probability")
-    ap.add_argument("--kernel-reps", type=int, default=20)
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--schedule", default="mask", choices=["mask", "stride"],
-                    help="mask: the seeded Bernoulli reuse mask (the headline metric); stride: the reference's own stride "
-                         "schedule from the HunyuanVideo redundancy map it ships (a separate, shorter report)")
-    ap.add_argument("--kernels-only", action="store_true",
-                    help="run only the per-kernel roofline launches (short; for rocprofv3 counter passes)")
-    args = ap.parse_args()
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py measures one sequence-parallel rank's share on ONE GPU; --gpus > 1 is not part of this build",
-              file=sys.stderr)
-        sys.exit(2)
-    if not torch.cuda.is_available():
-        print("bench.py needs a GPU", file=sys.stderr)
-        sys.exit(2)
+def load_traffic(workload):
+    """HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE runs, committed under profiles/
+    (``{"attn_fwd": {"<chunks per launch>": bytes, ...}, "merge_states": {"<states>": bytes}}``)."""
+    path = os.path.join(ROOT, "profiles", f"hbm_traffic_{workload}.json")
+    if not os.path.exists(path):
+        return {}
+    with open(path) as f:
+        return json.load(f).get("bytes_per_launch", {})
 
+
+def run_workload(name, args, steps, warmup, main, reuse=None, kernels_only=False):
+    """Layer calls plus per-kernel launches of one workload; returns the record (main: the full one)."""
     from ditango_amd import _hip
     from ditango_amd.core import config, parallel_state, redundancy_map as rmod
     from ditango_amd.core.attention import proAttention
     from ditango_amd.utils import update_timestep
-    _hip.load_library()
 
-    if args.schedule == "stride":
-        return bench_stride_schedule(args)
-    label, B, H, D, Sq, lens, T, L, p, diag, norm = WORKLOADS[args.workload]
-    if args.reuse is not None:
-        p = args.reuse
+    label, B, H, D, Sq, lens, T, L, p, diag, norm = WORKLOADS[name]
+    if reuse is not None:
+        p = reuse
     C = len(lens)
     L_run = min(L, args.layers) if args.layers else L
-    if args.workload == "sweep":
+    if name == "sweep":
         L_run = min(L_run, 2)   # 32 cached states of 743 MB per layer
         T = 2                   # step 0 fills the cache, step 1 is measured
     dev = torch.device("cuda", 0)
-    torch.cuda.set_device(dev)
     rank = max(diag, 0)
     parallel_state.init_local_groups(C, rank)
     cfg = config.init_config(None, num_inference_steps=T, num_layers=L)
@@ -226,137 +278,263 @@ def main():
         layers[l].attn(q, ks[rank], vs[rank])
     torch.cuda.synchronize()
 
-    calls = [(t, l) for t in range(1, T) for l in range(L_run)]
-    need = args.warmup + args.steps
-    seq = [calls[i % len(calls)] for i in range(need)]
+    rows_tl = [(t, l) for t in range(1, T) for l in range(L_run)]
+    counts = [int(rm.sched_counts_host[t, l, 0]) for t, l in rows_tl]
+    order = stratified_order(counts)
+    population_mean = float(np.mean(counts))
+    seq = [rows_tl[order[i % len(order)]] for i in range(warmup + steps)]
 
     def run(t, l):
         update_timestep(t)
         return layers[l].attn(q, ks[rank], vs[rank])
 
-    planned = seq[args.warmup:]   # the calls the default run times (also fixes the typical launch below)
-    if args.kernels_only:
-        args.warmup, args.steps = 0, 1
-        seq = seq[:1]
-    for t, l in seq[:args.warmup]:
+    timed = seq[warmup:]
+    if kernels_only:
+        warmup, steps, timed = 0, 1, seq[:1]
+    for t, l in seq[:warmup]:
         run(t, l)
     torch.cuda.synchronize()
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(len(timed) + 1)]
     t0 = time.perf_counter()
-    for t, l in seq[args.warmup:]:
+    marks[0].record()
+    for i, (t, l) in enumerate(timed):
         run(t, l)
+        marks[i + 1].record()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    ms_per_step = 1e3 * elapsed / args.steps
-    n_comp = [int(rm.sched_counts_host[t, l, 0]) for t, l in planned]
+    ms_per_step = 1e3 * elapsed / steps
+    n_comp = [int(rm.sched_counts_host[t, l, 0]) for t, l in timed]
     mean_computed = float(np.mean(n_comp))
+    # per-call device time by the number of chunks a call recomputes, and the mean over the WHOLE schedule it implies
+    per_count = {}
+    for i, k in enumerate(n_comp):
+        per_count.setdefault(k, []).append(marks[i].elapsed_time(marks[i + 1]))
+    hist = {k: counts.count(k) / len(counts) for k in set(counts)}
+    covered = sum(w for k, w in hist.items() if k in per_count)
+    schedule_mean_ms = sum(w * float(np.mean(per_count[k])) for k, w in hist.items() if k in per_count) / max(covered, 1e-9)
     Sk_mean = float(np.mean(lens))
     flops_per_chunk = 4.0 * B * H * Sq * Sk_mean * D
     rows = B * Sq * H
 
     # ---- per-kernel rooflines, measured live with HIP events on the launch stream ----------
-    reps = args.kernel_reps
-    out_s = torch.empty(B, Sq, H, D, dtype=torch.bfloat16, device=dev)
-    lse_s = torch.empty(B, H, Sq, dtype=torch.float32, device=dev)
+    reps = args.kernel_reps if main else max(5, args.kernel_reps // 2)
+    state_bytes = rows * (2 * D + 4)
     # the dominant kernel in its typical launch: as many single-chunk states as a layer call
-    # computes on average (rounded), written into cache slots, one launch
-    n_typ = max(1, min(C, int(round(mean_computed))))
+    # computes on average over the schedule (rounded), written into cache-form states, one launch
+    n_typ = max(1, min(C, int(round(population_mean))))
     table = _hip.ChunkTable(ks, vs)
-    typ_jobs = [[c] for c in range(n_typ)]
-    typ_outs = [torch.empty_like(out_s) for _ in range(n_typ)]
-    typ_lses = [torch.empty_like(lse_s) for _ in range(n_typ)]
     k1_ws = _hip.attn_workspace(dev)   # the launch as proAttention makes it: with the tail-balancing workspace
-    k1_ms = time_kernel(lambda: _hip.attn_jobs_fwd(q, table, typ_jobs, typ_outs, typ_lses, workspace=k1_ws), reps)
-    k1_flops = sum(4.0 * B * H * Sq * lens[c] * D for c in range(n_typ))
-    k1_tflops = k1_flops / (k1_ms * 1e-3) / 1e12
-    k1s_ms = time_kernel(lambda: _hip.attn_jobs_fwd(q, table, [[0]], [out_s], [lse_s], workspace=k1_ws), reps)
-    k1s_tflops = 4.0 * B * H * Sq * lens[0] * D / (k1s_ms * 1e-3) / 1e12
+    st_outs = [torch.empty(B, Sq, H, D, dtype=torch.bfloat16, device=dev) for _ in range(n_typ)]
+    st_lses = [torch.empty(B, H, Sq, dtype=torch.float32, device=dev) for _ in range(n_typ)]
+
+    def k1_launch(n, qq=q, pre=False):
+        _hip.attn_jobs_fwd(qq, table, [[c] for c in range(n)], st_outs[:n], st_lses[:n], workspace=k1_ws, q_prescaled=pre)
+
+    def k1_flops(n):
+        return sum(4.0 * B * H * Sq * lens[c] * D for c in range(n))
+
+    if kernels_only:   # one launch of every size up to the chunk count, for the profiler (first dispatches of the kernel)
+        st_outs += [torch.empty_like(st_outs[0]) for _ in range(C - n_typ)]
+        st_lses += [torch.empty_like(st_lses[0]) for _ in range(C - n_typ)]
+        for n in range(1, C + 1):
+            k1_launch(n)
+        torch.cuda.synchronize()
+    k1_ms = time_kernel(lambda: k1_launch(n_typ), reps)
+    k1_tflops = k1_flops(n_typ) / (k1_ms * 1e-3) / 1e12
+    k1s_ms = time_kernel(lambda: k1_launch(1), reps)
+    k1s_tflops = k1_flops(1) / (k1s_ms * 1e-3) / 1e12
     # the same typical launch in the opt-in mode of a caller that folds softmax_scale * log2(e) into q
     # (reported beside the drop-in figure, never in place of it)
     q_folded = (q.float() * (D ** -0.5 * math.log2(math.e))).to(torch.bfloat16)
-    k1p_ms = time_kernel(lambda: _hip.attn_jobs_fwd(q_folded, table, typ_jobs, typ_outs, typ_lses, workspace=k1_ws,
-                                                    q_prescaled=True), reps)
-    k1p_tflops = k1_flops / (k1p_ms * 1e-3) / 1e12
-    del typ_outs, typ_lses, q_folded
+    k1p_ms = time_kernel(lambda: k1_launch(n_typ, q_folded, True), reps)
+    k1p_tflops = k1_flops(n_typ) / (k1p_ms * 1e-3) / 1e12
+    clock = None
+    if main and not kernels_only:
+        clock = sample_clock_mhz(lambda: k1_launch(n_typ))
+    del q_folded
 
-    cache0 = layers[0].cache
-    m_outs = [cache0.arena_out[c] if c != diag else cache0.diag_out for c in range(C)]
-    m_lses = [cache0.arena_lse[c] if c != diag else cache0.diag_lse for c in range(C)]
-    dst_o = torch.empty(B, Sq, H, D, dtype=torch.float32, device=dev)
-    dst_l = torch.empty(B, Sq, H, 1, dtype=torch.float32, device=dev)
-    k2_ms = time_kernel(lambda: _hip.merge_states(m_outs, m_lses, dst_out=dst_o, dst_lse=dst_l), reps)
+    # merge of all C states of a layer into the fp32 result, rotating over the layers' arenas
+    dst_n = max(1, min(8, int(1.2e9 // (rows * (4 * D + 4))) + 1))
+    dst_os = [torch.empty(B, Sq, H, D, dtype=torch.float32, device=dev) for _ in range(dst_n)]
+    dst_ls = [torch.empty(B, Sq, H, 1, dtype=torch.float32, device=dev) for _ in range(dst_n)]
+
+    def merge_layer(i):
+        cache = layers[i % L_run].cache
+        outs = [cache.arena_out[c] if c != diag else cache.diag_out for c in range(C)]
+        lses = [cache.arena_lse[c] if c != diag else cache.diag_lse for c in range(C)]
+        _hip.merge_states(outs, lses, dst_out=dst_os[i % dst_n], dst_lse=dst_ls[i % dst_n])
+
+    k2_ms = time_kernel(Rotation(merge_layer, L_run * dst_n), reps)
     k2_bytes = rows * (C * (2 * D + 4) + (4 * D + 4))
     k2_gbs = k2_bytes / (k2_ms * 1e-3) / 1e9
+    k2_ws_mb = (L_run * C * state_bytes + dst_n * rows * (4 * D + 4)) / 1e6
 
-    k3s_ms = time_kernel(lambda: _hip.cache_store(dst_o, dst_l, out_s, lse_s), reps)
+    # cache store / load, over a rotation of cache slots of distinct layers and of source / destination tensors
+    slots = [(layers[l].cache.arena_out[c], layers[l].cache.arena_lse[c]) for l in range(L_run) for c in range(C) if c != diag]
+    n_slots = max(1, min(len(slots), int(1.5e9 // state_bytes) + 1))
+    k3s_ms = time_kernel(Rotation(lambda i: _hip.cache_store(dst_os[i % dst_n], dst_ls[i % dst_n], *slots[i % n_slots]),
+                                  n_slots * dst_n), reps)
     k3s_gbs = rows * ((4 * D + 4) + (2 * D + 4)) / (k3s_ms * 1e-3) / 1e9
-    slot2_o, slot2_l = torch.empty_like(out_s), torch.empty_like(lse_s)
-    k3c_ms = time_kernel(lambda: _hip.cache_store(out_s, lse_s, slot2_o, slot2_l), reps)
+    k3c_ms = time_kernel(Rotation(lambda i: _hip.cache_store(*slots[i % n_slots], *slots[(i + n_slots // 2 + 1) % n_slots]),
+                                  n_slots), reps)
     k3c_gbs = rows * 2 * (2 * D + 4) / (k3c_ms * 1e-3) / 1e9
-    k3l_ms = time_kernel(lambda: _hip.cache_load(out_s, lse_s, torch.float32, True), reps)
+    k3l_ms = time_kernel(Rotation(lambda i: _hip.cache_load(*slots[i % n_slots], dst_out=dst_os[i % dst_n],
+                                                            dst_lse=dst_ls[i % dst_n]), n_slots * dst_n), reps)
     k3l_gbs = rows * ((2 * D + 4) + (4 * D + 4)) / (k3l_ms * 1e-3) / 1e9
+    copy_ws_mb = (n_slots * state_bytes + dst_n * rows * (4 * D + 4)) / 1e6
 
-    # producer step of the callers: RMSNorm + interleaved RoPE of K over the whole KV sequence, read in
-    # place from a fused QKV projection ("B L (K H D)"), written as the [B,S,H,D] bf16 the attention reads
-    S_all = int(sum(lens))
-    qkv = torch.randn(B, S_all, 3, H, D, device=dev, dtype=torch.bfloat16)
-    ang = torch.rand(S_all, D // 2, device=dev) * 6.28
-    p_cos = ang.cos().repeat_interleave(2, -1).contiguous()
-    p_sin = ang.sin().repeat_interleave(2, -1).contiguous()
-    p_w = torch.ones(D, device=dev)
-    p_out = torch.empty(B, S_all, H, D, dtype=torch.bfloat16, device=dev)
-    kp_ms = time_kernel(lambda: _hip.qk_norm_rope(qkv[:, :, 1], norm=_hip.DT_NORM_RMS, weight=p_w, rope=_hip.DT_ROPE_INTERLEAVED,
-                                                  cos=p_cos, sin=p_sin, out=p_out), reps, warm=40)
-    kp_bytes = B * S_all * H * D * 4 + S_all * D * 8
-    kp_gbs = kp_bytes / (kp_ms * 1e-3) / 1e9
-    del qkv, ang, p_cos, p_sin, p_out
+    # the yardstick: what the memory system delivers to a read-only kernel with the merge's access pattern
+    # (the bf16 halves of C cache slots, rotating over the layers)
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    probe_bytes = rows * D * 2 // 256 * 256
 
-    dmask = torch.from_numpy(mask).to(dev)
-    k4_ms = time_kernel(lambda: _hip.build_schedule_table(dmask, diag), reps)
-    # a plain copy of known size: the yardstick the profiler's FETCH_SIZE / WRITE_SIZE counters are scaled by
-    ref_src = torch.empty(1 << 28, dtype=torch.float32, device=dev)   # 1 GiB
-    ref_dst = torch.empty_like(ref_src)
-    copy_ms = time_kernel(lambda: ref_dst.copy_(ref_src), max(3, reps // 4))
-    copy_gbs = 2 * ref_src.numel() * 4 / (copy_ms * 1e-3) / 1e9
-    del ref_src, ref_dst
+    def probe(i):
+        cache = layers[i % L_run].cache
+        _hip.hbm_read_probe([cache.arena_out[c] for c in range(C)], sink)
 
-    # HBM bytes per launch measured offline with rocprofv3 counters (FETCH_SIZE + WRITE_SIZE),
-    # committed as text under profiles/; only meaningful for the default workload
-    traffic = {}
-    tpath = os.path.join(ROOT, "profiles", "hbm_traffic_hunyuanvideo.json")
-    if args.workload == "hunyuanvideo" and args.reuse is None and os.path.exists(tpath):
-        with open(tpath) as f:
-            traffic = json.load(f).get("bytes_per_launch", {})
+    kr_ms = time_kernel(Rotation(probe, L_run), reps)
+    kr_gbs = C * probe_bytes / (kr_ms * 1e-3) / 1e9
 
-    result = {
-        "metric": "ms/layer", "value": round(ms_per_step, 4), "unit": "ms", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
-        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": label, "B": B, "H": H, "D": D, "Sq": Sq, "kv_chunks": C, "Sk": lens[0],
-                   "mask": f"Bernoulli({p}) seed 0 over {T}x{L}x{C}, diag {diag}", "layers_instantiated": L_run,
-                   "mean_chunks_computed_per_call": round(mean_computed, 3)},
-        "layer_attn_tflops": round(flops_per_chunk * mean_computed / (ms_per_step * 1e-3) / 1e12, 1),
-        "roofline": {"kernel": "attn_fwd_kernel<%d>" % D, "bound": "mfma", "achieved": round(k1_tflops, 1),
-                     "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(k1_tflops / PEAK_BF16_TFLOPS, 4),
-                     "traffic": traffic.get("attn_fwd"), "launch_ms": round(k1_ms, 4), "flop_per_launch": k1_flops,
-                     "chunks_per_launch": n_typ, "single_chunk_launch_tflops": round(k1s_tflops, 1),
-                     "single_chunk_launch_ms": round(k1s_ms, 4),
-                     "q_prescaled_launch_tflops": round(k1p_tflops, 1), "q_prescaled_launch_ms": round(k1p_ms, 4)},
-        "roofline_merge": {"kernel": "merge_states_kernel<%d>" % D, "bound": "hbm", "achieved": round(k2_gbs, 1),
-                           "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(k2_gbs / PEAK_HBM_GBS, 4),
-                           "traffic": traffic.get("merge_states"), "launch_us": round(k2_ms * 1e3, 2), "bytes_per_launch": k2_bytes,
-                           "states": C},
-        "cache_gbs": {"store_fp32_to_slot": round(k3s_gbs, 1), "store_bf16_to_slot": round(k3c_gbs, 1),
-                      "load_slot_to_fp32": round(k3l_gbs, 1), "peak": PEAK_HBM_GBS,
-                      "frac_store_bf16": round(k3c_gbs / PEAK_HBM_GBS, 4), "frac_load": round(k3l_gbs / PEAK_HBM_GBS, 4)},
-        "producer": {"kernel": "qk_norm_rope_kernel<%d>" % D, "bound": "hbm", "achieved": round(kp_gbs, 1),
-                     "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(kp_gbs / PEAK_HBM_GBS, 4),
-                     "launch_us": round(kp_ms * 1e3, 2), "bytes_per_launch": kp_bytes, "tokens": S_all,
-                     "what": "RMSNorm + interleaved RoPE of K over the whole KV sequence, strided read from a fused QKV tensor"},
-        "schedule_builder_us": round(k4_ms * 1e3, 2),
-        "plain_copy_1GiB_gbs": round(copy_gbs, 1),
-    }
+    traffic = load_traffic(name) if reuse is None else {}
+    # counter bytes of exactly the launch shape that is timed next to them, or nothing
+    k1_traffic = traffic.get("attn_fwd", {}).get(str(n_typ)) if isinstance(traffic.get("attn_fwd"), dict) else None
+    k2_traffic = traffic.get("merge_states", {}).get(str(C)) if isinstance(traffic.get("merge_states"), dict) else None
+    frac = k1_tflops / PEAK_BF16_TFLOPS
+    roofline = {"kernel": "attn_fwd_kernel<%d>" % D, "bound": "mfma", "achieved": round(k1_tflops, 1),
+                "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(frac, 4),
+                "traffic": k1_traffic, "launch_ms": round(k1_ms, 4), "flop_per_launch": k1_flops(n_typ),
+                "chunks_per_launch": n_typ, "single_chunk_launch_tflops": round(k1s_tflops, 1),
+                "single_chunk_launch_ms": round(k1s_ms, 4),
+                "q_prescaled_launch_tflops": round(k1p_tflops, 1), "q_prescaled_launch_ms": round(k1p_ms, 4)}
+    if clock:
+        # the part is power-limited under this kernel: what the kernel reaches of the peak AT THE CLOCK IT RUNS AT
+        roofline["clock_mhz_under_load"] = clock
+        roofline["frac_at_clock"] = round(frac * NOMINAL_CLOCK_MHZ / clock, 4)
+    roofline_merge = {"kernel": "merge_states_kernel<%d>" % D, "bound": "hbm", "achieved": round(k2_gbs, 1),
+                      "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(k2_gbs / PEAK_HBM_GBS, 4),
+                      "traffic": k2_traffic, "launch_us": round(k2_ms * 1e3, 2), "bytes_per_launch": k2_bytes,
+                      "states": C, "working_set_mb": round(k2_ws_mb, 0),
+                      "read_probe_gbs": round(kr_gbs, 1), "frac_of_read_probe": round(k2_gbs / kr_gbs, 4)}
+    cache_gbs = {"store_fp32_to_slot": round(k3s_gbs, 1), "store_bf16_to_slot": round(k3c_gbs, 1),
+                 "load_slot_to_fp32": round(k3l_gbs, 1), "peak": PEAK_HBM_GBS,
+                 "frac_store_bf16": round(k3c_gbs / PEAK_HBM_GBS, 4), "frac_load": round(k3l_gbs / PEAK_HBM_GBS, 4),
+                 "working_set_mb": round(copy_ws_mb, 0), "slots_rotated": n_slots}
+    cfg_rec = {"workload": label, "B": B, "H": H, "D": D, "Sq": Sq, "kv_chunks": C, "Sk": lens[0],
+               "mask": f"Bernoulli({p}) seed 0 over {T}x{L}x{C}, diag {diag}", "layers_instantiated": L_run,
+               "mean_chunks_computed_per_call": round(mean_computed, 3),
+               "schedule_mean_chunks_computed_per_call": round(population_mean, 3)}
+    layer_tflops = flops_per_chunk * mean_computed / (ms_per_step * 1e-3) / 1e12
+
+    if not main:
+        rec = {"config": cfg_rec, "ms_per_layer": round(ms_per_step, 4), "steps": steps,
+               "ms_per_layer_schedule_mean": round(schedule_mean_ms, 4),
+               "layer_attn_tflops": round(layer_tflops, 1),
+               "attn": {"frac": roofline["frac"], "tflops": roofline["achieved"], "chunks_per_launch": n_typ,
+                        "launch_ms": roofline["launch_ms"], "single_chunk_frac": round(k1s_tflops / PEAK_BF16_TFLOPS, 4),
+                        "q_prescaled_frac": round(k1p_tflops / PEAK_BF16_TFLOPS, 4), "traffic": k1_traffic},
+               "merge": {"frac": roofline_merge["frac"], "gbs": roofline_merge["achieved"], "states": C,
+                         "launch_us": roofline_merge["launch_us"], "read_probe_gbs": roofline_merge["read_probe_gbs"],
+                         "traffic": k2_traffic},
+               "cache_gbs": {"store_bf16_to_slot": cache_gbs["store_bf16_to_slot"], "load_slot_to_fp32": cache_gbs["load_slot_to_fp32"]}}
+    else:
+        # producer step of the callers: RMSNorm + interleaved RoPE of K over the whole KV sequence, read in
+        # place from a fused QKV projection ("B L (K H D)"), written as the [B,S,H,D] bf16 the attention reads
+        S_all = int(sum(lens))
+        qkv = torch.randn(B, S_all, 3, H, D, device=dev, dtype=torch.bfloat16)
+        ang = torch.rand(S_all, D // 2, device=dev) * 6.28
+        p_cos = ang.cos().repeat_interleave(2, -1).contiguous()
+        p_sin = ang.sin().repeat_interleave(2, -1).contiguous()
+        p_w = torch.ones(D, device=dev)
+        p_out = torch.empty(B, S_all, H, D, dtype=torch.bfloat16, device=dev)
+        kp_ms = time_kernel(lambda: _hip.qk_norm_rope(qkv[:, :, 1], norm=_hip.DT_NORM_RMS, weight=p_w, rope=_hip.DT_ROPE_INTERLEAVED,
+                                                      cos=p_cos, sin=p_sin, out=p_out), reps, warm=40)
+        kp_bytes = B * S_all * H * D * 4 + S_all * D * 8
+        kp_gbs = kp_bytes / (kp_ms * 1e-3) / 1e9
+        del qkv, ang, p_cos, p_sin, p_out
+        dmask = torch.from_numpy(mask).to(dev)
+        k4_ms = time_kernel(lambda: _hip.build_schedule_table(dmask, diag), reps)
+        # a plain copy of known size: the yardstick the profiler's FETCH_SIZE / WRITE_SIZE counters are scaled by
+        ref_src = torch.empty(1 << 28, dtype=torch.float32, device=dev)   # 1 GiB
+        ref_dst = torch.empty_like(ref_src)
+        copy_ms = time_kernel(lambda: ref_dst.copy_(ref_src), max(3, reps // 4))
+        copy_gbs = 2 * ref_src.numel() * 4 / (copy_ms * 1e-3) / 1e9
+        del ref_src, ref_dst
+        rec = {
+            "metric": "ms/layer", "value": round(ms_per_step, 4), "unit": "ms", "n_gpus": 1,
+            "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 4),
+            "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": cfg_rec,
+            "ms_per_layer_schedule_mean": round(schedule_mean_ms, 4),
+            "ms_by_chunks_computed": {str(k): round(float(np.mean(v)), 4) for k, v in sorted(per_count.items())},
+            "layer_attn_tflops": round(layer_tflops, 1),
+            "roofline": roofline, "roofline_merge": roofline_merge, "cache_gbs": cache_gbs,
+            "producer": {"kernel": "qk_norm_rope_kernel<%d>" % D, "bound": "hbm", "achieved": round(kp_gbs, 1),
+                         "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(kp_gbs / PEAK_HBM_GBS, 4),
+                         "launch_us": round(kp_ms * 1e3, 2), "bytes_per_launch": kp_bytes, "tokens": S_all,
+                         "what": "RMSNorm + interleaved RoPE of K over the whole KV sequence, strided read from a fused QKV tensor"},
+            "schedule_builder_us": round(k4_ms * 1e3, 2),
+            "plain_copy_1GiB_gbs": round(copy_gbs, 1),
+        }
+    # release this workload's memory before the next one
+    for a in layers:
+        a.cache.release()
+    del layers, q, ks, vs, table, st_outs, st_lses, dst_os, dst_ls, slots
+    group.set_kv_chunks([None] * C, [None] * C)
+    rmod.destroy_redundancy_map()
+    parallel_state.destroy_local_groups()
+    update_timestep(0)
+    torch.cuda.empty_cache()
+    rec["_mean_computed"] = mean_computed
+    return rec
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=120)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="hunyuanvideo", choices=list(WORKLOADS))
+    ap.add_argument("--layers", type=int, default=None, help="layers to instantiate (default: all of the model)")
+    ap.add_argument("--reuse", type=float, default=None, help="override the mask's reuse probability")
+    ap.add_argument("--kernel-reps", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true", help="skip the compact records of the other configurations")
+    ap.add_argument("--schedule", default="mask", choices=["mask", "stride"],
+                    help="mask: the seeded Bernoulli reuse mask (the headline metric); stride: the reference's own stride "
+                         "schedule from the HunyuanVideo redundancy map it ships (a separate, shorter report)")
+    ap.add_argument("--kernels-only", action="store_true",
+                    help="run only the per-kernel roofline launches (short; for rocprofv3 counter passes)")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one sequence-parallel rank's share on ONE GPU; --gpus > 1 is not part of this build",
+              file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+
+    from ditango_amd import _hip
+    _hip.load_library()
+    torch.cuda.set_device(0)
+    global PROFILING
+    PROFILING = args.kernels_only
+
+    if args.schedule == "stride":
+        return bench_stride_schedule(args)
+    result = run_workload(args.workload, args, args.steps, args.warmup, main=True, reuse=args.reuse,
+                          kernels_only=args.kernels_only)
+    mean_computed = result.pop("_mean_computed")
+    if not args.kernels_only and not args.no_other_configs and args.workload == "hunyuanvideo" and args.reuse is None:
+        others = {}
+        for name, reuse in (("cogvideox", None), ("stepvideo", None), ("sweep", 0.5), ("sweep", 0.9)):
+            steps = 40 if name != "sweep" else 6
+            rec = run_workload(name, args, steps, 4 if name != "sweep" else 2, main=False, reuse=reuse)
+            rec.pop("_mean_computed")
+            others[name if name != "sweep" else f"sweep_reuse_{reuse}"] = rec
+        result["other_configs"] = others
     if not args.no_cpu_baseline and not args.kernels_only:
-        result["cpu_baseline"] = cpu_baseline(B, H, D, Sq, lens, mean_computed, C, norm)
+        label, B, H, D, Sq, lens, T, L, p, diag, norm = WORKLOADS[args.workload]
+        result["cpu_baseline"] = cpu_baseline(B, H, D, Sq, lens, mean_computed, len(lens), norm)
     print(json.dumps(result), flush=True)
 
 

@@ -71,6 +71,7 @@ _SIGNATURES = {
     "dt_cache_load": (ctypes.c_int, [c_vp, c_vp, c_vp, c_i32, c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp]),
     "dt_build_schedule": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp, c_vp]),
     "dt_build_schedule_table": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp, c_vp]),
+    "dt_hbm_read_probe": (ctypes.c_int, [_P(c_vp), c_i32, c_i64, c_vp, c_vp]),
     "dt_rel_l1_sums": (ctypes.c_int, [c_vp, c_vp, c_i64, c_vp, c_vp]),
     "dt_qk_norm_rope": (ctypes.c_int, [c_vp, c_i64, c_i64, c_i64, c_vp, c_i32, c_i32, c_i32, c_i32,
                                        c_i32, c_vp, c_vp, c_f32, c_i32, c_vp, c_vp, c_i64, c_i32, c_i32,
@@ -469,13 +470,17 @@ def cache_store(src_out: torch.Tensor, src_lse: torch.Tensor, slot_out: torch.Te
 
 
 def cache_load(slot_out: torch.Tensor, slot_lse: torch.Tensor, dst_dtype: torch.dtype = torch.float32,
-               dst_lse_bsh: bool = False):
+               dst_lse_bsh: bool = False, dst_out: Optional[torch.Tensor] = None, dst_lse: Optional[torch.Tensor] = None):
     lib = load_library()
     B, Sq, H, D = slot_out.shape
     _require(slot_out.dtype == torch.bfloat16 and slot_out.is_contiguous(), "slot_out must be contiguous bf16")
     _require(slot_lse.dtype == torch.float32 and slot_lse.is_contiguous() and tuple(slot_lse.shape) == (B, H, Sq), "slot_lse must be contiguous fp32 [B,H,Sq]")
-    dst_out = torch.empty((B, Sq, H, D), dtype=dst_dtype, device=slot_out.device)
-    dst_lse = torch.empty((B, Sq, H, 1) if dst_lse_bsh else (B, H, Sq), dtype=torch.float32, device=slot_out.device)
+    if dst_out is None:
+        dst_out = torch.empty((B, Sq, H, D), dtype=dst_dtype, device=slot_out.device)
+    if dst_lse is None:
+        dst_lse = torch.empty((B, Sq, H, 1) if dst_lse_bsh else (B, H, Sq), dtype=torch.float32, device=slot_out.device)
+    _require(dst_out.is_contiguous() and tuple(dst_out.shape) == (B, Sq, H, D), "dst_out must be contiguous [B,Sq,H,D]")
+    dst_lse_bsh = lse_layout_of(dst_lse, B, Sq, H) == DT_LSE_BSH
     rc = lib.dt_cache_load(slot_out.data_ptr(), slot_lse.data_ptr(), dst_out.data_ptr(), _dtype_code(dst_out),
                            dst_lse.data_ptr(), DT_LSE_BSH if dst_lse_bsh else DT_LSE_BHS, B, Sq, H, D, _stream())
     _check(rc, "dt_cache_load")
@@ -509,6 +514,20 @@ def build_schedule_table(mask: torch.Tensor, diag: int = -1):
     rc = lib.dt_build_schedule_table(mask.data_ptr(), T, L, C, int(diag), comp.data_ptr(), reu.data_ptr(), cnt.data_ptr(), _stream())
     _check(rc, "dt_build_schedule_table")
     return comp, reu, cnt
+
+
+def hbm_read_probe(buffers: Sequence[torch.Tensor], sink: torch.Tensor) -> None:
+    """Read ``buffers`` (equally sized, contiguous, a multiple of 256 bytes each) with the merge kernel's
+    access pattern and discard the data: the bandwidth yardstick of the HBM-bound kernels."""
+    lib = load_library()
+    n = len(buffers)
+    nbytes = buffers[0].numel() * buffers[0].element_size()
+    for b in buffers:
+        _require(b.is_cuda and b.is_contiguous() and b.numel() * b.element_size() == nbytes, "probe buffers must be equally sized contiguous device tensors")
+    _require(sink.is_cuda and sink.numel() * sink.element_size() >= 4, "sink must be a device tensor of at least 4 bytes")
+    ptrs = (c_vp * n)(*[b.data_ptr() for b in buffers])
+    rc = lib.dt_hbm_read_probe(ptrs, n, nbytes // 256 * 256, sink.data_ptr(), _stream())
+    _check(rc, "dt_hbm_read_probe")
 
 
 def rel_l1_sums(a: torch.Tensor, b: torch.Tensor, sums: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -6,8 +6,8 @@
 //
 // Shape of the computation
 //   * One workgroup = 8 wavefronts = 256 queries of one (batch, head); each
-//     wavefront owns 32 queries.  One workgroup per CU, two wavefronts per SIMD
-//     (256 VGPRs each).
+//     wavefront owns 32 queries.  D = 128: one workgroup per CU, two wavefronts per
+//     SIMD (256 VGPRs each); D = 64: two workgroups per CU (128 VGPRs each).
 //   * The 8 wavefronts form two groups of 4 that run the same loop ONE PHASE
 //     APART ("ping-pong"): while group A issues the MFMAs of a tile
 //     (O^T += V^T P^T of the previous tile, then S^T = K Q^T of this one), group B
@@ -211,8 +211,15 @@ __device__ __forceinline__ void load_block_to_lds(u32x4 rsrc, uint32_t lane_off,
                : "memory", "m0");
 }
 
+// Wavefronts per SIMD the register budget is set for.  D = 128: two (one workgroup per CU: its LDS
+// tiles fill the CU).  D = 64: four, i.e. TWO workgroups per CU (64 KB of LDS and at most 128
+// registers each): the second workgroup's wavefronts issue into the barrier waits, the start-up and
+// the epilogue of the first, which at 35 key tiles per work item are a tenth of its time (+10 %).
+#ifndef DT_D64_WAVES
+#define DT_D64_WAVES 4
+#endif
 template <int D, bool kPre>
-__global__ __launch_bounds__(kThreads, 2) void attn_fwd_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd_kernel(const AttnArgs a) {
   using T = Tile<D>;
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 

@@ -289,6 +289,15 @@ int dt_build_schedule_table(const uint8_t* mask, int32_t T, int32_t L, int32_t C
 int dt_rel_l1_sums(const float* a, const float* b, int64_t n, double* sums, void* stream);
 
 /*
+ * Measurement aid, no counterpart in the reference: reads n_streams device buffers of `bytes` bytes
+ * each (a multiple of 256) with the access pattern of dt_merge_states (a workgroup takes 32
+ * consecutive 256-byte rows of every stream, eight streams in flight at a time) and discards the
+ * data.  Its rate is what this part's memory system delivers to that pattern, the yardstick next to
+ * the nominal HBM peak for the merge and cache kernels.  sink: one device word, (almost) never written.
+ */
+int dt_hbm_read_probe(const void* const* streams, int32_t n_streams, int64_t bytes, uint32_t* sink, void* stream);
+
+/*
  * Producer side of an attention call: normalise every head row of x over D, apply the
  * rotary position embedding to the token rows [rope_begin, rope_end) and write the result
  * as bf16 [B,S,H,D] contiguous, the layout the attention entry points read -- one pass over

@@ -265,3 +265,29 @@ def test_tail_balancing_random_launches_match_plain(hip, seed):
         assert torch.isfinite(bo).all()
         assert (po - bo).abs().max() <= 2.0 ** -7 * po.abs().max()
         assert (res[0][1][j] - res[1][1][j]).abs().max() <= 1e-5
+
+
+def test_read_probe_and_its_argument_checks(hip):
+    """The bandwidth yardstick reads its streams and writes nothing; bad arguments are refused without a launch."""
+    bufs = [torch.full((1000, 64), 3, dtype=torch.int32, device="cuda") for _ in range(11)]    # 256 000 bytes each
+    sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+    hip.hbm_read_probe(bufs, sink)
+    torch.cuda.synchronize()
+    assert int(sink.item()) == 0 and all(int(b.sum().item()) == 3 * 64000 for b in bufs)
+    with pytest.raises(hip.DitangoHipError):
+        hip.hbm_read_probe(bufs + [bufs[0][:500]], sink)
+    with pytest.raises(hip.DitangoHipError):
+        hip.hbm_read_probe(bufs * 6, sink)                     # 66 streams: more than one launch takes
+
+
+def test_cache_load_into_given_tensors(hip):
+    B, S, H, D = 1, 70, 2, 64
+    g = torch.Generator().manual_seed(9)
+    o = _rand((B, S, H, D), g).cuda()
+    l = torch.randn(B, H, S, generator=g).cuda()
+    dst_o = torch.empty(B, S, H, D, dtype=torch.float32, device="cuda")
+    dst_l = torch.empty(B, S, H, 1, dtype=torch.float32, device="cuda")
+    ro, rl = hip.cache_load(o, l, dst_out=dst_o, dst_lse=dst_l)
+    torch.cuda.synchronize()
+    assert ro is dst_o and rl is dst_l
+    assert torch.equal(dst_o, o.float()) and torch.equal(dst_l.squeeze(-1).transpose(1, 2), l)
