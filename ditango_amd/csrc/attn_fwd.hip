@@ -612,7 +612,9 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
     // the vector issue port, the one doing the softmax goes first.  With equal priorities the older
     // wavefront wins in either role and the phases of the two groups come out unequal (measured
     // 1.43k vs 1.24k cycles of vector work), so every other barrier waits for a squeezed softmax.
-    __builtin_amdgcn_s_setprio(1);
+    // (D = 64: four wavefronts of two workgroups share the SIMD and the raised priority only gets in
+    // the way of the other workgroup's matrix phase: measured -3 %, so it is left at 0 there)
+    __builtin_amdgcn_s_setprio(D == 64 ? 0 : 1);
     if constexpr (!kLoadAfterMatrix) load_tile((kU + 3 + group) & (kNumBuf - 1));
     // (kPre: the same rare branch takes the reference off the scores of a wavefront in which some
     // row has left the band; everywhere else the reference is 0 and there is nothing to subtract)

@@ -337,6 +337,38 @@ __global__ __launch_bounds__(kThreads) void state_copy_kernel(const CopyArgs a) 
   }
 }
 
+// Same dtype and same lse layout on both sides: the state is two flat byte ranges (out, lse).  A
+// workgroup moves 16 KB: four 16-byte loads per lane, each instruction 1 KB contiguous per wavefront,
+// all in flight before the first store; non-temporal stores.
+struct FlatCopyArgs {
+  const uint8_t* src[2];
+  uint8_t* dst[2];
+  int64_t bytes[2];   // multiples of 4
+  uint32_t wgs0;      // workgroups of the first range
+};
+
+__global__ __launch_bounds__(kThreads) void flat_copy_kernel(const FlatCopyArgs a) {
+  const int which = blockIdx.x >= a.wgs0 ? 1 : 0;
+  const int64_t wg = which ? blockIdx.x - a.wgs0 : blockIdx.x;
+  const uint8_t* src = a.src[which];
+  uint8_t* dst = a.dst[which];
+  const int64_t bytes = a.bytes[which];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int64_t base = wg * 16384 + wave * 4096 + lane * 16;
+  const bool vec_ok = ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) == 0;
+  if (vec_ok && base - lane * 16 + 4096 <= bytes) {
+    u32x4 v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) v[k] = *reinterpret_cast<const u32x4*>(src + base + k * 1024);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) __builtin_nontemporal_store(v[k], reinterpret_cast<u32x4*>(dst + base + k * 1024));
+  } else {
+    // the range's last, partial 4 KB (or a range that is not 16-byte aligned): 4 bytes at a time
+    for (int64_t off = wg * 16384 + wave * 4096 + lane * 4; off < bytes && off < wg * 16384 + (wave + 1) * 4096; off += 256)
+      *reinterpret_cast<uint32_t*>(dst + off) = *reinterpret_cast<const uint32_t*>(src + off);
+  }
+}
+
 // One wavefront per (t, l) row: ballot + prefix popcount compaction.
 __global__ __launch_bounds__(64) void build_schedule_kernel(const uint8_t* mask, int /*T*/, int /*L*/, int C, int row0,
                                                             int diag, int32_t* compute_ids, int32_t* reuse_ids,
@@ -485,6 +517,25 @@ int launch_merge(const MergeArgs& a, int D, hipStream_t stream) {
 }
 
 int launch_copy(const CopyArgs& a, int D, hipStream_t stream) {
+  const bool with_lse = a.dst_lse != nullptr && a.src_lse != nullptr;
+  if (a.src_fp32 == a.dst_fp32 && (!with_lse || a.src_bsh == a.dst_bsh) && (D == 64 || D == 128)) {
+    const int64_t rows = (int64_t)a.B * a.Sq * a.H;
+    FlatCopyArgs f{};
+    f.src[0] = static_cast<const uint8_t*>(a.src_out);
+    f.dst[0] = static_cast<uint8_t*>(a.dst_out);
+    f.bytes[0] = rows * D * (a.src_fp32 ? 4 : 2);
+    f.src[1] = reinterpret_cast<const uint8_t*>(a.src_lse);
+    f.dst[1] = reinterpret_cast<uint8_t*>(a.dst_lse);
+    f.bytes[1] = with_lse ? rows * 4 : 0;
+    const int64_t w0 = (f.bytes[0] + 16383) / 16384, w1 = (f.bytes[1] + 16383) / 16384;
+    if (w0 + w1 > 0x7fffffffLL) {
+      set_error("copy grid too large");
+      return DT_ERR_INVALID;
+    }
+    f.wgs0 = (uint32_t)w0;
+    if (w0 + w1 > 0) hipLaunchKernelGGL(flat_copy_kernel, dim3((unsigned)(w0 + w1)), dim3(kThreads), 0, stream, f);
+    return hip_fail(hipGetLastError(), "flat_copy launch");
+  }
   const int rows_per_wg = kThreads / (D / 8) * kCopyRows;
   const int n_st = (a.Sq + rows_per_wg - 1) / rows_per_wg;
   const int64_t wgs = (int64_t)a.B * a.H * n_st;

@@ -191,6 +191,31 @@ def test_cache_store_load_roundtrip(hip):
     assert torch.equal(l.cpu(), lse)
 
 
+@pytest.mark.parametrize("B,Sq,H,D", [(1, 1, 1, 64), (2, 131, 3, 64), (1, 77, 3, 128), (1, 2222, 5, 64), (3, 700, 7, 128)])
+def test_same_format_copies_are_bit_exact(hip, B, Sq, H, D):
+    """State copies whose two sides share dtype and lse layout take the flat-range path: slot -> slot
+    (bf16 / [B,H,S]) and fp32 -> fp32 loads in either lse layout, with sizes that are no multiple of the
+    4 KB a wavefront moves, destinations inside larger buffers (nothing outside the state may be
+    written) and lse slices that are not 16-byte aligned."""
+    g = torch.Generator().manual_seed(B * 1000 + Sq)
+    rows = B * Sq * H
+    src_o = torch.randn(B, Sq, H, D, generator=g).bfloat16().cuda()
+    src_l = torch.randn(B, H, Sq, generator=g).cuda()
+    # destinations: slices of poisoned arenas, so that a write outside the state shows
+    pad = 3
+    arena_o = torch.full((3, B, Sq, H, D), 7.0, dtype=torch.bfloat16, device="cuda")
+    arena_l = torch.full((3 * rows + 2 * pad,), 7.0, dtype=torch.float32, device="cuda")
+    dst_l = arena_l[rows + pad: 2 * rows + pad].view(B, H, Sq)          # 12 bytes off a 16-byte boundary (for odd sizes)
+    hip.cache_store(src_o, src_l, arena_o[1], dst_l)
+    torch.cuda.synchronize()
+    assert torch.equal(arena_o[1], src_o) and torch.equal(dst_l, src_l)
+    assert (arena_o[0].float() == 7).all() and (arena_o[2].float() == 7).all()
+    assert (arena_l[:rows + pad] == 7).all() and (arena_l[2 * rows + pad:] == 7).all()
+    back_o, back_l = hip.cache_load(arena_o[1], dst_l.contiguous(), torch.bfloat16, dst_lse_bsh=False)
+    torch.cuda.synchronize()
+    assert torch.equal(back_o, src_o) and torch.equal(back_l, src_l)
+
+
 @pytest.mark.parametrize("T,L,C,p,diag", [(3, 4, 8, 0.5, 0), (2, 3, 32, 0.9, -1), (2, 2, 1, 0.5, 0), (1, 2, 100, 0.3, 77), (2, 2, 64, 0.0, 3), (1, 1, 65, 1.0, 64)])
 def test_schedule_builder_bit_exact(hip, T, L, C, p, diag):
     mask = ms.seeded_mask(T, L, C, p, seed=C + T, diag=diag, cold_first_step=False)
