@@ -223,7 +223,7 @@ def test_config1_fp32_inputs_as_stated(env):
     to bf16 at the kernel boundary (flash_attn_func itself takes no fp32).  Two comparisons: the strict
     bar against the oracle on the rounded inputs (same numbers as test_config1_cpu_plumbing_case), and
     the distance to fp32 attention of the UNROUNDED inputs, which is the price of the bf16 inputs:
-    observed 4e-3 in out and 6e-3 in lse for N(0,1) inputs at D = 64; the test allows 2e-2 / 2e-2."""
+    observed 8.6e-4 in out and 1.3e-3 in lse for N(0,1) inputs at D = 64; the test allows 5e-3 / 5e-3."""
     from ditango_amd.core.attention import proAttention
     from ditango_amd.core.parallel_state import get_usp_group
     from ditango_amd.utils import update_timestep
@@ -258,7 +258,7 @@ def test_config1_fp32_inputs_as_stated(env):
         lerr = (attn.last_lse.cpu().squeeze(-1).transpose(1, 2) - f_lse).abs().max().item()
         print(f"config1 fp32 inputs t={t}: distance to fp32 attention of the unrounded inputs: out {err:.3e} lse {lerr:.3e}",
               flush=True)
-        assert err <= 2e-2 and lerr <= 2e-2
+        assert err <= 5e-3 and lerr <= 5e-3
     with pytest.raises(TypeError):
         attn.attn(q1.double().cuda(), dk[0], dv[0])
 
