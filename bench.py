@@ -6,10 +6,10 @@ diffusion step) at the HunyuanVideo per-rank shape: local query shard of 14882 t
 KV = 8 chunks of 14882 tokens, H=24, D=128, bf16, under the seeded Bernoulli(0.6) reuse mask
 over 50 steps x 60 layers.  Inputs are resident in HBM before the timed region.
 
-The timed calls are a stratified sample of the schedule's (step, layer) rows: the rows are sorted by
-the number of chunks they recompute and visited with a fixed stride through that order, so any
-number of steps sees the schedule's mix of cheap and expensive rows and ``value`` does not depend
-on ``--steps``.
+The timed calls are a stratified sample of the schedule's (step, layer) rows: the rows are grouped by
+the number of chunks they recompute and the next row always comes from the group that is furthest
+behind its share, so any number of steps sees the schedule's mix of cheap and expensive rows and
+``value`` does not depend on ``--steps``.
 
 Prints ONE JSON line: ms per layer call plus
   * ``roofline``        the fresh-chunk attention kernel against the bf16 dense MFMA peak,
@@ -135,15 +135,29 @@ def sample_clock_mhz(fn, seconds=2.0):
 
 
 def stratified_order(counts):
-    """A fixed visiting order of the schedule rows in which every prefix has (nearly) the whole
-    schedule's distribution of ``counts``: rows sorted by count, visited with a stride of about
-    1/golden-ratio of their number (coprime with it)."""
-    order = sorted(range(len(counts)), key=lambda i: (counts[i], i))
-    m = len(order)
-    stride = max(1, int(m * 0.6180339887))
-    while math.gcd(stride, m) != 1:
-        stride += 1
-    return [order[(j * stride) % m] for j in range(m)]
+    """A fixed visiting order of the schedule rows in which every prefix has (as nearly as whole rows allow)
+    the whole schedule's distribution of ``counts``: the rows are grouped by count, and the next row always
+    comes from the group that is furthest behind its share of the schedule (ties: the group nearest the
+    mean); inside a group the rows are taken with a stride of about 1/golden-ratio of its size."""
+    groups = {}
+    for i, c in enumerate(counts):
+        groups.setdefault(c, []).append(i)
+    m = len(counts)
+    mean = sum(counts) / max(m, 1)
+    for c, rows in groups.items():
+        n = len(rows)
+        stride = max(1, int(n * 0.6180339887))
+        while math.gcd(stride, n) != 1:
+            stride += 1
+        groups[c] = [rows[(j * stride) % n] for j in range(n)]
+    taken = {c: 0 for c in groups}
+    order = []
+    for j in range(m):
+        best = max((c for c in groups if taken[c] < len(groups[c])),
+                   key=lambda c: (len(groups[c]) / m * (j + 1) - taken[c], -abs(c - mean)))
+        order.append(groups[best][taken[best]])
+        taken[best] += 1
+    return order
 
 
 def cpu_baseline(B, H, D, Sq, lens, mean_computed, n_chunks, norm, budget_s=20.0):
