@@ -63,3 +63,46 @@ def test_sched_attention_and_merge_replay_in_a_graph(hip):
         assert torch.equal(graphed["out"], eager["out"]) and torch.equal(graphed["lse"], eager["lse"]), f"replay {t}"
         assert torch.equal(graphed["arena_o"], eager["arena_o"]) and torch.equal(graphed["arena_l"], eager["arena_l"])
     assert np.array_equal(comp.cpu().numpy(), ms.build_schedule_table(mask, diag)[0])
+
+
+def test_noalloc_attention_replays_in_a_graph(hip):
+    """The allocation-free entry point under capture: the attention launch (with its tail split inside the
+    library's own scratch array and the fold kernel behind it) plus the merge, replayed four times
+    while K/V drift, against the same launches made eagerly through the workspace entry point."""
+    B, H, D, Sq, lens = 1, 24, 128, 3000, [2000, 1500]        # 2 x 288 work items: a tail of 64 is split
+    dev = "cuda"
+    g = torch.Generator(device=dev).manual_seed(21)
+    q = torch.randn(B, Sq, H, D, generator=g, device=dev).bfloat16()
+    ks = [torch.randn(B, n, H, D, generator=g, device=dev).bfloat16() for n in lens]
+    vs = [torch.randn(B, n, H, D, generator=g, device=dev).bfloat16() for n in lens]
+    table = hip.ChunkTable(ks, vs)
+    jobs = [[0], [1]]
+    ws = torch.empty(hip.DT_NOALLOC_TAIL_SLOTS * (256 * 128 * 2 + 256 * 4), dtype=torch.uint8, device=dev)
+
+    def buffers():
+        return dict(o=[torch.zeros(B, Sq, H, D, dtype=torch.bfloat16, device=dev) for _ in jobs],
+                    l=[torch.zeros(B, H, Sq, device=dev) for _ in jobs],
+                    out=torch.zeros(B, Sq, H, D, device=dev), lse=torch.zeros(B, Sq, H, 1, device=dev))
+
+    def call(b, **how):
+        hip.attn_jobs_fwd(q, table, jobs, b["o"], b["l"], **how)
+        hip.merge_states(b["o"], b["l"], dst_out=b["out"], dst_lse=b["lse"])
+
+    eager, graphed, plain = buffers(), buffers(), buffers()
+    call(graphed, no_alloc=True)            # outside the capture: the scratch address is looked up here
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(graphed, no_alloc=True)
+    for step in range(4):
+        for k in ks + vs:
+            k.add_(0.01 * torch.randn_like(k))
+        call(eager, workspace=ws)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(graphed["out"], eager["out"]) and torch.equal(graphed["lse"], eager["lse"]), f"replay {step}"
+        assert all(torch.equal(a, b) for a, b in zip(graphed["o"], eager["o"]))
+    call(plain)
+    torch.cuda.synchronize()
+    assert any(not torch.equal(a, b) for a, b in zip(graphed["o"], plain["o"])), "the tail was expected to be split"
