@@ -60,15 +60,18 @@ def _cmp(out, lse_bsh1, ref_out, ref_lse_bhs, what):
     assert err <= OUT_TOL and lerr <= LSE_TOL and rel <= 1e-2, what
 
 
-@pytest.mark.parametrize("N,rank,D,col", [
-    (4, 1, 128, (1, 1, 1, 2, 2, 2, 1, 4, 2, 2, 1, 1)),     # includes the stride-1 -> 2 misalignment
-    (8, 3, 64, (1, 1, 1, 4, 4, 4, 2, 2, 2, 2, 1, 1)),
-    (8, 0, 128, (1, 1, 1, 8, 8, 4, 4, 2, 1, 8, 1, 1)),
+@pytest.mark.parametrize("N,rank,D,col,max_job_chunks", [
+    (4, 1, 128, (1, 1, 1, 2, 2, 2, 1, 4, 2, 2, 1, 1), None),     # includes the stride-1 -> 2 misalignment
+    (8, 3, 64, (1, 1, 1, 4, 4, 4, 2, 2, 2, 2, 1, 1), None),
+    (8, 0, 128, (1, 1, 1, 8, 8, 4, 4, 2, 1, 8, 1, 1), None),
+    # the same with blocks of more than 3 chunks computed in pieces that are folded into the block's state
+    # (what a ring of 128 positions and more needs at the real limit of 32 chunks per job)
+    (8, 5, 128, (1, 1, 1, 4, 4, 2, 2, 2, 1, 2, 1, 1), 3),
     # a ring of 64 positions (strides 64 / 32 / 16 / 8, two-level ring above 8): a full-stride step that
     # announces stride 8 files 64 fine-grained states, more than one merge launch or chunk table holds
-    (64, 37, 64, (1, 1, 1, 8, 8, 4, 4, 2, 1, 8, 1, 1)),
+    (64, 37, 64, (1, 1, 1, 8, 8, 4, 4, 2, 1, 8, 1, 1), None),
 ])
-def test_stride_mode_matches_numeric_oracle(env, N, rank, D, col):
+def test_stride_mode_matches_numeric_oracle(env, N, rank, D, col, max_job_chunks):
     from ditango_amd.core.attention import proAttention
     from ditango_amd.core.parallel_state import get_usp_group
     from ditango_amd.utils import update_timestep
@@ -99,6 +102,8 @@ def test_stride_mode_matches_numeric_oracle(env, N, rank, D, col):
 
     ring = RingOracle(N, attn_fn=attn_fn, merge_fn=merge_fn, store_fn=store_fn)
     attn = proAttention(0, get_usp_group())
+    if max_job_chunks is not None:
+        attn._MAX_JOB_CHUNKS = max_job_chunks
     group = get_usp_group()
     for t in range(T):
         print(f"case stride N={N} rank={rank} D={D} t={t} curr={curr[t]} next={nxt[t]}", flush=True)
