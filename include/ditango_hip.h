@@ -213,7 +213,7 @@ int dt_attn_sched_seg_ws_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, in
  * scratch need does not grow with the input and no shape is turned away on its account; a plan
  * that does not fit is refused with DT_ERR_INVALID instead of being launched.  The call makes no
  * hipMalloc / hipFree; the array's device address is looked up once per device on the first call
- * there.  All calls on one GPU share the array: calls that overlap in time on one GPU (different
+ * there (hipGetSymbolAddress: make that first call outside a graph capture).  All calls on one GPU share the array: calls that overlap in time on one GPU (different
  * streams or threads) race on it; order them on one stream.  Nothing in the array has to start at
  * zero (every partial state that is read was written by the same call).
  */
