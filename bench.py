@@ -528,6 +528,12 @@ def main():
         sys.exit(2)
 
     from ditango_amd import _hip
+    from ditango_amd.logger import init_logger
+    import logging
+    init_logger("bench")
+    for h in logging.getLogger("ditango_amd").handlers:     # stdout carries the one JSON line only
+        if isinstance(h, logging.StreamHandler) and not isinstance(h, logging.FileHandler):
+            h.setStream(sys.stderr)
     _hip.load_library()
     torch.cuda.set_device(0)
     global PROFILING
