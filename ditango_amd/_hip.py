@@ -36,6 +36,8 @@ _SIGNATURES = {
     "dt_last_error": (ctypes.c_char_p, []),
     "dt_attn_chunk_fwd": (ctypes.c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_i32,
                                          c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_f32, c_vp]),
+    "dt_attn_chunk_f32_fwd": (ctypes.c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_i32,
+                                             c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_f32, c_vp]),
     "dt_attn_jobs_fwd": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i64, c_i64, c_i64,
                                         c_i32, _P(c_vp), _P(c_vp), _P(c_i32), _P(c_i64), c_i64, c_i64,
                                         c_i32, _P(c_i32), _P(c_i32), _P(c_vp), _P(c_vp), c_f32, c_vp]),
@@ -176,6 +178,25 @@ def attn_chunk_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_sc
                                B, Sq, Sk, H, D, q.stride(0), q.stride(1), q.stride(2),
                                k.stride(0), k.stride(1), k.stride(2), float(softmax_scale), _stream())
     _check(rc, "dt_attn_chunk_fwd")
+    return out, lse
+
+
+def attn_chunk_f32_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_scale: float = 0.0):
+    """(out fp32 [B,Sq,H,D], lse fp32 [B,H,Sq]) of fp32 q against one fp32 KV chunk, computed in fp32."""
+    lib = load_library()
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        _require(t.is_cuda and t.dtype == torch.float32 and t.dim() == 4 and t.stride(-1) == 1,
+                 f"{name} must be fp32 [B,S,H,D] on the GPU with contiguous D")
+    B, Sq, H, D = q.shape
+    Sk = k.shape[1]
+    _require(k.shape == v.shape and k.shape[0] == B and k.shape[2] == H and k.shape[3] == D, "k/v shape mismatch")
+    _require(k.stride() == v.stride(), "k and v must share strides")
+    out = torch.empty((B, Sq, H, D), dtype=torch.float32, device=q.device)
+    lse = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device)
+    rc = lib.dt_attn_chunk_f32_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
+                                   B, Sq, Sk, H, D, q.stride(0), q.stride(1), q.stride(2),
+                                   k.stride(0), k.stride(1), k.stride(2), float(softmax_scale), _stream())
+    _check(rc, "dt_attn_chunk_f32_fwd")
     return out, lse
 
 

@@ -18,7 +18,7 @@ ROOT = PKG.parent
 CSRC = PKG / "csrc"
 LIB_DIR = PKG / "lib"
 LIB_PATH = LIB_DIR / "libditango_hip.so"
-SOURCES = ["attn_fwd.hip", "state_ops.hip", "producer.hip", "capi.hip"]
+SOURCES = ["attn_fwd.hip", "attn_f32.hip", "state_ops.hip", "producer.hip", "capi.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 COMMON = [
@@ -49,7 +49,7 @@ def build_lib(verbose: bool = False, extra_flags=()) -> Path:
         _run(cmd)
         return obj
 
-    with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as ex:
+    with ThreadPoolExecutor(max_workers=min(5, len(SOURCES))) as ex:
         objs = list(ex.map(compile_one, SOURCES))
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objs), "-o", str(LIB_PATH)]
     if verbose:

@@ -197,6 +197,12 @@ class proAttention:
         # kernels then skip the scaling (a quarter of the softmax's vector instructions).  Not what the
         # reference's callers pass (flash_attn_func scales inside, core/attention.py:137-143).
         self.q_prescaled = False
+        # What happens to fp32 inputs (flash_attn_func takes none; the reference's CPU-runnable configuration is
+        # stated in fp32): "round" = rounded to bf16 at the kernel boundary, the bf16 MFMA kernels run;
+        # "exact" = every fresh state is computed in fp32 from the fp32 tensors (dt_attn_chunk_f32_fwd, a
+        # plain vector-ALU kernel for small problems) and only cached states are rounded to bf16.
+        self.fp32_inputs = "round"
+        self._exact_f32 = False
         self._segments = None  # (cu_seqlens_q, chunk -> cu_seqlens_kv) while a variable-length call runs
         if self.layer_id == 0:
             logger.info(f"R{self.global_rank}L{layer_id} | cached block attention on HIP kernels (gfx950)")
@@ -213,10 +219,12 @@ class proAttention:
         """query ``[B,Sq,H,D]``, key/value ``[B,Sk,H,D]`` = this rank's shard (bf16).
         Returns fp32 ``[B,Sq,H,D]`` (core/attention.py:74-237)."""
         rm = get_redundancy_map()
-        if not self.dry_run:
+        self._exact_f32 = (not self.dry_run and self.fp32_inputs == "exact" and query is not None
+                           and query.dtype == torch.float32)
+        if not self.dry_run and not self._exact_f32:
             query, key, value = _kernel_input(query), _kernel_input(key), _kernel_input(value)
         if rm is not None and rm.chunk_mask is not None and not self.dry_run:
-            return self._attn_masked(query, key, value)
+            return self._attn_masked_f32(query, key, value) if self._exact_f32 else self._attn_masked(query, key, value)
         timestep = get_timestep()
         N, r = self.isp_size, self.local_chunk_id
         curr, nxt = self._strides(timestep)
@@ -285,10 +293,42 @@ class proAttention:
         else:
             cache.update_cache_blocks(nxt, next_target_block)
 
+    def _chunk_f32(self, c: int, key, value, B: int):
+        """fp32 K/V of chunk ``c`` as ``[B,S,H,D]`` (exact-fp32 mode: no rounding)."""
+        k_c, v_c = (key, value) if (c == self.local_chunk_id and key is not None) else self.group.kv_chunk(c)
+        if k_c.dtype != torch.float32 or v_c.dtype != torch.float32:
+            raise TypeError("fp32_inputs = 'exact' needs fp32 K/V chunks as well")
+        k_c = k_c if k_c.dim() == 4 else k_c.view(B, k_c.shape[0] // B, k_c.shape[1], k_c.shape[2])
+        v_c = v_c if v_c.dim() == 4 else v_c.view(B, v_c.shape[0] // B, v_c.shape[1], v_c.shape[2])
+        return k_c, v_c
+
+    def _job_state_f32(self, query, chunks, key, value):
+        """The fp32 state of ``query`` against the concatenation of ``chunks``, computed in fp32."""
+        if self._segments is not None:
+            raise NotImplementedError("fp32_inputs = 'exact' does not cover variable-length calls")
+        B = query.shape[0]
+        states = [_hip.attn_chunk_f32_fwd(query, *self._chunk_f32(c, key, value, B)) for c in chunks]
+        if len(states) == 1:
+            return states[0]
+        return _hip.merge_states([s[0] for s in states], [s[1] for s in states], dst_dtype=torch.float32)
+
     def _execute(self, plan: CallPlan, query, key, value, merge_outs, merge_lses, segments=None) -> torch.Tensor:
         B, Sq, H, D = query.shape
         N, r = self.isp_size, self.local_chunk_id
         dev = query.device
+        if self._exact_f32:
+            seen = {}
+            for job in plan.jobs:
+                if job.chunks not in seen:
+                    seen[job.chunks] = self._job_state_f32(query, job.chunks, key, value)
+                o, l = seen[job.chunks]
+                if job.store_slot is not None:
+                    self.cache.store_block(job.store_slot, o, l)      # rounded to bf16 on its way into the cache
+                merge_outs.append(o)
+                merge_lses.append(l)
+            out, lse = _hip.merge_states(merge_outs, merge_lses, dst_dtype=self.out_dtype, dst_lse_bsh=True)
+            self.last_lse = lse
+            return out
         # chunk table: the local chunk is (key, value); the others come from the ring stand-in
         needed = sorted({c for job in plan.jobs for c in job.chunks})
         ks: List[torch.Tensor] = []
@@ -409,6 +449,36 @@ class proAttention:
                     cache.arena_valid[c] = True
                 outs.append(cache.arena_out[c])
                 lses.append(cache.arena_lse[c])
+        out, lse = _hip.merge_states(outs, lses, dst_dtype=self.out_dtype, dst_lse_bsh=True)
+        self.last_lse = lse
+        rm.record_out_redundancy(timestep=t, layer_id=l, curr_out=out)
+        return out
+
+    def _attn_masked_f32(self, query, key, value) -> torch.Tensor:
+        """Mask mode on fp32 tensors in exact mode: fresh states in fp32, cached ones bf16 in the arena."""
+        rm = get_redundancy_map()
+        t, l = get_timestep(), self.layer_id
+        C, diag = rm.chunk_mask.shape[2], rm.mask_diag
+        B, Sq, H, D = query.shape
+        cache = self.cache
+        row = rm.chunk_mask[t, l]
+        have_arena = cache.ensure_arena(C, B, Sq, H, D, query.device)
+        compute = ([diag] if 0 <= diag < C else []) + [c for c in range(C) if c != diag and (row[c] == 0 or not have_arena)]
+        outs, lses = [], []
+        for c in range(C):
+            if c in compute:
+                continue
+            if not cache.arena_valid[c]:
+                raise RuntimeError(f"T{t}L{l}: mask asks to reuse chunk {c} but no state was ever stored for it")
+            outs.append(cache.arena_out[c])
+            lses.append(cache.arena_lse[c])
+        for c in compute:
+            o, s = self._job_state_f32(query, (c,), key if c == diag else None, value if c == diag else None)
+            if c != diag and have_arena:
+                _hip.cache_store(o, s, cache.arena_out[c], cache.arena_lse[c])
+                cache.arena_valid[c] = True
+            outs.append(o)
+            lses.append(s)
         out, lse = _hip.merge_states(outs, lses, dst_dtype=self.out_dtype, dst_lse_bsh=True)
         self.last_lse = lse
         rm.record_out_redundancy(timestep=t, layer_id=l, curr_out=out)

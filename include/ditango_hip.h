@@ -75,6 +75,21 @@ int dt_attn_chunk_fwd(const void* q, const void* k, const void* v, void* out, fl
                       float softmax_scale, void* stream);
 
 /*
+ * The same for fp32 tensors, computed in fp32 throughout (vector ALU, expf / logf): the attention
+ * of the fp32 numbers themselves, not of their bf16 roundings.  flash_attn_func takes no fp32; the
+ * reference runs its CPU-runnable configuration (fp32, B=1, H=4, d=64, 512 queries x 4 chunks of
+ * 512 keys) on its torch math path, and this entry point is that path's counterpart here.  q / k / v
+ * fp32 with element strides and a contiguous last dimension; out fp32 [B,Sq,H,D] contiguous, lse
+ * fp32 [B,H,Sq].  Sk = 0 yields out = 0, lse = -inf.  Not tuned (about 1 TFLOP/s): model-sized
+ * bf16 work belongs on dt_attn_chunk_fwd.
+ */
+int dt_attn_chunk_f32_fwd(const float* q, const float* k, const float* v, float* out, float* lse,
+                          int32_t B, int32_t Sq, int32_t Sk, int32_t H, int32_t D,
+                          int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
+                          int64_t kv_stride_b, int64_t kv_stride_s, int64_t kv_stride_h,
+                          float softmax_scale, void* stream);
+
+/*
  * Several attention states in one launch.  Job j attends q to the
  * concatenation of the chunks job_chunks[job_begin[j] .. job_begin[j+1]) and
  * writes ONE state (out_ptrs[j], lse_ptrs[j]).  A job of one chunk is the call

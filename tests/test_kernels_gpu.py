@@ -64,6 +64,37 @@ def test_chunk_attention_matches_oracle(hip, B, Sq, Sk, H, D):
     _check_state(out, lse, ref_out, ref_lse, "chunk")
 
 
+@pytest.mark.parametrize("B,Sq,Sk,H,D", [
+    (1, 512, 512, 4, 64),      # the CPU-runnable configuration's chunk
+    (2, 100, 77, 3, 128),      # ragged queries and keys, batch > 1
+    (1, 1, 1, 1, 64),
+    (1, 65, 130, 2, 128),
+    (1, 33, 0, 2, 64),         # empty chunk: out = 0, lse = -inf
+])
+def test_fp32_chunk_attention_matches_fp64_closed_form(hip, B, Sq, Sk, H, D):
+    """dt_attn_chunk_f32_fwd computes in fp32 from fp32 inputs: it must agree with the closed form in
+    fp64 to fp32 rounding error (1e-5), far inside the bar of the bf16 path."""
+    g = torch.Generator().manual_seed(Sq * 7 + Sk)
+    q = torch.randn(B, Sq, H, D, generator=g) * 1.5
+    k = torch.randn(B, Sk, H, D, generator=g)
+    v = torch.randn(B, Sk, H, D, generator=g)
+    ref_out, ref_lse = om.chunk_attention(q, k, v, compute_dtype=torch.float64)
+    out, lse = hip.attn_chunk_f32_fwd(q.cuda(), k.cuda(), v.cuda())
+    torch.cuda.synchronize()
+    assert out.dtype == torch.float32 and tuple(lse.shape) == (B, H, Sq)
+    if Sk == 0:
+        assert (out == 0).all() and torch.isinf(lse).all() and (lse < 0).all()
+        return
+    assert (out.double().cpu() - ref_out).abs().max().item() <= 1e-5
+    assert (lse.double().cpu() - ref_lse).abs().max().item() <= 1e-5
+    # strided inputs (slices of a fused projection) give the same numbers
+    qkv = torch.stack([q, k[:, :Sq] if Sk >= Sq else q, q], dim=2).cuda() if Sk >= Sq else None
+    if qkv is not None:
+        out2, lse2 = hip.attn_chunk_f32_fwd(qkv[:, :, 0], k.cuda(), v.cuda())
+        torch.cuda.synchronize()
+        assert torch.equal(out2, out) and torch.equal(lse2, lse)
+
+
 def test_chunk_attention_strided_inputs(hip):
     """q/k/v as slices of a fused [B,S,3,H,D] projection (non-contiguous token stride)."""
     B, S, H, D = 1, 300, 2, 128
