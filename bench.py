@@ -465,6 +465,36 @@ def run_workload(name, args, steps, warmup, main, reuse=None, kernels_only=False
         kp_bytes = B * S_all * H * D * 4 + S_all * D * 8
         kp_gbs = kp_bytes / (kp_ms * 1e-3) / 1e9
         del qkv, ang, p_cos, p_sin, p_out
+        # the variable-length entry (HunyuanVideo's real one: two segments per sample, the valid tokens and the
+        # padded text tokens, core/attention.py:239-419) on the same schedule rows: every scheduled chunk runs
+        # once per segment inside one launch
+        pad_rows = 64
+        cu = [0, Sq - pad_rows, Sq]
+        group.set_kv_chunks(ks, vs, cu_seqlens_kv=[[0, n - pad_rows, n] for n in lens])
+        q3, k3, v3 = q.view(B * Sq, H, D), ks[rank].view(B * lens[rank], H, D), vs[rank].view(B * lens[rank], H, D)
+        cu_t = torch.tensor(cu, dtype=torch.int32)
+        cu_kv_t = torch.tensor([0, lens[rank] - pad_rows, lens[rank]], dtype=torch.int32)
+        n_var = 1 if kernels_only else min(24, len(timed))
+
+        def run_varlen(t, l):
+            update_timestep(t)
+            return layers[l].varlen_attn(q3, k3, v3, cu_t, cu_kv_t, Sq - pad_rows, max(lens) - pad_rows)
+
+        for t, l in timed[:2]:
+            run_varlen(t, l)
+        torch.cuda.synchronize()
+        t0v = time.perf_counter()
+        for t, l in timed[:n_var]:
+            run_varlen(t, l)
+        torch.cuda.synchronize()
+        var_ms = 1e3 * (time.perf_counter() - t0v) / n_var
+        var_chunks = float(np.mean(n_comp[:n_var]))
+        var_flops = 4.0 * H * D * ((Sq - pad_rows) * (Sk_mean - pad_rows) + pad_rows * pad_rows) * B * var_chunks
+        group.set_kv_chunks(ks, vs)
+        # profiling mode: the relative-L1 sums of two fp32 outputs (record_out_redundancy, utils.py:202-267)
+        sums = torch.zeros(4, dtype=torch.float64, device=dev)
+        kl_ms = time_kernel(Rotation(lambda i: _hip.rel_l1_sums(dst_os[i % dst_n], dst_os[(i + 1) % dst_n], sums), dst_n), reps)
+        kl_gbs = 2 * rows * D * 4 / (kl_ms * 1e-3) / 1e9
         dmask = torch.from_numpy(mask).to(dev)
         k4_ms = time_kernel(lambda: _hip.build_schedule_table(dmask, diag), reps)
         # a plain copy of known size: the yardstick the profiler's FETCH_SIZE / WRITE_SIZE counters are scaled by
@@ -486,6 +516,13 @@ def run_workload(name, args, steps, warmup, main, reuse=None, kernels_only=False
                          "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(kp_gbs / PEAK_HBM_GBS, 4),
                          "launch_us": round(kp_ms * 1e3, 2), "bytes_per_launch": kp_bytes, "tokens": S_all,
                          "what": "RMSNorm + interleaved RoPE of K over the whole KV sequence, strided read from a fused QKV tensor"},
+            "varlen": {"what": f"proAttention.varlen_attn, two segments per sample ({Sq - pad_rows} + {pad_rows} query rows; "
+                               f"{lens[0] - pad_rows} + {pad_rows} keys per chunk), same schedule rows",
+                       "ms_per_layer": round(var_ms, 4), "calls": n_var, "mean_chunks_computed_per_call": round(var_chunks, 3),
+                       "layer_attn_tflops": round(var_flops / (var_ms * 1e-3) / 1e12, 1)},
+            "rel_l1": {"kernel": "rel_l1_sums_kernel", "bound": "hbm", "achieved": round(kl_gbs, 1), "peak": PEAK_HBM_GBS,
+                       "unit": "GB/s", "frac": round(kl_gbs / PEAK_HBM_GBS, 4), "launch_us": round(kl_ms * 1e3, 2),
+                       "bytes_per_launch": 2 * rows * D * 4},
             "schedule_builder_us": round(k4_ms * 1e3, 2),
             "plain_copy_1GiB_gbs": round(copy_gbs, 1),
         }
