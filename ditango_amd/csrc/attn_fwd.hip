@@ -602,6 +602,16 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
     cp_left -= kBK;
     if (cp_left <= 0) cp_next_chunk();
   }
+  // Behind this barrier the leading group computes the scores of tile 1, so K of tile 1 has to be in
+  // the LDS from ALL wavefronts.  The leading group waits for its share at the end of its vector
+  // phase; the trailing group is in its score-only phase here and has no vector phase in between,
+  // so it waits for its share now (of its 8 kLoads loads, the 4 kLoads oldest: V(-1), K0, V0, K1).
+  // From tile 2 on, the wait that ends a group's vector phase covers the tile the other group
+  // reads next.
+  if (group == 1) {
+    if constexpr (T::kLoads == 2) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+  }
   phase_barrier_after_matrix(s_acc, o_acc);
 
   // one iteration = vector phase of tile t, then matrix phase (P V of tile t, scores of t+1)

@@ -313,3 +313,45 @@ def test_chunk_attention_with_drifting_maximum(hip, case):
     print(f"{case}: out max-abs {err:.3e}, lse max rel/abs {lerr:.3e}, lse range [{ref_lse.min():.1f}, {ref_lse.max():.1f}]", flush=True)
     assert err <= OUT_TOL
     assert lerr <= LSE_TOL
+
+
+@pytest.mark.parametrize("D", [128, 64])
+def test_short_work_items_repeat_bit_exactly(hip, D):
+    """Work items of two key tiles, many per launch, many launches on K/V just copied in from the host: every launch
+    must return the bits of the first one, and the first one the oracle's numbers.
+
+    With two tiles the trailing half of a workgroup has no softmax phase of its own before the leading
+    half reads K of the second tile, so its share of that tile needs a wait of its own: the loads were
+    issued long before and nearly always land in time, which is why only repetition shows a missing one
+    (some rows of one head lose a few per cent of their softmax mass, about once in 40 000 work items)."""
+    B, Sq, H, Sk, n_chunks, launches = 1, 90, 3, 90, 40, 2500
+    g = torch.Generator().manual_seed(90 + D)
+    q = torch.randn(B, Sq, H, D, generator=g).bfloat16()
+    k_all = torch.randn(n_chunks, B, Sk, H, D, generator=g).bfloat16()
+    v_all = torch.randn(n_chunks, B, Sk, H, D, generator=g).bfloat16()
+    dq = q.cuda()
+    jobs = [[c] for c in range(n_chunks)]
+
+    def launch():
+        dk, dv = k_all.cuda(), v_all.cuda()      # copied by the DMA engine: in no cache of the GPU, new addresses
+        table = hip.ChunkTable(list(dk.unbind(0)), list(dv.unbind(0)))
+        out = torch.empty(n_chunks, B, Sq, H, D, dtype=torch.bfloat16, device="cuda")
+        lse = torch.empty(n_chunks, B, H, Sq, dtype=torch.float32, device="cuda")
+        hip.attn_jobs_fwd(dq, table, jobs, list(out.unbind(0)), list(lse.unbind(0)))
+        return out, lse, (dk, dv)
+
+    out0, lse0, _ = launch()
+    torch.cuda.synchronize()
+    for c in (0, 17, n_chunks - 1):
+        ref_out, ref_lse = om.chunk_attention(q, k_all[c], v_all[c])
+        _check_state(out0[c], lse0[c], ref_out, ref_lse, f"chunk {c}")
+    differing = torch.zeros((), dtype=torch.int64, device="cuda")
+    keep = []                                                   # a few generations stay allocated: addresses vary
+    for i in range(launches):
+        out, lse, kv = launch()
+        differing += ((out != out0).flatten(1).any(1) | (lse != lse0).flatten(1).any(1)).sum()
+        keep.append(kv)
+        if len(keep) > (i % 7) + 1:
+            keep.clear()
+    torch.cuda.synchronize()
+    assert int(differing) == 0, f"{int(differing)} chunk states of {launches * n_chunks} differ from the first launch"
