@@ -363,8 +363,21 @@ def run_workload(name, args, steps, warmup, main, reuse=None, kernels_only=False
     k1p_ms = time_kernel(lambda: k1_launch(n_typ, q_folded, True), reps)
     k1p_tflops = k1_flops(n_typ) / (k1p_ms * 1e-3) / 1e12
     clock = None
+    mfma_probe = None
     if main and not kernels_only:
         clock = sample_clock_mhz(lambda: k1_launch(n_typ))
+        # the yardstick: back-to-back MFMAs on registers in the same launch shape, sized to last about as long
+        # as the typical launch -- what the power limit leaves of the nominal peak when only the matrix pipes work
+        probe_sink = torch.zeros(1, dtype=torch.float32, device=dev)
+        probe_wgs, probe_iters = 256 * 8, 8192
+        probe_flops = [0.0]
+
+        def probe_launch():
+            probe_flops[0] = _hip.mfma_probe(probe_wgs, probe_iters, probe_sink)
+
+        kp_ms = time_kernel(probe_launch, reps)
+        mfma_probe = {"tflops": round(probe_flops[0] / (kp_ms * 1e-3) / 1e12, 1), "launch_ms": round(kp_ms, 4),
+                      "clock_mhz_under_load": sample_clock_mhz(probe_launch, seconds=1.5)}
     del q_folded
 
     # merge of all C states of a layer into the fp32 result, rotating over the layers' arenas
@@ -424,6 +437,10 @@ def run_workload(name, args, steps, warmup, main, reuse=None, kernels_only=False
         # the part is power-limited under this kernel: what the kernel reaches of the peak AT THE CLOCK IT RUNS AT
         roofline["clock_mhz_under_load"] = clock
         roofline["frac_at_clock"] = round(frac * NOMINAL_CLOCK_MHZ / clock, 4)
+    if mfma_probe:
+        roofline["mfma_probe_tflops"] = mfma_probe["tflops"]
+        roofline["mfma_probe_clock_mhz"] = mfma_probe["clock_mhz_under_load"]
+        roofline["frac_of_mfma_probe"] = round(k1_tflops / mfma_probe["tflops"], 4)
     roofline_merge = {"kernel": "merge_states_kernel<%d>" % D, "bound": "hbm", "achieved": round(k2_gbs, 1),
                       "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(k2_gbs / PEAK_HBM_GBS, 4),
                       "traffic": k2_traffic, "launch_us": round(k2_ms * 1e3, 2), "bytes_per_launch": k2_bytes,

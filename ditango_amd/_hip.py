@@ -74,6 +74,7 @@ _SIGNATURES = {
     "dt_build_schedule": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp, c_vp]),
     "dt_build_schedule_table": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp, c_vp]),
     "dt_hbm_read_probe": (ctypes.c_int, [_P(c_vp), c_i32, c_i64, c_vp, c_vp]),
+    "dt_mfma_probe": (ctypes.c_int, [c_i32, c_i32, c_vp, c_vp]),
     "dt_rel_l1_sums": (ctypes.c_int, [c_vp, c_vp, c_i64, c_vp, c_vp]),
     "dt_qk_norm_rope": (ctypes.c_int, [c_vp, c_i64, c_i64, c_i64, c_vp, c_i32, c_i32, c_i32, c_i32,
                                        c_i32, c_vp, c_vp, c_f32, c_i32, c_vp, c_vp, c_i64, c_i32, c_i32,
@@ -549,6 +550,16 @@ def hbm_read_probe(buffers: Sequence[torch.Tensor], sink: torch.Tensor) -> None:
     ptrs = (c_vp * n)(*[b.data_ptr() for b in buffers])
     rc = lib.dt_hbm_read_probe(ptrs, n, nbytes // 256 * 256, sink.data_ptr(), _stream())
     _check(rc, "dt_hbm_read_probe")
+
+
+def mfma_probe(workgroups: int, iters: int, sink: torch.Tensor) -> float:
+    """Launch the register-only MFMA loop (the sustained-rate yardstick of the attention kernel) and return
+    the FLOP the launch performs: ``workgroups * 8`` wavefronts x ``4 * iters`` bf16 MFMAs of 32 x 32 x 16."""
+    lib = load_library()
+    _require(sink.is_cuda and sink.numel() * sink.element_size() >= 4, "sink must be a device tensor of at least 4 bytes")
+    rc = lib.dt_mfma_probe(int(workgroups), int(iters), sink.data_ptr(), _stream())
+    _check(rc, "dt_mfma_probe")
+    return float(workgroups) * 8 * 4 * iters * 32768.0
 
 
 def rel_l1_sums(a: torch.Tensor, b: torch.Tensor, sums: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -871,6 +871,44 @@ __global__ __launch_bounds__(256) void attn_tail_fold_kernel(const AttnArgs a) {
   }
 }
 
+// Measurement aid: back-to-back bf16 MFMAs on registers, nothing else -- the rate (and the shader
+// clock) this part sustains when only the matrix pipes work, i.e. what the power limit leaves of the
+// nominal peak.  Same launch shape as the attention kernel (512 threads, two wavefronts per SIMD).
+// Four accumulators keep four independent MFMAs in flight; the operands rotate through four register
+// sets of pseudo-random values so that the operand buses toggle as they do on real data.
+__global__ __launch_bounds__(kThreads, 2) void mfma_probe_kernel(float* sink, int iters) {
+  const uint32_t lane = threadIdx.x;
+  bf16x8 av[4], bv[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      uint32_t ha = (lane * 8u + e + 1u) * 2654435761u + j * 40503u;
+      uint32_t hb = (lane * 8u + e + 7u) * 2246822519u + j * 9973u;
+      ha ^= ha >> 15;
+      hb ^= hb >> 13;
+      av[j][e] = (__bf16)((float)(int)(ha & 255u) * (1.f / 128.f) - 1.f);
+      bv[j][e] = (__bf16)((float)(int)(hb & 255u) * (1.f / 128.f) - 1.f);
+    }
+  f32x16 acc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[j][r] = 0.f;
+  for (int i = 0; i < iters; i += 4) {   // iters is rounded up to a multiple of 4; register indices stay static
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[j], bv[(j + u) & 3], acc[j], 0, 0, 0);
+  }
+  float total = 0.f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) total += acc[j][r];
+  if (total == 12345.678f) sink[0] = total;   // keeps the MFMAs alive; (almost) never true
+}
+
 template <int D, bool kPre>
 static int launch_one(const AttnArgs& a, dim3 grid, hipStream_t stream) {
   // more than 64 KB of dynamic LDS has to be allowed once per kernel and device
@@ -1017,3 +1055,12 @@ int launch_attn(const AttnArgs& a_in, int D, int n_jobs, hipStream_t stream, voi
 }
 
 }  // namespace dt
+
+extern "C" int dt_mfma_probe(int32_t workgroups, int32_t iters, float* sink, void* stream) {
+  if (workgroups <= 0 || iters <= 0 || iters % 4 != 0 || !sink) {
+    dt::set_error("mfma probe: workgroups and iters must be positive, iters a multiple of 4, and sink non-null");
+    return DT_ERR_INVALID;
+  }
+  hipLaunchKernelGGL(dt::mfma_probe_kernel, dim3((unsigned)workgroups), dim3(dt::kThreads), 0, (hipStream_t)stream, sink, iters);
+  return dt::hip_fail(hipGetLastError(), "mfma_probe launch");
+}

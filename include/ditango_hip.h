@@ -313,6 +313,16 @@ int dt_rel_l1_sums(const float* a, const float* b, int64_t n, double* sums, void
 int dt_hbm_read_probe(const void* const* streams, int32_t n_streams, int64_t bytes, uint32_t* sink, void* stream);
 
 /*
+ * Measurement aid, no counterpart in the reference: `workgroups` workgroups of 8 wavefronts (two per
+ * SIMD, the attention kernel's launch shape) each issue 4 * iters (iters a multiple of 4) back-to-back
+ * v_mfma_f32_32x32x16_bf16 on registers -- 32768 FLOP apiece, so a launch does
+ * workgroups * 8 * 4 * iters * 32768 FLOP -- and nothing else.  Its rate is what the part sustains
+ * when only the matrix pipes work (the power limit holds the shader clock below nominal): the
+ * yardstick next to the nominal MFMA peak for dt_attn_*.  sink: one device word, (almost) never written.
+ */
+int dt_mfma_probe(int32_t workgroups, int32_t iters, float* sink, void* stream);
+
+/*
  * Producer side of an attention call: normalise every head row of x over D, apply the
  * rotary position embedding to the token rows [rope_begin, rope_end) and write the result
  * as bf16 [B,S,H,D] contiguous, the layout the attention entry points read -- one pass over

@@ -280,6 +280,16 @@ def test_read_probe_and_its_argument_checks(hip):
         hip.hbm_read_probe(bufs * 6, sink)                     # 66 streams: more than one launch takes
 
 
+def test_mfma_probe_runs_and_checks_its_arguments(hip):
+    sink = torch.zeros(1, dtype=torch.float32, device="cuda")
+    flop = hip.mfma_probe(64, 16, sink)
+    torch.cuda.synchronize()
+    assert flop == 64 * 8 * 4 * 16 * 32768.0 and float(sink) == 0.0
+    for bad in ((0, 16), (64, 0), (-1, 4), (64, 6)):
+        with pytest.raises(hip.DitangoHipError):
+            hip.mfma_probe(*bad, sink)
+
+
 def test_cache_load_into_given_tensors(hip):
     B, S, H, D = 1, 70, 2, 64
     g = torch.Generator().manual_seed(9)
