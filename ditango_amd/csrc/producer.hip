@@ -86,7 +86,7 @@ __global__ __launch_bounds__(kThreads) void qk_norm_rope_kernel(const PrepArgs a
   u32x4 raw[kHeads];
 #pragma unroll
   for (int r = 0; r < kHeads; ++r)
-    if (r < nh) raw[r] = *reinterpret_cast<const u32x4*>(xp + (int64_t)r * a.xs_h);
+    if (r < nh) raw[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(xp + (int64_t)r * a.xs_h));
 
   const bool do_rope = a.rope != DT_ROPE_NONE && s >= a.rope_begin && s < a.rope_end;
   float cs[8], sn[8];

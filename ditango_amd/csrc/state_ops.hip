@@ -9,6 +9,8 @@
 // (query, head) and moves 16 bytes of bf16 (8 elements) per lane per state, so a
 // row is one contiguous 128/256-byte access, and the lse values of consecutive
 // rows are consecutive floats in the [B,H,Sq] layout.
+#include <algorithm>
+
 #include "dt_common.h"
 
 namespace dt {
@@ -51,12 +53,12 @@ __device__ __forceinline__ Row8 load_row8(const void* base, bool fp32, int64_t r
   Row8 r;
   if (fp32) {
     const float* p = reinterpret_cast<const float*>(base) + row_elem + 4 * c;
-    r.lo = *reinterpret_cast<const u32x4*>(p);
-    r.hi = *reinterpret_cast<const u32x4*>(p + D / 2);
+    r.lo = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+    r.hi = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p + D / 2));
   } else {
     const uint16_t* p = reinterpret_cast<const uint16_t*>(base) + row_elem + 4 * c;
-    const u32x2 g0 = *reinterpret_cast<const u32x2*>(p);
-    const u32x2 g1 = *reinterpret_cast<const u32x2*>(p + D / 2);
+    const u32x2 g0 = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p));
+    const u32x2 g1 = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p + D / 2));
     r.lo.x = g0.x; r.lo.y = g0.y; r.lo.z = g1.x; r.lo.w = g1.y;
     r.hi = r.lo;
   }
@@ -157,8 +159,8 @@ __device__ __forceinline__ void load_batch(const MergeArgs& a, int i0, const int
         g.l[p][j] = lp[lse_index(bsh, b[p], h[p], s[p], a.H, a.Sq)];
         if (ALL_BF16) {
           const uint16_t* q = reinterpret_cast<const uint16_t*>(op) + elem[p] + 4 * cc;
-          const u32x2 g0 = *reinterpret_cast<const u32x2*>(q);
-          const u32x2 g1 = *reinterpret_cast<const u32x2*>(q + D / 2);
+          const u32x2 g0 = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(q));
+          const u32x2 g1 = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(q + D / 2));
           g.rb[p][j].x = g0.x; g.rb[p][j].y = g0.y; g.rb[p][j].z = g1.x; g.rb[p][j].w = g1.y;
         } else {
           g.r[p][j] = load_row8<D>(op, (a.fp32_mask >> i) & 1, elem[p], cc);
@@ -301,7 +303,7 @@ struct CopyArgs {
 };
 
 
-constexpr int kCopyRows = 2;  // rows per lane group, both in flight
+constexpr int kCopyRows = 1;  // rows per lane group (2 and 4 measured: -6 % and -12 %)
 
 template <int D>
 __global__ __launch_bounds__(kThreads) void state_copy_kernel(const CopyArgs a) {
@@ -337,34 +339,82 @@ __global__ __launch_bounds__(kThreads) void state_copy_kernel(const CopyArgs a) 
   }
 }
 
+// bf16 state -> fp32 state (a cache load): `out` is an elementwise widening in the same element order,
+// so it runs as a flat pass -- a lane takes 4 consecutive elements (8 bytes in, 16 bytes out), one
+// load and one store, both non-temporal (+5 % over the row-mapped kernel above in this direction; in
+// the narrowing direction the row-mapped kernel is the faster one by 5-13 %, so it keeps that).  The
+// workgroups in front of those of `out` (dispatched first, so that they run beside the streaming ones
+// instead of as a tail) move the lse: one run of `lse_run` query positions x all heads per workgroup,
+// read in the source's order, written in the destination's, through the LDS in between, so that
+// both sides are coalesced whichever way the [H][S] / [S][H] layouts differ.
+constexpr int kConvThreads = 256;
+
+__global__ __launch_bounds__(kConvThreads) void state_widen_kernel(const CopyArgs a, int64_t groups, uint32_t wgs_lse,
+                                                                   int lse_run) {
+  extern __shared__ float conv_lds[];   // [H][lse_run]
+  if (blockIdx.x >= wgs_lse) {
+    const int64_t g = (int64_t)(blockIdx.x - wgs_lse) * kConvThreads + threadIdx.x;   // 4 elements
+    if (g >= groups) return;
+    const u32x2 v = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(a.src_out) + g);
+    u32x4 o;
+    o.x = v.x << 16;
+    o.y = v.x & 0xffff0000u;
+    o.z = v.y << 16;
+    o.w = v.y & 0xffff0000u;
+    __builtin_nontemporal_store(o, reinterpret_cast<u32x4*>(a.dst_out) + g);
+    return;
+  }
+  const int runs = (a.Sq + lse_run - 1) / lse_run;
+  const int b = blockIdx.x / runs;
+  const int s0 = (blockIdx.x - b * runs) * lse_run;
+  const int ns = min(lse_run, a.Sq - s0);
+  const int n = ns * a.H;
+  // element i of the piece in a layout's own order -> (h, s)
+  auto decode = [&](bool bsh, int i, int& h, int& s) {
+    if (bsh) { s = i / a.H; h = i - s * a.H; }
+    else { h = i / ns; s = i - h * ns; }
+  };
+  for (int i = threadIdx.x; i < n; i += kConvThreads) {
+    int h, s;
+    decode(a.src_bsh != 0, i, h, s);
+    conv_lds[h * ns + s] = a.src_lse[lse_index(a.src_bsh != 0, b, h, s0 + s, a.H, a.Sq)];
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < n; i += kConvThreads) {
+    int h, s;
+    decode(a.dst_bsh != 0, i, h, s);
+    a.dst_lse[lse_index(a.dst_bsh != 0, b, h, s0 + s, a.H, a.Sq)] = conv_lds[h * ns + s];
+  }
+}
+
 // Same dtype and same lse layout on both sides: the state is two flat byte ranges (out, lse).  A
-// workgroup moves 16 KB: four 16-byte loads per lane, each instruction 1 KB contiguous per wavefront,
-// all in flight before the first store; non-temporal stores.
+// workgroup of 512 threads moves 8 KB: one 16-byte load per lane (1 KB contiguous per wavefront), both
+// the load and the store non-temporal.  Measured against 2 / 4 / 8 loads per lane in flight, 256 and
+// 1024 threads and grid-stride loops: more, simpler workgroups are the fastest copy on this part.
 struct FlatCopyArgs {
   const uint8_t* src[2];
   uint8_t* dst[2];
   int64_t bytes[2];   // multiples of 4
   uint32_t wgs0;      // workgroups of the first range
 };
+constexpr int kFlatThreads = 512;
+constexpr int kFlatWgBytes = kFlatThreads * 16;
 
-__global__ __launch_bounds__(kThreads) void flat_copy_kernel(const FlatCopyArgs a) {
+__global__ __launch_bounds__(kFlatThreads) void flat_copy_kernel(const FlatCopyArgs a) {
   const int which = blockIdx.x >= a.wgs0 ? 1 : 0;
   const int64_t wg = which ? blockIdx.x - a.wgs0 : blockIdx.x;
   const uint8_t* src = a.src[which];
   uint8_t* dst = a.dst[which];
   const int64_t bytes = a.bytes[which];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int64_t base = wg * 16384 + wave * 4096 + lane * 16;
+  const int64_t wave_base = wg * kFlatWgBytes + wave * 1024;
   const bool vec_ok = ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) == 0;
-  if (vec_ok && base - lane * 16 + 4096 <= bytes) {
-    u32x4 v[4];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) v[k] = *reinterpret_cast<const u32x4*>(src + base + k * 1024);
-#pragma unroll
-    for (int k = 0; k < 4; ++k) __builtin_nontemporal_store(v[k], reinterpret_cast<u32x4*>(dst + base + k * 1024));
+  if (vec_ok && wave_base + 1024 <= bytes) {
+    const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src + wave_base + lane * 16));
+    __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dst + wave_base + lane * 16));
   } else {
-    // the range's last, partial 4 KB (or a range that is not 16-byte aligned): 4 bytes at a time
-    for (int64_t off = wg * 16384 + wave * 4096 + lane * 4; off < bytes && off < wg * 16384 + (wave + 1) * 4096; off += 256)
+    // the range's last, partial 1 KB (or a range that is not 16-byte aligned): 4 bytes at a time
+    for (int64_t off = wave_base + lane * 4; off < bytes && off < wave_base + 1024; off += 256)
       *reinterpret_cast<uint32_t*>(dst + off) = *reinterpret_cast<const uint32_t*>(src + off);
   }
 }
@@ -413,8 +463,8 @@ __global__ __launch_bounds__(kThreads) void rel_l1_sums_kernel(const float* a, c
   for (int64_t i = ((int64_t)blockIdx.x * kThreads + threadIdx.x) * 4; i < n; i += stride) {
     float xa[4], xb[4];
     if (i + 4 <= n) {
-      const f32x4 va = *reinterpret_cast<const f32x4*>(a + i);
-      const f32x4 vb = *reinterpret_cast<const f32x4*>(b + i);
+      const f32x4 va = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(a + i));
+      const f32x4 vb = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(b + i));
       xa[0] = va.x; xa[1] = va.y; xa[2] = va.z; xa[3] = va.w;
       xb[0] = vb.x; xb[1] = vb.y; xb[2] = vb.z; xb[3] = vb.w;
     } else {
@@ -481,7 +531,7 @@ __global__ __launch_bounds__(kThreads) void hbm_read_probe_kernel(const ProbeArg
       for (int p = 0; p < 2; ++p) {
         const int64_t r = row + 16 * p;
         v[s][p] = u32x4{0u, 0u, 0u, 0u};
-        if (s0 + s < a.n && r < a.rows) v[s][p] = *reinterpret_cast<const u32x4*>(a.stream[s0 + s] + r * 256 + 16 * c);
+        if (s0 + s < a.n && r < a.rows) v[s][p] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(a.stream[s0 + s] + r * 256 + 16 * c));
       }
 #pragma unroll
     for (int s = 0; s < kBatch; ++s)
@@ -538,14 +588,33 @@ int launch_copy(const CopyArgs& a, int D, hipStream_t stream) {
     f.src[1] = reinterpret_cast<const uint8_t*>(a.src_lse);
     f.dst[1] = reinterpret_cast<uint8_t*>(a.dst_lse);
     f.bytes[1] = with_lse ? rows * 4 : 0;
-    const int64_t w0 = (f.bytes[0] + 16383) / 16384, w1 = (f.bytes[1] + 16383) / 16384;
+    const int64_t w0 = (f.bytes[0] + kFlatWgBytes - 1) / kFlatWgBytes, w1 = (f.bytes[1] + kFlatWgBytes - 1) / kFlatWgBytes;
     if (w0 + w1 > 0x7fffffffLL) {
       set_error("copy grid too large");
       return DT_ERR_INVALID;
     }
     f.wgs0 = (uint32_t)w0;
-    if (w0 + w1 > 0) hipLaunchKernelGGL(flat_copy_kernel, dim3((unsigned)(w0 + w1)), dim3(kThreads), 0, stream, f);
+    if (w0 + w1 > 0) hipLaunchKernelGGL(flat_copy_kernel, dim3((unsigned)(w0 + w1)), dim3(kFlatThreads), 0, stream, f);
     return hip_fail(hipGetLastError(), "flat_copy launch");
+  }
+  if (D != 64 && D != 128) {
+    set_error("head dim %d not built (64 and 128 are)", D);
+    return DT_ERR_UNSUPPORTED;
+  }
+  if (!a.src_fp32 && a.dst_fp32) {
+    const int64_t rows = (int64_t)a.B * a.Sq * a.H;
+    const int64_t groups = rows * D / 4;
+    const int64_t w_out = (groups + kConvThreads - 1) / kConvThreads;
+    const int lse_run = a.H <= 256 ? 64 : std::max(1, 16384 / a.H);   // at most 64 KB of LDS
+    const int64_t w_lse = with_lse ? (int64_t)a.B * ((a.Sq + lse_run - 1) / lse_run) : 0;
+    if (w_out + w_lse <= 0) return DT_OK;
+    if (w_out + w_lse > 0x7fffffffLL || (int64_t)lse_run * a.H * 4 > 65536) {
+      set_error("copy grid too large");
+      return DT_ERR_INVALID;
+    }
+    hipLaunchKernelGGL(state_widen_kernel, dim3((unsigned)(w_out + w_lse)), dim3(kConvThreads),
+                       with_lse ? (size_t)lse_run * a.H * 4 : 0, stream, a, groups, (uint32_t)w_lse, lse_run);
+    return hip_fail(hipGetLastError(), "state_widen launch");
   }
   const int rows_per_wg = kThreads / (D / 8) * kCopyRows;
   const int n_st = (a.Sq + rows_per_wg - 1) / rows_per_wg;
@@ -555,14 +624,8 @@ int launch_copy(const CopyArgs& a, int D, hipStream_t stream) {
     set_error("copy grid too large");
     return DT_ERR_INVALID;
   }
-  if (D == 128) {
-    hipLaunchKernelGGL(state_copy_kernel<128>, dim3((unsigned)wgs), dim3(kThreads), 0, stream, a);
-  } else if (D == 64) {
-    hipLaunchKernelGGL(state_copy_kernel<64>, dim3((unsigned)wgs), dim3(kThreads), 0, stream, a);
-  } else {
-    set_error("head dim %d not built (64 and 128 are)", D);
-    return DT_ERR_UNSUPPORTED;
-  }
+  if (D == 128) hipLaunchKernelGGL(state_copy_kernel<128>, dim3((unsigned)wgs), dim3(kThreads), 0, stream, a);
+  else hipLaunchKernelGGL(state_copy_kernel<64>, dim3((unsigned)wgs), dim3(kThreads), 0, stream, a);
   return hip_fail(hipGetLastError(), "state_copy launch");
 }
 

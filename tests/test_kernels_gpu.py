@@ -222,6 +222,23 @@ def test_cache_store_load_roundtrip(hip):
     assert torch.equal(l.cpu(), lse)
 
 
+@pytest.mark.parametrize("B,Sq,H,D", [(1, 1, 1, 64), (2, 131, 3, 64), (1, 64, 24, 128), (3, 700, 7, 128), (1, 65, 300, 64),
+                                      (2, 1000, 48, 64)])
+@pytest.mark.parametrize("lse_bsh", [False, True])
+def test_cache_load_widens_bit_exactly_in_both_lse_layouts(hip, B, Sq, H, D, lse_bsh):
+    """bf16 slot -> fp32 state: the flat widening pass and the lse's trip through the LDS (runs of 64 query
+    positions x all heads; fewer positions per run above 256 heads), ragged last run included."""
+    g = torch.Generator().manual_seed(B * 1000 + Sq + H)
+    slot_out = torch.randn(B, Sq, H, D, generator=g).bfloat16()
+    slot_lse = torch.randn(B, H, Sq, generator=g)
+    slot_lse[0, 0, 0] = float("-inf")
+    o, l = hip.cache_load(slot_out.cuda(), slot_lse.cuda(), torch.float32, dst_lse_bsh=lse_bsh)
+    torch.cuda.synchronize()
+    assert torch.equal(o.cpu(), slot_out.float())
+    want = slot_lse.transpose(1, 2).unsqueeze(-1).contiguous() if lse_bsh else slot_lse
+    assert l.shape == want.shape and torch.equal(l.cpu(), want)
+
+
 @pytest.mark.parametrize("B,Sq,H,D", [(1, 1, 1, 64), (2, 131, 3, 64), (1, 77, 3, 128), (1, 2222, 5, 64), (3, 700, 7, 128)])
 def test_same_format_copies_are_bit_exact(hip, B, Sq, H, D):
     """State copies whose two sides share dtype and lse layout take the flat-range path: slot -> slot
