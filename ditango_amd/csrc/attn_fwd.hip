@@ -795,7 +795,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
       *reinterpret_cast<u32x4*>(dst) = val;
     } else if (qg < q_end) {
       __bf16* dst = out_ptr + (((int64_t)b * a.Sq + qg) * a.H + h) * D + cc * 8;
-      *reinterpret_cast<u32x4*>(dst) = val;
+      __builtin_nontemporal_store(val, reinterpret_cast<u32x4*>(dst));
     }
   }
 }
