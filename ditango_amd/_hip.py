@@ -205,10 +205,12 @@ _workspaces = {}
 
 
 def attn_workspace(device) -> torch.Tensor:
-    """The per-device workspace of the attention launches (allocated once, ``dt_attn_workspace_bytes()``
-    bytes).  Launches that share it must be ordered on one stream, which is how ``proAttention`` runs."""
+    """The workspace of the attention launches made on the current stream of ``device`` (allocated once per
+    device and stream, ``dt_attn_workspace_bytes()`` bytes).  Launches that share a workspace must be ordered
+    on one stream; keyed by the stream, launches made on different streams never share one."""
     dev = torch.device(device)
-    key = (dev.type, dev.index if dev.index is not None else torch.cuda.current_device())
+    index = dev.index if dev.index is not None else torch.cuda.current_device()
+    key = (dev.type, index, torch.cuda.current_stream(index).cuda_stream)
     ws = _workspaces.get(key)
     if ws is None:
         ws = torch.empty(int(load_library().dt_attn_workspace_bytes()), dtype=torch.uint8, device=dev)

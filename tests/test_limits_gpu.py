@@ -280,6 +280,18 @@ def test_read_probe_and_its_argument_checks(hip):
         hip.hbm_read_probe(bufs * 6, sink)                     # 66 streams: more than one launch takes
 
 
+def test_attention_workspace_is_per_stream(hip):
+    """Launches on different streams must not share the tail-balancing workspace (they would race on it)."""
+    a = hip.attn_workspace("cuda")
+    assert hip.attn_workspace("cuda").data_ptr() == a.data_ptr()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        b = hip.attn_workspace("cuda")
+        assert hip.attn_workspace("cuda").data_ptr() == b.data_ptr()
+    assert a.data_ptr() != b.data_ptr() and a.numel() == b.numel()
+    assert hip.attn_workspace("cuda").data_ptr() == a.data_ptr()
+
+
 def test_mfma_probe_runs_and_checks_its_arguments(hip):
     sink = torch.zeros(1, dtype=torch.float32, device="cuda")
     flop = hip.mfma_probe(64, 16, sink)
