@@ -58,6 +58,13 @@ class proCache:
     def memory_constraint(self, mb: float) -> None:
         self._memory_constraint = mb
 
+    def get_curr_isp_stride(self, layer_id: int) -> int:
+        """Stride of the current (step, layer).  The reference's method of this name (core/cache.py:24-26)
+        indexes the RedundancyMap object, which has no ``__getitem__``: nothing calls it there.  Here it
+        returns what the attention call itself asks the map for (core/attention.py:90)."""
+        from .redundancy_map import get_redundancy_map
+        return int(get_redundancy_map().get_curr_isp_stride(get_timestep(), layer_id))
+
     def set_block_size_mb(self, tensor: torch.Tensor) -> float:
         """Size of one cached state for a K/V shard shaped like ``tensor`` ``[B,S,H,D]``:
         bf16 ``out`` plus fp32 ``lse`` = ``(2D + 4)`` bytes per (token, head).  (The

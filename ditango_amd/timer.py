@@ -12,7 +12,7 @@ _ENABLED = False
 _RECORDS: Dict[str, List[float]] = {}
 
 
-def init_timer(enable: bool = False) -> None:
+def init_timer(enable: bool = True) -> None:
     global _ENABLED
     _ENABLED = bool(enable)
     _RECORDS.clear()

@@ -80,6 +80,12 @@ def test_strides_follow_divider_map(ditango_env):
             assert rm.get_curr_isp_stride(t, l) == od.curr_stride(div, 8, t, l)
             assert rm.get_next_isp_stride(t, l) == od.next_stride(div, 8, t, l)
     assert rm.get_next_isp_stride(5, 0) == 8  # last step announces a full refresh
+    # the cache's accessor of the same name reads the current step
+    from ditango_amd.core.cache import proCache
+    from ditango_amd.utils import update_timestep
+    update_timestep(2)
+    assert proCache(8, 1).get_curr_isp_stride(1) == od.curr_stride(div, 8, 2, 1)
+    update_timestep(0)
     rm.auto_setting = True
     assert rm.get_curr_isp_stride(1, 0) == 8 and rm.get_next_isp_stride(1, 0) == 8
     rm.auto_setting = False
