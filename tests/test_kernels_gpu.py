@@ -372,3 +372,41 @@ def test_short_work_items_repeat_bit_exactly(hip, D):
             keep.clear()
     torch.cuda.synchronize()
     assert int(differing) == 0, f"{int(differing)} chunk states of {launches * n_chunks} differ from the first launch"
+
+
+def test_scheduled_launch_with_split_tail_and_merge_repeat_bit_exactly(hip):
+    """The device-scheduled launch with its tail run as parts, the fold kernel behind it and the merge of the
+    resulting states, 150 times on K/V just copied in from the host: every repetition returns the bits of
+    the first (the kernels share nothing but the workspace, and its users are ordered on the stream)."""
+    B, H, D, Sq, lens, diag = 1, 24, 128, 3000, [2000, 1500, 1800], 1
+    C = len(lens)
+    g = torch.Generator().manual_seed(77)
+    q = torch.randn(B, Sq, H, D, generator=g).bfloat16()
+    ks = [torch.randn(B, n, H, D, generator=g).bfloat16() for n in lens]
+    vs = [torch.randn(B, n, H, D, generator=g).bfloat16() for n in lens]
+    ids = torch.arange(C, dtype=torch.int32, device="cuda")
+    cnt = torch.tensor([C], dtype=torch.int32, device="cuda")
+    ws = hip.attn_workspace("cuda")
+    dq = q.cuda()
+
+    def run():
+        dk, dv = [k.cuda() for k in ks], [v.cuda() for v in vs]
+        so = torch.zeros(C, B, Sq, H, D, dtype=torch.bfloat16, device="cuda")
+        sl = torch.zeros(C, B, H, Sq, device="cuda")
+        do = torch.zeros(B, Sq, H, D, dtype=torch.bfloat16, device="cuda")
+        dl = torch.zeros(B, H, Sq, device="cuda")
+        hip.attn_sched_fwd(dq, hip.ChunkTable(dk, dv), ids, cnt, C, so, sl, diag, do, dl, workspace=ws)
+        out, lse = hip.merge_states([so[c] if c != diag else do for c in range(C)],
+                                    [sl[c] if c != diag else dl for c in range(C)])
+        return so, sl, do, dl, out, lse
+
+    first = run()
+    torch.cuda.synchronize()
+    full_out, full_lse = om.full_attention(q, ks, vs)
+    _check_state(first[4], first[5], full_out, full_lse, "merged")
+    differing = torch.zeros((), dtype=torch.int64, device="cuda")
+    for _ in range(150):
+        for a, b in zip(run(), first):
+            differing += (a != b).any().long()
+    torch.cuda.synchronize()
+    assert int(differing) == 0
