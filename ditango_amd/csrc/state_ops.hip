@@ -4,11 +4,10 @@
 //   * schedule builder      (per-chunk generalisation of core/attention.py:90-116)
 //   * relative-L1 sums      (utils.py:214-241)
 //
-// Work decomposition of the row kernels: one workgroup handles a run of
-// consecutive queries of ONE (batch, head).  A group of D/8 lanes owns one row
-// (query, head) and moves 16 bytes of bf16 (8 elements) per lane per state, so a
-// row is one contiguous 128/256-byte access, and the lse values of consecutive
-// rows are consecutive floats in the [B,H,Sq] layout.
+// Work decomposition of the row-mapped copy kernel: one workgroup handles a run of
+// consecutive queries of ONE (batch, head), a group of D/8 lanes owns one row
+// (query, head), and the lse values of consecutive rows are consecutive floats in
+// the [B,H,Sq] layout.  The merge works on 256-byte units instead (see there).
 #include <algorithm>
 
 #include "dt_common.h"
@@ -126,170 +125,257 @@ __device__ __forceinline__ void decode_wg(int wg, int B, int H, int& st, int& b,
   h = bh - b * H;
 }
 
-// Running state of one output row while states are folded in.
-struct RowAcc {
+// ---- N-way merge ------------------------------------------------------------------------------
+// A group of 16 lanes owns one UNIT = 128 consecutive elements of the [B,Sq,H,D] tensors: one row
+// at D = 128, two rows that are neighbours in memory at D = 64.  A lane owns elements [4c, 4c+4) and
+// [64+4c, 64+4c+4) of its unit, so every load and store instruction of the group covers 128 (bf16) or
+// 256 (fp32) contiguous bytes for either head dimension (a lane owning 8 consecutive elements would
+// write fp32 as two interleaved half-sector streams); at D = 64 the two halves of a lane belong to
+// two different rows and carry their own lse, maximum and denominator (with a lane group per 128-byte
+// row instead, every load instruction touched half of each cache line: -10 to -30 % at D = 64).
+// Units go to workgroups (16 per pass, P passes) in one of two ways:
+//   MAP_LINEAR  consecutive units in memory order: every stream a workgroup reads is one contiguous
+//               block, but its lse values in the [B,H,Sq] layout are one 32-byte sector apiece;
+//   MAP_TILED   a tile of 4*P consecutive queries x 4 consecutive head units, tiles ordered head-fastest:
+//               every row read is still part of a contiguous kilobyte that the neighbouring workgroup
+//               continues, and the lse values of a head are a run of 4*P consecutive floats, i.e. whole
+//               sectors at P = 2 (fetched bytes 1.11 -> 1.0x of the state bytes at 8 states).
+// States are consumed in branch-free, fully unrolled batches of kBatch (all loads of a batch are in
+// flight before the first use; the pointers come from the kernel arguments with a uniform index, so
+// they are scalar loads issued together) and folded with the running-maximum rescale; the remainder
+// goes through a fully unrolled smaller batch.
+constexpr int kUnitLanes = 16;
+constexpr int kUnitsPerPass = kThreads / kUnitLanes;
+constexpr int kTileHeadUnits = 4;
+enum { MAP_LINEAR = 1, MAP_TILED = 2 };
+
+template <int R>
+struct UnitPos {           // where the R rows of a unit sit
+  int b[R], h[R], s[R];
+  bool live[R];
+  int64_t elem;            // element offset of the unit in [B,Sq,H,D]
+};
+
+template <int R>
+struct UnitAcc {
   float acc[8];
-  float m, den;
+  float m[R], den[R];
 };
 
-constexpr int kMergeRows = 2;  // rows a lane group folds at once
-
-// The loads of one batch of NB states for kMergeRows rows, and their fold into the running rows.
-template <int NB>
-struct BatchRegs {
-  float l[kMergeRows][NB];
-  Row8 r[kMergeRows][NB];     // mixed dtypes
-  u32x4 rb[kMergeRows][NB];   // all states bf16: 8 elements per lane in 4 registers
+template <int R, int NB, int P>
+struct UnitRegs {
+  float l[P][R][NB];
+  u32x4 rb[P][NB];   // all states bf16
+  Row8 r[P][NB];     // mixed dtypes
 };
 
-template <int D, int NB, bool ALL_BF16>
-__device__ __forceinline__ void load_batch(const MergeArgs& a, int i0, const int (&b)[kMergeRows],
-                                           const int (&h)[kMergeRows], const int (&s)[kMergeRows],
-                                           const bool (&live)[kMergeRows], const int64_t (&elem)[kMergeRows], int cc,
-                                           BatchRegs<NB>& g) {
+template <int R, int NB, bool ALL_BF16, int P>
+__device__ __forceinline__ void unit_load(const MergeArgs& a, int i0, const UnitPos<R> (&u)[P], int cc,
+                                          UnitRegs<R, NB, P>& g) {
 #pragma unroll
   for (int j = 0; j < NB; ++j) {
     const int i = i0 + j;
     const float* lp = a.lse[i];
     const void* op = a.out[i];
     const bool bsh = (a.bsh_mask >> i) & 1;
+    const bool f32 = (a.fp32_mask >> i) & 1;
 #pragma unroll
-    for (int p = 0; p < kMergeRows; ++p) {
-      if (live[p]) {
-        g.l[p][j] = lp[lse_index(bsh, b[p], h[p], s[p], a.H, a.Sq)];
-        if (ALL_BF16) {
-          const uint16_t* q = reinterpret_cast<const uint16_t*>(op) + elem[p] + 4 * cc;
-          const u32x2 g0 = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(q));
-          const u32x2 g1 = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(q + D / 2));
-          g.rb[p][j].x = g0.x; g.rb[p][j].y = g0.y; g.rb[p][j].z = g1.x; g.rb[p][j].w = g1.y;
-        } else {
-          g.r[p][j] = load_row8<D>(op, (a.fp32_mask >> i) & 1, elem[p], cc);
-        }
+    for (int p = 0; p < P; ++p) {
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+        g.l[p][r][j] = u[p].live[r] ? lp[lse_index(bsh, u[p].b[r], u[p].h[r], u[p].s[r], a.H, a.Sq)] : -INFINITY;
+      const bool live_lo = u[p].live[0], live_hi = u[p].live[R - 1];
+      if (ALL_BF16) {
+        const uint16_t* q = reinterpret_cast<const uint16_t*>(op) + u[p].elem + 4 * cc;
+        u32x2 g0 = u32x2{0u, 0u}, g1 = u32x2{0u, 0u};
+        if (live_lo) g0 = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(q));
+        if (live_hi) g1 = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(q + 64));
+        g.rb[p][j].x = g0.x; g.rb[p][j].y = g0.y; g.rb[p][j].z = g1.x; g.rb[p][j].w = g1.y;
       } else {
-        g.l[p][j] = -INFINITY;
-      }
-    }
-  }
-}
-
-template <int NB, bool ALL_BF16>
-__device__ __forceinline__ void fold_batch(const MergeArgs& a, int i0, const BatchRegs<NB>& g, RowAcc (&ra)[kMergeRows]) {
-#pragma unroll
-  for (int p = 0; p < kMergeRows; ++p) {
-    float m_new = ra[p].m;
-#pragma unroll
-    for (int j = 0; j < NB; ++j) m_new = fmaxf(m_new, g.l[p][j]);
-    if (m_new > -INFINITY) {
-      const float rescale = __expf(ra[p].m - m_new);  // exp(-inf) = 0 on the first non-empty batch
-      ra[p].den *= rescale;
-#pragma unroll
-      for (int k = 0; k < 8; ++k) ra[p].acc[k] *= rescale;
-#pragma unroll
-      for (int j = 0; j < NB; ++j) {
-        const float w = __expf(g.l[p][j] - m_new);
-        float x[8];
-        if (ALL_BF16) {
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            x[2 * q] = __uint_as_float(g.rb[p][j][q] << 16);
-            x[2 * q + 1] = __uint_as_float(g.rb[p][j][q] & 0xffff0000u);
-          }
+        Row8 v;
+        v.lo = u32x4{0u, 0u, 0u, 0u};
+        v.hi = v.lo;
+        if (f32) {
+          const float* q = reinterpret_cast<const float*>(op) + u[p].elem + 4 * cc;
+          if (live_lo) v.lo = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(q));
+          if (live_hi) v.hi = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(q + 64));
         } else {
-          unpack_row8(g.r[p][j], (a.fp32_mask >> (i0 + j)) & 1, x);
+          const uint16_t* q = reinterpret_cast<const uint16_t*>(op) + u[p].elem + 4 * cc;
+          u32x2 g0 = u32x2{0u, 0u}, g1 = u32x2{0u, 0u};
+          if (live_lo) g0 = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(q));
+          if (live_hi) g1 = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(q + 64));
+          v.lo.x = g0.x; v.lo.y = g0.y; v.lo.z = g1.x; v.lo.w = g1.y;
         }
-        ra[p].den += w;
-#pragma unroll
-        for (int k = 0; k < 8; ++k) ra[p].acc[k] = __builtin_fmaf(w, x[k], ra[p].acc[k]);
+        g.r[p][j] = v;
       }
-      ra[p].m = m_new;
     }
   }
 }
 
-// Folds states [i0, i0 + NB) into kMergeRows rows at once.  Branch free: all NB x kMergeRows
-// lse loads and row loads are issued back to back before the first use (the pointers come
-// from the kernel arguments with a uniform index, so they are scalar loads issued together).
-template <int D, int NB, bool ALL_BF16>
-__device__ __forceinline__ void merge_batch(const MergeArgs& a, int i0, const int (&b)[kMergeRows],
-                                            const int (&h)[kMergeRows], const int (&s)[kMergeRows],
-                                            const bool (&live)[kMergeRows], const int64_t (&elem)[kMergeRows], int cc,
-                                            RowAcc (&ra)[kMergeRows]) {
-  BatchRegs<NB> g;
-  load_batch<D, NB, ALL_BF16>(a, i0, b, h, s, live, elem, cc, g);
-  fold_batch<NB, ALL_BF16>(a, i0, g, ra);
+template <int R, int NB, bool ALL_BF16, int P>
+__device__ __forceinline__ void unit_fold(const MergeArgs& a, int i0, const UnitRegs<R, NB, P>& g,
+                                          UnitAcc<R> (&ua)[P]) {
+  constexpr int kPer = 8 / R;   // elements of a lane that belong to one row
+#pragma unroll
+  for (int p = 0; p < P; ++p) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      float m_new = ua[p].m[r];
+#pragma unroll
+      for (int j = 0; j < NB; ++j) m_new = fmaxf(m_new, g.l[p][r][j]);
+      if (m_new > -INFINITY) {
+        const float rescale = __expf(ua[p].m[r] - m_new);  // exp(-inf) = 0 on the first non-empty batch
+        ua[p].den[r] *= rescale;
+#pragma unroll
+        for (int k = 0; k < kPer; ++k) ua[p].acc[r * kPer + k] *= rescale;
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+          const float w = __expf(g.l[p][r][j] - m_new);
+          float x[8];
+          if (ALL_BF16) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              x[2 * q] = __uint_as_float(g.rb[p][j][q] << 16);
+              x[2 * q + 1] = __uint_as_float(g.rb[p][j][q] & 0xffff0000u);
+            }
+          } else {
+            unpack_row8(g.r[p][j], (a.fp32_mask >> (i0 + j)) & 1, x);
+          }
+          ua[p].den[r] += w;
+#pragma unroll
+          for (int k = 0; k < kPer; ++k)
+            ua[p].acc[r * kPer + k] = __builtin_fmaf(w, x[r * kPer + k], ua[p].acc[r * kPer + k]);
+        }
+        ua[p].m[r] = m_new;
+      }
+    }
+  }
 }
 
-// The last, smaller batch: fully unrolled for its size (sizes NB, NB - 1, ..., 1 are tried in turn).
-template <int D, bool ALL_BF16, int NB>
-__device__ __forceinline__ void merge_rest(const MergeArgs& a, int i0, int rest, const int (&b)[kMergeRows],
-                                           const int (&h)[kMergeRows], const int (&s)[kMergeRows],
-                                           const bool (&live)[kMergeRows], const int64_t (&elem)[kMergeRows], int cc,
-                                           RowAcc (&ra)[kMergeRows]) {
+template <int R, int NB, bool ALL_BF16, int P>
+__device__ __forceinline__ void unit_batch(const MergeArgs& a, int i0, const UnitPos<R> (&u)[P], int cc,
+                                           UnitAcc<R> (&ua)[P]) {
+  UnitRegs<R, NB, P> g;
+  unit_load<R, NB, ALL_BF16, P>(a, i0, u, cc, g);
+  unit_fold<R, NB, ALL_BF16, P>(a, i0, g, ua);
+}
+
+template <int R, bool ALL_BF16, int NB, int P>
+__device__ __forceinline__ void unit_rest(const MergeArgs& a, int i0, int rest, const UnitPos<R> (&u)[P],
+                                          int cc, UnitAcc<R> (&ua)[P]) {
   if constexpr (NB >= 1) {
-    if (rest == NB) merge_batch<D, NB, ALL_BF16>(a, i0, b, h, s, live, elem, cc, ra);
-    else merge_rest<D, ALL_BF16, NB - 1>(a, i0, rest, b, h, s, live, elem, cc, ra);
+    if (rest == NB) unit_batch<R, NB, ALL_BF16, P>(a, i0, u, cc, ua);
+    else unit_rest<R, ALL_BF16, NB - 1, P>(a, i0, rest, u, cc, ua);
   }
 }
 
-// One workgroup = kMergeRows * 256/(D/8) rows; a group of D/8 lanes owns kMergeRows rows.  Two
-// ways of handing rows to workgroups: consecutive queries of one (batch, head), workgroups ordered
-// head-fastest (the lse reads are contiguous, the row reads of concurrently running workgroups
-// are neighbours) -- or, LINEAR, consecutive rows of the [B,Sq,H,D] tensors (every stream a
-// workgroup reads is one contiguous block), which wins once many states are read at a time
-// (measured: 8 states +5 %, 16 states +3 %, 4 states +-3 %, 1-2 states -6 to -12 %).
-// States are consumed in batches of kBatch (the remainder through a fully unrolled smaller
-// batch) and folded with the running-maximum rescale.
-template <int D, bool ALL_BF16, bool LINEAR>
+template <int D, bool ALL_BF16, int MAP, int P>
 __global__ __launch_bounds__(kThreads) void merge_states_kernel(const MergeArgs a) {
-  constexpr int kLanesPerRow = D / 8;
-  constexpr int kRowsPerPass = kThreads / kLanesPerRow;
-  constexpr int kRowsPerWg = kRowsPerPass * kMergeRows;
-  int st = 0, b0 = 0, h0 = 0;
-  if constexpr (!LINEAR) decode_wg(blockIdx.x, a.B, a.H, st, b0, h0);
-  const int rr = threadIdx.x / kLanesPerRow;
-  const int cc = threadIdx.x % kLanesPerRow;
-  int s[kMergeRows], b[kMergeRows], h[kMergeRows];
-  bool live[kMergeRows];
-  int64_t elem[kMergeRows];
-  RowAcc ra[kMergeRows];
+  constexpr int R = 128 / D;
+  constexpr int kUnitsPerWg = kUnitsPerPass * P;
+  constexpr int kTileQueries = kUnitsPerWg / kTileHeadUnits;
+  constexpr int kTileQueriesPerPass = kUnitsPerPass / kTileHeadUnits;
+  const int rr = threadIdx.x / kUnitLanes;
+  const int cc = threadIdx.x % kUnitLanes;
+  UnitPos<R> u[P];
+  UnitAcc<R> ua[P];
   const int64_t rows_total = (int64_t)a.B * a.Sq * a.H;
+  int tb = 0, ts0 = 0, thu0 = 0;
+  if constexpr (MAP == MAP_TILED) {
+    const int n_hg = a.H / (R * kTileHeadUnits);
+    const int n_qt = (a.Sq + kTileQueries - 1) / kTileQueries;
+    const int hg = blockIdx.x % n_hg;
+    const int t = blockIdx.x / n_hg;
+    const int qt = t % n_qt;
+    tb = t / n_qt;
+    ts0 = qt * kTileQueries;
+    thu0 = hg * kTileHeadUnits;
+  }
 #pragma unroll
-  for (int p = 0; p < kMergeRows; ++p) {
-    if constexpr (LINEAR) {
-      const int64_t row = (int64_t)blockIdx.x * kRowsPerWg + p * kRowsPerPass + rr;
-      live[p] = row < rows_total;
-      const int64_t rc = live[p] ? row : 0;
-      const int64_t bs = rc / a.H;
-      h[p] = (int)(rc - bs * a.H);
-      b[p] = (int)(bs / a.Sq);
-      s[p] = (int)(bs - (int64_t)b[p] * a.Sq);
-      elem[p] = rc * D;
+  for (int p = 0; p < P; ++p) {
+    if constexpr (MAP == MAP_TILED) {
+      const int s = ts0 + p * kTileQueriesPerPass + rr / kTileHeadUnits;
+      const int h0 = (thu0 + rr % kTileHeadUnits) * R;
+      const bool ok = s < a.Sq;
+      const int sc = ok ? s : 0;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        u[p].b[r] = tb;
+        u[p].h[r] = h0 + r;
+        u[p].s[r] = sc;
+        u[p].live[r] = ok;
+      }
+      u[p].elem = (((int64_t)tb * a.Sq + sc) * a.H + h0) * D;
     } else {
-      b[p] = b0;
-      h[p] = h0;
-      s[p] = st * kRowsPerWg + p * kRowsPerPass + rr;
-      live[p] = s[p] < a.Sq;
-      elem[p] = (((int64_t)b0 * a.Sq + s[p]) * a.H + h0) * D;
-    }
-    ra[p].m = -INFINITY;
-    ra[p].den = 0.f;
+      const int64_t unit = (int64_t)blockIdx.x * kUnitsPerWg + p * kUnitsPerPass + rr;
 #pragma unroll
-    for (int k = 0; k < 8; ++k) ra[p].acc[k] = 0.f;
+      for (int r = 0; r < R; ++r) {
+        const int64_t row = unit * R + r;
+        u[p].live[r] = row < rows_total;
+        const int64_t rc = u[p].live[r] ? row : 0;
+        if (rows_total <= 0x7fffffffLL) {   // uniform: the common case divides in 32 bits
+          const uint32_t bs = (uint32_t)rc / (uint32_t)a.H;
+          u[p].h[r] = (int)((uint32_t)rc - bs * (uint32_t)a.H);
+          u[p].b[r] = (int)(bs / (uint32_t)a.Sq);
+          u[p].s[r] = (int)(bs - (uint32_t)u[p].b[r] * (uint32_t)a.Sq);
+        } else {
+          const int64_t bs = rc / a.H;
+          u[p].h[r] = (int)(rc - bs * a.H);
+          u[p].b[r] = (int)(bs / a.Sq);
+          u[p].s[r] = (int)(bs - (int64_t)u[p].b[r] * a.Sq);
+        }
+      }
+      u[p].elem = u[p].live[0] ? unit * 128 : 0;
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      ua[p].m[r] = -INFINITY;
+      ua[p].den[r] = 0.f;
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) ua[p].acc[k] = 0.f;
   }
   int i0 = 0;
-  for (; i0 + kBatch <= a.n; i0 += kBatch) merge_batch<D, kBatch, ALL_BF16>(a, i0, b, h, s, live, elem, cc, ra);
-  merge_rest<D, ALL_BF16, kBatch - 1>(a, i0, a.n - i0, b, h, s, live, elem, cc, ra);
+  for (; i0 + kBatch <= a.n; i0 += kBatch) unit_batch<R, kBatch, ALL_BF16, P>(a, i0, u, cc, ua);
+  unit_rest<R, ALL_BF16, kBatch - 1, P>(a, i0, a.n - i0, u, cc, ua);
+  constexpr int kPer = 8 / R;
 #pragma unroll
-  for (int p = 0; p < kMergeRows; ++p) {
-    if (!live[p]) continue;
-    const float inv = ra[p].den > 0.f ? 1.f / ra[p].den : 0.f;
+  for (int p = 0; p < P; ++p) {
     float o[8];
 #pragma unroll
-    for (int k = 0; k < 8; ++k) o[k] = ra[p].acc[k] * inv;
-    store_row8<D>(a.dst_out, a.dst_fp32 != 0, elem[p], cc, o);
-    if (cc == 0 && a.dst_lse != nullptr)
-      a.dst_lse[lse_index(a.dst_bsh != 0, b[p], h[p], s[p], a.H, a.Sq)] =
-          ra[p].den > 0.f ? ra[p].m + __logf(ra[p].den) : -INFINITY;
+    for (int r = 0; r < R; ++r) {
+      const float inv = ua[p].den[r] > 0.f ? 1.f / ua[p].den[r] : 0.f;
+#pragma unroll
+      for (int k = 0; k < kPer; ++k) o[r * kPer + k] = ua[p].acc[r * kPer + k] * inv;
+    }
+    const bool live_lo = u[p].live[0], live_hi = u[p].live[R - 1];
+    if (a.dst_fp32) {
+      float* q = reinterpret_cast<float*>(a.dst_out) + u[p].elem + 4 * cc;
+      u32x4 v0, v1;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        v0[i] = __float_as_uint(o[i]);
+        v1[i] = __float_as_uint(o[4 + i]);
+      }
+      if (live_lo) __builtin_nontemporal_store(v0, reinterpret_cast<u32x4*>(q));
+      if (live_hi) __builtin_nontemporal_store(v1, reinterpret_cast<u32x4*>(q + 64));
+    } else {
+      uint16_t* q = reinterpret_cast<uint16_t*>(a.dst_out) + u[p].elem + 4 * cc;
+      u32x2 g0, g1;
+      g0.x = pack_bf16x2(o[0], o[1]);
+      g0.y = pack_bf16x2(o[2], o[3]);
+      g1.x = pack_bf16x2(o[4], o[5]);
+      g1.y = pack_bf16x2(o[6], o[7]);
+      if (live_lo) __builtin_nontemporal_store(g0, reinterpret_cast<u32x2*>(q));
+      if (live_hi) __builtin_nontemporal_store(g1, reinterpret_cast<u32x2*>(q + 64));
+    }
+    if (a.dst_lse != nullptr) {
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+        if (cc == r && u[p].live[r])
+          a.dst_lse[lse_index(a.dst_bsh != 0, u[p].b[r], u[p].h[r], u[p].s[r], a.H, a.Sq)] =
+              ua[p].den[r] > 0.f ? ua[p].m[r] + __logf(ua[p].den[r]) : -INFINITY;
+    }
   }
 }
 
@@ -544,16 +630,29 @@ __global__ __launch_bounds__(kThreads) void hbm_read_probe_kernel(const ProbeArg
 
 // ---- host-side launchers ---------------------------------------------------------------
 
-constexpr int kLinearFrom = 6;  // states per launch from which rows are handed out in memory order
+// Which mapping and how many passes a launch gets (A/B on one box, states rotating through HBM; TB/s):
+//   * D = 128, up to 5 states: linear, one pass (2 states 6.3 against 6.2 tiled; two passes 5.2-5.6);
+//   * D = 128, 6 states and more: tiled, two passes (8 states 6.52-6.56 against 6.43 linear; 32 states of
+//     743 MB 5.88 against 5.74 with one pass);
+//   * D = 64: tiled; one pass while the launch is small (8 states of 14 MB: 5.6 against 5.2 with two
+//     passes -- finer workgroups fill the last round of the chip better), two passes on large ones.
+constexpr int kTiledFrom = 6;
+constexpr int64_t kTwoPassUnits = 1 << 20;
+
+template <int D, int MAP, int P>
+static void launch_merge_k(const MergeArgs& a, unsigned wgs, hipStream_t stream) {
+  if (a.fp32_mask == 0) hipLaunchKernelGGL((merge_states_kernel<D, true, MAP, P>), dim3(wgs), dim3(kThreads), 0, stream, a);
+  else hipLaunchKernelGGL((merge_states_kernel<D, false, MAP, P>), dim3(wgs), dim3(kThreads), 0, stream, a);
+}
 
 template <int D>
-static void launch_merge_d(const MergeArgs& a, bool all_bf16, bool linear, unsigned wgs, hipStream_t stream) {
-  if (linear) {
-    if (all_bf16) hipLaunchKernelGGL((merge_states_kernel<D, true, true>), dim3(wgs), dim3(kThreads), 0, stream, a);
-    else hipLaunchKernelGGL((merge_states_kernel<D, false, true>), dim3(wgs), dim3(kThreads), 0, stream, a);
+static void launch_merge_d(const MergeArgs& a, bool tiled, int passes, unsigned wgs, hipStream_t stream) {
+  if (tiled) {
+    if (passes == 2) launch_merge_k<D, MAP_TILED, 2>(a, wgs, stream);
+    else launch_merge_k<D, MAP_TILED, 1>(a, wgs, stream);
   } else {
-    if (all_bf16) hipLaunchKernelGGL((merge_states_kernel<D, true, false>), dim3(wgs), dim3(kThreads), 0, stream, a);
-    else hipLaunchKernelGGL((merge_states_kernel<D, false, false>), dim3(wgs), dim3(kThreads), 0, stream, a);
+    if (passes == 2) launch_merge_k<D, MAP_LINEAR, 2>(a, wgs, stream);
+    else launch_merge_k<D, MAP_LINEAR, 1>(a, wgs, stream);
   }
 }
 
@@ -562,18 +661,27 @@ int launch_merge(const MergeArgs& a, int D, hipStream_t stream) {
     set_error("head dim %d not built (64 and 128 are)", D);
     return DT_ERR_UNSUPPORTED;
   }
-  const int rows_per_wg = kThreads / (D / 8) * kMergeRows;
-  const bool linear = a.n >= kLinearFrom;
-  const int n_st = (a.Sq + rows_per_wg - 1) / rows_per_wg;
-  const int64_t wgs = linear ? ((int64_t)a.B * a.Sq * a.H + rows_per_wg - 1) / rows_per_wg : (int64_t)a.B * a.H * n_st;
+  const int R = 128 / D;   // rows per unit
+  const int64_t units = ((int64_t)a.B * a.Sq * a.H + R - 1) / R;
+  const bool tiled = (D == 64 || a.n >= kTiledFrom) && a.H % (R * kTileHeadUnits) == 0;
+  int passes;
+  if (D == 64) passes = units >= kTwoPassUnits ? 2 : 1;
+  else passes = a.n >= kTiledFrom ? 2 : 1;
+  const int units_per_wg = kUnitsPerPass * passes;
+  int64_t wgs;
+  if (tiled) {
+    const int tile_q = units_per_wg / kTileHeadUnits;
+    wgs = (int64_t)a.B * ((a.Sq + tile_q - 1) / tile_q) * (a.H / (R * kTileHeadUnits));
+  } else {
+    wgs = (units + units_per_wg - 1) / units_per_wg;
+  }
   if (wgs <= 0) return DT_OK;
   if (wgs > 0x7fffffffLL) {
     set_error("merge grid too large");
     return DT_ERR_INVALID;
   }
-  const bool all_bf16 = (a.fp32_mask == 0);
-  if (D == 128) launch_merge_d<128>(a, all_bf16, linear, (unsigned)wgs, stream);
-  else launch_merge_d<64>(a, all_bf16, linear, (unsigned)wgs, stream);
+  if (D == 128) launch_merge_d<128>(a, tiled, passes, (unsigned)wgs, stream);
+  else launch_merge_d<64>(a, tiled, passes, (unsigned)wgs, stream);
   return hip_fail(hipGetLastError(), "merge_states launch");
 }
 

@@ -186,6 +186,54 @@ def test_merge_all_empty_and_layouts(hip):
     assert (a_lse.cpu().squeeze(-1).transpose(1, 2) - ref_lse).abs().max() < 1e-5
 
 
+@pytest.mark.parametrize("B,Sq,H", [(1, 77, 5), (2, 150, 8), (1, 37, 24), (1, 19, 48), (3, 9, 16)])
+@pytest.mark.parametrize("D,n", [(64, 2), (64, 8), (128, 3), (128, 8), (128, 17)])
+def test_merge_row_mappings(hip, B, Sq, H, D, n):
+    """The merge hands rows to workgroups in memory order or as tiles of queries x heads, depending on the
+    head count, the head dimension and the number of states; at D = 64 two neighbouring rows share a lane
+    group.  Head counts that do and do not divide into tiles, an odd row count, query counts that leave
+    partial tiles; fp32 and bf16 destinations; one state fp32, one lse in the [B,S,H,1] layout."""
+    g = torch.Generator().manual_seed(B * 1000 + Sq * 10 + H + D + n)
+    outs = [torch.randn(B, Sq, H, D, generator=g).bfloat16() for _ in range(n)]
+    lses = [torch.randn(B, H, Sq, generator=g) * 3 for _ in range(n)]
+    lses[0][:, :, ::4] = -math.inf
+    lses[n - 1][:, ::2, :] = -math.inf
+    ref_out, ref_lse = om.merge_states_closed_form([o.float() for o in outs], lses)
+    d_outs = [o.cuda() for o in outs]
+    d_lses = [l.cuda() for l in lses]
+    def lse_close(got, tol=1e-5):   # rows without any state keep -inf
+        fin = torch.isfinite(ref_lse)
+        return bool((got[~fin] == ref_lse[~fin]).all()) and float((got[fin] - ref_lse[fin]).abs().max()) < tol
+
+    o, l = hip.merge_states(d_outs, d_lses)
+    torch.cuda.synchronize()
+    assert (o.cpu() - ref_out).abs().max() < 1e-5 * n and lse_close(l.cpu())
+    d_outs[1] = d_outs[1].float()
+    d_lses[n - 1] = d_lses[n - 1].transpose(1, 2).contiguous().unsqueeze(-1)
+    dst_l = torch.empty(B, Sq, H, 1, device="cuda")
+    o2, l2 = hip.merge_states(d_outs, d_lses, dst_dtype=torch.bfloat16, dst_lse=dst_l)
+    torch.cuda.synchronize()
+    assert l2.data_ptr() == dst_l.data_ptr()
+    assert (o2.float().cpu() - ref_out).abs().max() <= 2.0 ** -8 * float(ref_out.abs().max())
+    assert lse_close(dst_l.cpu().squeeze(-1).transpose(1, 2))
+
+
+def test_merge_large_launch_d64(hip):
+    """A D = 64 launch of more than 2^20 lane groups takes two tile passes per workgroup."""
+    B, Sq, H, D, n = 1, 16400, 128, 64, 2
+    g = torch.Generator(device="cuda").manual_seed(5)
+    outs = [torch.randn(B, Sq, H, D, generator=g, device="cuda").bfloat16() for _ in range(n)]
+    lses = [torch.randn(B, H, Sq, generator=g, device="cuda") * 2 for _ in range(n)]
+    o, l = hip.merge_states(outs, lses)
+    torch.cuda.synchronize()
+    rows = torch.randperm(Sq)[:257]
+    ref_out, ref_lse = om.merge_states_closed_form([x[:, rows].float().cpu() for x in outs],
+                                                   [x[:, :, rows].cpu() for x in lses])
+    assert (o[:, rows].cpu() - ref_out).abs().max() < 1e-5 and (l[:, :, rows].cpu() - ref_lse).abs().max() < 1e-5
+    # every row was written: the lse of all rows against torch's logaddexp
+    assert (l - torch.logaddexp(lses[0], lses[1])).abs().max() < 1e-5
+
+
 @pytest.mark.parametrize("D", [64, 128])
 def test_merge_many_states_in_place_with_row_layout_lse(hip, D):
     """Six states and more take the kernel's other row-to-workgroup mapping: in place into the first
