@@ -139,7 +139,9 @@ __device__ __forceinline__ void decode_wg(int wg, int B, int H, int& st, int& b,
 //   MAP_TILED   a tile of 4*P consecutive queries x 4 consecutive head units, tiles ordered head-fastest:
 //               every row read is still part of a contiguous kilobyte that the neighbouring workgroup
 //               continues, and the lse values of a head are a run of 4*P consecutive floats, i.e. whole
-//               sectors at P = 2 (fetched bytes 1.11 -> 1.0x of the state bytes at 8 states).
+//               sectors at P = 2; two tiles that follow each other along the queries go to the same XCD
+//               (fetched bytes 1.108 -> 1.029 x the state bytes at 8 states of 93 MB; what is left are
+//               runs that straddle a 64-byte line because a head's lse row starts at any multiple of 4).
 // States are consumed in branch-free, fully unrolled batches of kBatch (all loads of a batch are in
 // flight before the first use; the pointers come from the kernel arguments with a uniform index, so
 // they are scalar loads issued together) and folded with the running-maximum rescale; the remainder
@@ -284,10 +286,18 @@ __global__ __launch_bounds__(kThreads) void merge_states_kernel(const MergeArgs 
   if constexpr (MAP == MAP_TILED) {
     const int n_hg = a.H / (R * kTileHeadUnits);
     const int n_qt = (a.Sq + kTileQueries - 1) / kTileQueries;
-    const int hg = blockIdx.x % n_hg;
-    const int t = blockIdx.x / n_hg;
-    const int qt = t % n_qt;
-    tb = t / n_qt;
+    // Two tiles that follow each other along the queries share the 64-byte lines of their lse runs.
+    // Workgroups go to the 8 XCDs in turn; the pair is handed to ONE XCD as two consecutive workgroups
+    // of it, so that the line is fetched into one L2 once instead of into two.
+    const int n_qt2 = (n_qt + 1) >> 1;
+    const uint32_t xcd = blockIdx.x & 7u, j = blockIdx.x >> 3;
+    const uint32_t sup = (j >> 1) * 8u + xcd;
+    if (sup >= (uint32_t)a.B * n_qt2 * n_hg) return;
+    const int hg = sup % n_hg;
+    const int t = sup / n_hg;
+    const int qt = 2 * (t % n_qt2) + (int)(j & 1u);
+    if (qt >= n_qt) return;
+    tb = t / n_qt2;
     ts0 = qt * kTileQueries;
     thu0 = hg * kTileHeadUnits;
   }
@@ -671,7 +681,9 @@ int launch_merge(const MergeArgs& a, int D, hipStream_t stream) {
   int64_t wgs;
   if (tiled) {
     const int tile_q = units_per_wg / kTileHeadUnits;
-    wgs = (int64_t)a.B * ((a.Sq + tile_q - 1) / tile_q) * (a.H / (R * kTileHeadUnits));
+    // pairs of query tiles, 8 pairs (one per XCD) x 2 workgroups at a time
+    const int64_t n_qt2 = ((a.Sq + tile_q - 1) / tile_q + 1) / 2;
+    wgs = 16 * (((int64_t)a.B * n_qt2 * (a.H / (R * kTileHeadUnits)) + 7) / 8);
   } else {
     wgs = (units + units_per_wg - 1) / units_per_wg;
   }
