@@ -422,7 +422,7 @@ def run_workload(name, args, steps, warmup, main, reuse=None, kernels_only=False
     kr_ms = time_kernel(Rotation(probe, L_run), reps)
     kr_gbs = C * probe_bytes / (kr_ms * 1e-3) / 1e9
 
-    traffic = load_traffic(name) if reuse is None else {}
+    traffic = load_traffic(name)   # per launch shape: the same whatever reuse fraction drew the mask
     # counter bytes of exactly the launch shape that is timed next to them, or nothing
     k1_traffic = traffic.get("attn_fwd", {}).get(str(n_typ)) if isinstance(traffic.get("attn_fwd"), dict) else None
     k2_traffic = traffic.get("merge_states", {}).get(str(C)) if isinstance(traffic.get("merge_states"), dict) else None
