@@ -271,32 +271,31 @@ __device__ __forceinline__ void unit_rest(const MergeArgs& a, int i0, int rest, 
   }
 }
 
-template <int D, bool ALL_BF16, int MAP, int P>
-__global__ __launch_bounds__(kThreads) void merge_states_kernel(const MergeArgs a) {
+// Where the P units of this lane group sit (see the two mappings above); false when the workgroup is one
+// of those that pad the tiled grid.
+template <int D, int MAP, int P>
+__device__ __forceinline__ bool unit_positions(int B, int Sq, int H, UnitPos<128 / D> (&u)[P]) {
   constexpr int R = 128 / D;
   constexpr int kUnitsPerWg = kUnitsPerPass * P;
   constexpr int kTileQueries = kUnitsPerWg / kTileHeadUnits;
   constexpr int kTileQueriesPerPass = kUnitsPerPass / kTileHeadUnits;
   const int rr = threadIdx.x / kUnitLanes;
-  const int cc = threadIdx.x % kUnitLanes;
-  UnitPos<R> u[P];
-  UnitAcc<R> ua[P];
-  const int64_t rows_total = (int64_t)a.B * a.Sq * a.H;
+  const int64_t rows_total = (int64_t)B * Sq * H;
   int tb = 0, ts0 = 0, thu0 = 0;
   if constexpr (MAP == MAP_TILED) {
-    const int n_hg = a.H / (R * kTileHeadUnits);
-    const int n_qt = (a.Sq + kTileQueries - 1) / kTileQueries;
+    const int n_hg = H / (R * kTileHeadUnits);
+    const int n_qt = (Sq + kTileQueries - 1) / kTileQueries;
     // Two tiles that follow each other along the queries share the 64-byte lines of their lse runs.
     // Workgroups go to the 8 XCDs in turn; the pair is handed to ONE XCD as two consecutive workgroups
     // of it, so that the line is fetched into one L2 once instead of into two.
     const int n_qt2 = (n_qt + 1) >> 1;
     const uint32_t xcd = blockIdx.x & 7u, j = blockIdx.x >> 3;
     const uint32_t sup = (j >> 1) * 8u + xcd;
-    if (sup >= (uint32_t)a.B * n_qt2 * n_hg) return;
+    if (sup >= (uint32_t)B * n_qt2 * n_hg) return false;
     const int hg = sup % n_hg;
     const int t = sup / n_hg;
     const int qt = 2 * (t % n_qt2) + (int)(j & 1u);
-    if (qt >= n_qt) return;
+    if (qt >= n_qt) return false;
     tb = t / n_qt2;
     ts0 = qt * kTileQueries;
     thu0 = hg * kTileHeadUnits;
@@ -306,7 +305,7 @@ __global__ __launch_bounds__(kThreads) void merge_states_kernel(const MergeArgs 
     if constexpr (MAP == MAP_TILED) {
       const int s = ts0 + p * kTileQueriesPerPass + rr / kTileHeadUnits;
       const int h0 = (thu0 + rr % kTileHeadUnits) * R;
-      const bool ok = s < a.Sq;
+      const bool ok = s < Sq;
       const int sc = ok ? s : 0;
 #pragma unroll
       for (int r = 0; r < R; ++r) {
@@ -315,7 +314,7 @@ __global__ __launch_bounds__(kThreads) void merge_states_kernel(const MergeArgs 
         u[p].s[r] = sc;
         u[p].live[r] = ok;
       }
-      u[p].elem = (((int64_t)tb * a.Sq + sc) * a.H + h0) * D;
+      u[p].elem = (((int64_t)tb * Sq + sc) * H + h0) * D;
     } else {
       const int64_t unit = (int64_t)blockIdx.x * kUnitsPerWg + p * kUnitsPerPass + rr;
 #pragma unroll
@@ -324,19 +323,47 @@ __global__ __launch_bounds__(kThreads) void merge_states_kernel(const MergeArgs 
         u[p].live[r] = row < rows_total;
         const int64_t rc = u[p].live[r] ? row : 0;
         if (rows_total <= 0x7fffffffLL) {   // uniform: the common case divides in 32 bits
-          const uint32_t bs = (uint32_t)rc / (uint32_t)a.H;
-          u[p].h[r] = (int)((uint32_t)rc - bs * (uint32_t)a.H);
-          u[p].b[r] = (int)(bs / (uint32_t)a.Sq);
-          u[p].s[r] = (int)(bs - (uint32_t)u[p].b[r] * (uint32_t)a.Sq);
+          const uint32_t bs = (uint32_t)rc / (uint32_t)H;
+          u[p].h[r] = (int)((uint32_t)rc - bs * (uint32_t)H);
+          u[p].b[r] = (int)(bs / (uint32_t)Sq);
+          u[p].s[r] = (int)(bs - (uint32_t)u[p].b[r] * (uint32_t)Sq);
         } else {
-          const int64_t bs = rc / a.H;
-          u[p].h[r] = (int)(rc - bs * a.H);
-          u[p].b[r] = (int)(bs / a.Sq);
-          u[p].s[r] = (int)(bs - (int64_t)u[p].b[r] * a.Sq);
+          const int64_t bs = rc / H;
+          u[p].h[r] = (int)(rc - bs * H);
+          u[p].b[r] = (int)(bs / Sq);
+          u[p].s[r] = (int)(bs - (int64_t)u[p].b[r] * Sq);
         }
       }
       u[p].elem = u[p].live[0] ? unit * 128 : 0;
     }
+  }
+  return true;
+}
+
+// Workgroups a launch over these units needs.
+static int64_t unit_grid(int B, int Sq, int H, int D, bool tiled, int passes) {
+  const int R = 128 / D;
+  const int units_per_wg = kUnitsPerPass * passes;
+  if (tiled) {
+    // pairs of query tiles, 8 pairs (one per XCD) x 2 workgroups at a time
+    const int tile_q = units_per_wg / kTileHeadUnits;
+    const int64_t n_qt2 = ((Sq + tile_q - 1) / tile_q + 1) / 2;
+    return 16 * (((int64_t)B * n_qt2 * (H / (R * kTileHeadUnits)) + 7) / 8);
+  }
+  const int64_t units = ((int64_t)B * Sq * H + R - 1) / R;
+  return (units + units_per_wg - 1) / units_per_wg;
+}
+static bool unit_tiles_fit(int H, int D) { return H % ((128 / D) * kTileHeadUnits) == 0; }
+
+template <int D, bool ALL_BF16, int MAP, int P>
+__global__ __launch_bounds__(kThreads) void merge_states_kernel(const MergeArgs a) {
+  constexpr int R = 128 / D;
+  const int cc = threadIdx.x % kUnitLanes;
+  UnitPos<R> u[P];
+  UnitAcc<R> ua[P];
+  if (!unit_positions<D, MAP, P>(a.B, a.Sq, a.H, u)) return;
+#pragma unroll
+  for (int p = 0; p < P; ++p) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       ua[p].m[r] = -INFINITY;
@@ -433,6 +460,72 @@ __global__ __launch_bounds__(kThreads) void state_copy_kernel(const CopyArgs a) 
       if (copy_lse) a.dst_lse[lse_index(a.dst_bsh != 0, b, h, s, a.H, a.Sq)] = l[p];
     }
   }
+}
+
+// The same copy on 256-byte units (see the merge): at D = 64 a lane group then moves two neighbouring
+// rows and every load / store instruction covers whole 128-byte lines, where the row-mapped kernel above
+// touches half of each line per instruction.
+template <int D, int MAP>
+__global__ __launch_bounds__(kThreads) void state_copy_units_kernel(const CopyArgs a) {
+  constexpr int R = 128 / D;
+  const int cc = threadIdx.x % kUnitLanes;
+  UnitPos<R> u[1];
+  if (!unit_positions<D, MAP, 1>(a.B, a.Sq, a.H, u)) return;
+  const bool live_lo = u[0].live[0], live_hi = u[0].live[R - 1];
+  const bool with_lse = a.dst_lse != nullptr && a.src_lse != nullptr;
+  float l = 0.f;
+  bool my_lse = false;
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+    if (with_lse && cc == r && u[0].live[r]) {
+      my_lse = true;
+      l = a.src_lse[lse_index(a.src_bsh != 0, u[0].b[r], u[0].h[r], u[0].s[r], a.H, a.Sq)];
+    }
+  float x[8];
+  if (a.src_fp32) {
+    const float* q = reinterpret_cast<const float*>(a.src_out) + u[0].elem + 4 * cc;
+    u32x4 v0 = u32x4{0u, 0u, 0u, 0u}, v1 = v0;
+    if (live_lo) v0 = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(q));
+    if (live_hi) v1 = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(q + 64));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      x[i] = __uint_as_float(v0[i]);
+      x[4 + i] = __uint_as_float(v1[i]);
+    }
+  } else {
+    const uint16_t* q = reinterpret_cast<const uint16_t*>(a.src_out) + u[0].elem + 4 * cc;
+    u32x2 g0 = u32x2{0u, 0u}, g1 = g0;
+    if (live_lo) g0 = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(q));
+    if (live_hi) g1 = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(q + 64));
+    x[0] = __uint_as_float(g0.x << 16); x[1] = __uint_as_float(g0.x & 0xffff0000u);
+    x[2] = __uint_as_float(g0.y << 16); x[3] = __uint_as_float(g0.y & 0xffff0000u);
+    x[4] = __uint_as_float(g1.x << 16); x[5] = __uint_as_float(g1.x & 0xffff0000u);
+    x[6] = __uint_as_float(g1.y << 16); x[7] = __uint_as_float(g1.y & 0xffff0000u);
+  }
+  if (a.dst_fp32) {
+    float* q = reinterpret_cast<float*>(a.dst_out) + u[0].elem + 4 * cc;
+    u32x4 v0, v1;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v0[i] = __float_as_uint(x[i]);
+      v1[i] = __float_as_uint(x[4 + i]);
+    }
+    if (live_lo) __builtin_nontemporal_store(v0, reinterpret_cast<u32x4*>(q));
+    if (live_hi) __builtin_nontemporal_store(v1, reinterpret_cast<u32x4*>(q + 64));
+  } else {
+    uint16_t* q = reinterpret_cast<uint16_t*>(a.dst_out) + u[0].elem + 4 * cc;
+    u32x2 g0, g1;
+    g0.x = pack_bf16x2(x[0], x[1]);
+    g0.y = pack_bf16x2(x[2], x[3]);
+    g1.x = pack_bf16x2(x[4], x[5]);
+    g1.y = pack_bf16x2(x[6], x[7]);
+    if (live_lo) __builtin_nontemporal_store(g0, reinterpret_cast<u32x2*>(q));
+    if (live_hi) __builtin_nontemporal_store(g1, reinterpret_cast<u32x2*>(q + 64));
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+    if (my_lse && cc == r)
+      a.dst_lse[lse_index(a.dst_bsh != 0, u[0].b[r], u[0].h[r], u[0].s[r], a.H, a.Sq)] = l;
 }
 
 // bf16 state -> fp32 state (a cache load): `out` is an elementwise widening in the same element order,
@@ -673,20 +766,11 @@ int launch_merge(const MergeArgs& a, int D, hipStream_t stream) {
   }
   const int R = 128 / D;   // rows per unit
   const int64_t units = ((int64_t)a.B * a.Sq * a.H + R - 1) / R;
-  const bool tiled = (D == 64 || a.n >= kTiledFrom) && a.H % (R * kTileHeadUnits) == 0;
+  const bool tiled = (D == 64 || a.n >= kTiledFrom) && unit_tiles_fit(a.H, D);
   int passes;
   if (D == 64) passes = units >= kTwoPassUnits ? 2 : 1;
   else passes = a.n >= kTiledFrom ? 2 : 1;
-  const int units_per_wg = kUnitsPerPass * passes;
-  int64_t wgs;
-  if (tiled) {
-    const int tile_q = units_per_wg / kTileHeadUnits;
-    // pairs of query tiles, 8 pairs (one per XCD) x 2 workgroups at a time
-    const int64_t n_qt2 = ((a.Sq + tile_q - 1) / tile_q + 1) / 2;
-    wgs = 16 * (((int64_t)a.B * n_qt2 * (a.H / (R * kTileHeadUnits)) + 7) / 8);
-  } else {
-    wgs = (units + units_per_wg - 1) / units_per_wg;
-  }
+  const int64_t wgs = unit_grid(a.B, a.Sq, a.H, D, tiled, passes);
   if (wgs <= 0) return DT_OK;
   if (wgs > 0x7fffffffLL) {
     set_error("merge grid too large");
@@ -735,6 +819,18 @@ int launch_copy(const CopyArgs& a, int D, hipStream_t stream) {
     hipLaunchKernelGGL(state_widen_kernel, dim3((unsigned)(w_out + w_lse)), dim3(kConvThreads),
                        with_lse ? (size_t)lse_run * a.H * 4 : 0, stream, a, groups, (uint32_t)w_lse, lse_run);
     return hip_fail(hipGetLastError(), "state_widen launch");
+  }
+  if (D == 64 && unit_tiles_fit(a.H, D)) {
+    // two neighbouring rows per lane group, query x head tiles (fp32 -> slot at 714 336 rows: 5.70 against 5.44 TB/s
+    // for the row mapping; at D = 128 the row mapping with its contiguous lse runs is the faster one, 6.3 against 6.0)
+    const int64_t wgs = unit_grid(a.B, a.Sq, a.H, D, true, 1);
+    if (wgs <= 0) return DT_OK;
+    if (wgs > 0x7fffffffLL) {
+      set_error("copy grid too large");
+      return DT_ERR_INVALID;
+    }
+    hipLaunchKernelGGL((state_copy_units_kernel<64, MAP_TILED>), dim3((unsigned)wgs), dim3(kThreads), 0, stream, a);
+    return hip_fail(hipGetLastError(), "state_copy_units launch");
   }
   const int rows_per_wg = kThreads / (D / 8) * kCopyRows;
   const int n_st = (a.Sq + rows_per_wg - 1) / rows_per_wg;

@@ -253,9 +253,11 @@ def test_merge_many_states_in_place_with_row_layout_lse(hip, D):
     assert (a_lse.cpu().squeeze(-1).transpose(1, 2) - ref_lse).abs().max() < 1e-5
 
 
-def test_cache_store_load_roundtrip(hip):
-    B, Sq, H, D = 2, 131, 3, 64
-    g = torch.Generator().manual_seed(9)
+@pytest.mark.parametrize("B,Sq,H,D", [(2, 131, 3, 64), (2, 131, 8, 64), (1, 19, 48, 64), (3, 77, 16, 128), (1, 5, 5, 128)])
+def test_cache_store_load_roundtrip(hip, B, Sq, H, D):
+    """fp32 state with a [B,S,H,1] lse -> slot -> fp32.  At D = 64 head counts that divide into tiles of 8 heads
+    take the kernel that moves two neighbouring rows per lane group, the others the row-mapped one."""
+    g = torch.Generator().manual_seed(9 + H)
     src = torch.randn(B, Sq, H, D, generator=g)
     lse = torch.randn(B, Sq, H, 1, generator=g)
     slot_out = torch.empty(B, Sq, H, D, dtype=torch.bfloat16, device="cuda")
