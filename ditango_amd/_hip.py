@@ -140,20 +140,22 @@ def _check_qkv(q: torch.Tensor, name: str = "q") -> None:
 
 
 def lse_layout_of(lse: torch.Tensor, B: int, S: int, H: int) -> int:
-    """Classify an lse tensor as [B,H,S] or [B,S,H(,1)] storage; it must be dense in that order."""
-    if lse.dim() == 4 and lse.shape[-1] == 1:
+    """Classify an lse tensor as [B,H,S] or [B,S,H(,1)] storage; it must be dense in that order.  Where the
+    shape alone cannot tell (S == H), a 4-D tensor is read as the running layout [B,S,H,1] of utils.py:49 and a
+    3-D tensor as flash-attn's [B,H,S]."""
+    four_d = lse.dim() == 4 and lse.shape[-1] == 1
+    if four_d:
         lse = lse.squeeze(-1)
     _require(lse.dim() == 3 and lse.dtype == torch.float32, "lse must be fp32 with 3 (or 4, last=1) dims")
-    if tuple(lse.shape) == (B, H, S):
-        if lse.is_contiguous():
-            return DT_LSE_BHS
-        if lse.transpose(1, 2).is_contiguous():
-            return DT_LSE_BSH
-    if tuple(lse.shape) == (B, S, H):
-        if lse.is_contiguous():
-            return DT_LSE_BSH
-        if lse.transpose(1, 2).is_contiguous():
-            return DT_LSE_BHS
+    named = [((B, S, H), DT_LSE_BSH, DT_LSE_BHS), ((B, H, S), DT_LSE_BHS, DT_LSE_BSH)]
+    if not four_d:
+        named.reverse()
+    for shape, as_is, transposed in named:
+        if tuple(lse.shape) == shape:
+            if lse.is_contiguous():
+                return as_is
+            if lse.transpose(1, 2).is_contiguous():
+                return transposed
     raise DitangoHipError(f"lse of shape {tuple(lse.shape)} / strides {lse.stride()} is not a dense [B,H,S] or [B,S,H]")
 
 

@@ -139,3 +139,18 @@ def test_mask_mode_arena_consults_the_memory_guard(ditango_env):
     assert c.arena_valid == [False] * 8
     c.clear()                                                                   # the reference's clear() keeps the states
     assert c.arena_out is not None
+
+
+def test_lse_layout_when_query_and_head_counts_coincide():
+    """With Sq == H the shape cannot tell [B,H,S] from [B,S,H]: a 4-D [.,.,.,1] tensor is the running layout of
+    utils.py:49 ([B,S,H,1]), a 3-D one flash-attn's [B,H,S]; everywhere else shape and strides decide."""
+    import torch
+    from ditango_amd._hip import DT_LSE_BHS, DT_LSE_BSH, DitangoHipError, lse_layout_of
+    assert lse_layout_of(torch.zeros(2, 5, 5, 1), 2, 5, 5) == DT_LSE_BSH
+    assert lse_layout_of(torch.zeros(2, 5, 5), 2, 5, 5) == DT_LSE_BHS
+    assert lse_layout_of(torch.zeros(1, 5, 7, 1), 1, 5, 7) == DT_LSE_BSH
+    assert lse_layout_of(torch.zeros(1, 7, 5), 1, 5, 7) == DT_LSE_BHS
+    assert lse_layout_of(torch.zeros(1, 7, 5).transpose(1, 2), 1, 5, 7) == DT_LSE_BHS      # a view of [B,H,S] storage
+    assert lse_layout_of(torch.zeros(1, 5, 7).transpose(1, 2), 1, 5, 7) == DT_LSE_BSH
+    with pytest.raises(DitangoHipError):
+        lse_layout_of(torch.zeros(1, 6, 7), 1, 5, 7)
