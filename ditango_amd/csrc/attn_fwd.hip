@@ -182,10 +182,10 @@ __device__ __forceinline__ s16x4 lds_read_tr(const uint8_t* p) {
 // Raw buffer descriptor: base address, stride 0, number of valid bytes, flags.
 __device__ __forceinline__ u32x4 make_rsrc(const void* base, uint32_t valid_bytes) {
   const uint64_t p = reinterpret_cast<uint64_t>(base);
-  u32x4 r;
-  r.x = (uint32_t)p;
-  r.y = (uint32_t)(p >> 32) & 0xffffu;
-  r.z = valid_bytes;
+  u32x4 r;   // uniform by construction; say so, the descriptor then lives in scalar registers
+  r.x = __builtin_amdgcn_readfirstlane((uint32_t)p);
+  r.y = __builtin_amdgcn_readfirstlane((uint32_t)(p >> 32) & 0xffffu);
+  r.z = __builtin_amdgcn_readfirstlane(valid_bytes);
   r.w = (uint32_t)kRsrcFlags;
   return r;
 }
@@ -327,18 +327,30 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
   // (ahead of the compute cursor: base pointers of the tile and keys left in its chunk) and
   // the compute cursor (keys left in the chunk of the tile whose scores are being computed).
   int ld_seg = seg_begin - 1, ld_left = 0;
-  const uint8_t* ld_k = nullptr;
-  const uint8_t* ld_v = nullptr;
   int cp_seg = seg_begin - 1, cp_left = 0;
-  auto ld_next_chunk = [&]() {
+  // The load cursor addresses a tile as (buffer descriptor of its chunk, byte offset of its first key from the
+  // chunk's first key).  The descriptors (base of the chunk's keys for this batch and head, number of valid
+  // bytes) only change with the chunk; per tile the cursor moves one scalar offset.  A chunk's (batch, head)
+  // plane is below 2 GiB (checked on the host), so offsets fit 32 bits with room for the lane's part.
+  const uint32_t row_bytes = (uint32_t)a.kv_ss * 2u;
+  const uint32_t tile_bytes = (uint32_t)kBK * row_bytes;
+  u32x4 rk = make_rsrc(nullptr, 0u), rv = rk;   // K and V of the chunk under the load cursor
+  uint32_t k_off = 0u;
+  auto ld_next_chunk = [&]() __attribute__((always_inline)) {
     do { ++ld_seg; } while (ld_seg < seg_end && kv_len_of(ld_seg) == 0);
+    k_off = 0u;
     if (ld_seg < seg_end) {
       const int cid = chunk_of(ld_seg);
       const int64_t head_off =
           (int64_t)b * a.kv_sb[cid] + (int64_t)h * a.kv_sh + (int64_t)kv_begin_of(ld_seg) * a.kv_ss;
-      ld_k = reinterpret_cast<const uint8_t*>(a.k[cid] + head_off);
-      ld_v = reinterpret_cast<const uint8_t*>(a.v[cid] + head_off);
       ld_left = kv_len_of(ld_seg);
+      const uint32_t valid = (uint32_t)(ld_left - 1) * row_bytes + (uint32_t)(D * 2);
+      rk = make_rsrc(a.k[cid] + head_off, valid);
+      rv = make_rsrc(a.v[cid] + head_off, valid);
+    } else {
+      // past the last chunk: an empty descriptor, loads store zeros without touching memory
+      rk = make_rsrc(nullptr, 0u);
+      rv = rk;
     }
   };
   auto cp_next_chunk = [&]() {
@@ -358,8 +370,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
         skip -= in_chunk;
         ld_next_chunk();
       } else {
-        ld_k += (int64_t)skip * kBK * ((int64_t)a.kv_ss * 2);
-        ld_v += (int64_t)skip * kBK * ((int64_t)a.kv_ss * 2);
+        k_off += (uint32_t)skip * tile_bytes;
         ld_left -= skip * kBK;
         skip = 0;
       }
@@ -383,11 +394,11 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
   // wave + 8 i = rows kRowsPerBlock * (wave + 8 i) ...).  Lane L of a load lands at LDS bytes
   // 16 L .. 16 L + 15 of the block, i.e. at row L / kChunks, chunk position L % kChunks; it
   // therefore fetches the chunk of global memory that the swizzle assigns to that position.
-  // Raw buffer loads: the descriptor (base of the tile's first key for this batch and head,
-  // number of valid bytes) lives in scalar registers, and rows past the end of the chunk fail
+  // Raw buffer loads: the descriptor (base of the chunk's first key for this batch and head,
+  // number of valid bytes) lives in scalar registers, the tile's offset from there travels as the
+  // load's scalar offset (which the range check includes), and rows past the end of the chunk fail
   // the hardware bounds check and arrive as zeros (their scores are masked to -inf; zero V rows
   // add nothing).
-  const uint32_t row_bytes = (uint32_t)a.kv_ss * 2u;
   uint32_t k_goff, v_goff;  // this lane's byte offset from the tile's first key, loop invariant
   {
     const int lrow = T::kRowsPerBlock * wave + lane / T::kChunks;  // + 8 * kRowsPerBlock * i
@@ -396,39 +407,41 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
     v_goff = (uint32_t)lrow * row_bytes + 16u * (uint32_t)((((pos >> 2) ^ T::swz_v(lrow)) << 2) | (pos & 3));
   }
   static_assert((8 * T::kRowsPerBlock) % 16 == 0, "the swizzle must not depend on the load index");
-  const int64_t tile_bytes = (int64_t)kBK * row_bytes;
   typedef __attribute__((address_space(3))) uint8_t* lds_ptr_t;
   const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
+  const uint32_t block_step = (uint32_t)(8 * T::kRowsPerBlock) * row_bytes;   // from a wavefront's block to its next one
   // Issues this wavefront's loads of V of the tile before the one under the load cursor and of
   // K of the tile under it (tile X, into K buffer X & 3; V is needed two phases later than K, so
-  // its loads run one tile behind and reuse the descriptor the previous call made for K), and
-  // moves the cursor on.  Past the last tile the loads are still issued, against an empty descriptor (they store
-  // zeros without touching memory): with the same number of loads in every iteration the counter
-  // the barrier waits on is static.
-  const uint8_t* prev_v = nullptr;  // V of the tile the previous call loaded K of
-  uint32_t prev_valid = 0u;
+  // its loads run one tile behind), and moves the cursor on.  Past the last tile the loads are still
+  // issued, against an empty descriptor (they store zeros without touching memory): with the same
+  // number of loads in every iteration the counter the barrier waits on is static.
+  // V of the previous tile: its offset, and -- only in the call after the cursor changed chunks -- the
+  // descriptor of the chunk it belongs to.
+  uint32_t v_off = 0u;
+  u32x4 rv_old = make_rsrc(nullptr, 0u);   // the very first call has no previous tile: zeros into a buffer nobody reads
+  bool v_lags = true;
   auto load_tile = [&](int kbuf) __attribute__((always_inline)) {
-    const bool have = __builtin_expect(ld_seg < seg_end, 1);
-    const uint32_t valid = have ? (uint32_t)(ld_left - 1) * row_bytes + (uint32_t)(D * 2) : 0u;
-    const u32x4 rk = make_rsrc(ld_k, valid);
-    const u32x4 rv = make_rsrc(prev_v, prev_valid);
-    prev_v = ld_v;
-    prev_valid = valid;
     const int vbuf = (kbuf + kNumBuf - 1) & (kNumBuf - 1);
     const uint32_t kdst = lds_base + kbuf * T::kBytesK + wave * 1024;
     const uint32_t vdst = lds_base + T::kOffV + vbuf * T::kBytesV + wave * 1024;
     // V first: the barrier waits let the K half of a call stay in flight one vector phase longer
+    if (__builtin_expect(v_lags, 0)) {
 #pragma unroll
-    for (int i = 0; i < T::kLoads; ++i)
-      load_block_to_lds(rv, v_goff, (uint32_t)(i * 8 * T::kRowsPerBlock) * row_bytes, vdst + i * 8192);
+      for (int i = 0; i < T::kLoads; ++i) load_block_to_lds(rv_old, v_goff, v_off + i * block_step, vdst + i * 8192);
+      v_lags = false;
+    } else {
 #pragma unroll
-    for (int i = 0; i < T::kLoads; ++i)
-      load_block_to_lds(rk, k_goff, (uint32_t)(i * 8 * T::kRowsPerBlock) * row_bytes, kdst + i * 8192);
-    if (have) {
-      ld_left -= kBK;
-      ld_k += tile_bytes;
-      ld_v += tile_bytes;
-      if (__builtin_expect(ld_left <= 0, 0)) ld_next_chunk();
+      for (int i = 0; i < T::kLoads; ++i) load_block_to_lds(rv, v_goff, v_off + i * block_step, vdst + i * 8192);
+    }
+#pragma unroll
+    for (int i = 0; i < T::kLoads; ++i) load_block_to_lds(rk, k_goff, k_off + i * block_step, kdst + i * 8192);
+    v_off = k_off;
+    k_off += tile_bytes;
+    ld_left -= kBK;
+    if (__builtin_expect(ld_left <= 0 && ld_seg < seg_end, 0)) {
+      rv_old = rv;
+      v_lags = true;
+      ld_next_chunk();
     }
   };
 

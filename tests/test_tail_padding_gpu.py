@@ -25,7 +25,7 @@ def _padded(B, S, H, D, g, pad):
 
 
 @pytest.mark.parametrize("D", [64, 128])
-@pytest.mark.parametrize("Sk", [1, 17, 32, 33, 47, 63, 64 + 5, 64 + 40, 128 + 31, 128 + 32, 128 + 60])
+@pytest.mark.parametrize("Sk", [1, 17, 32, 33, 47, 63, 64 + 5, 64 + 40, 128 + 31, 128 + 32, 128 + 60, 64 * 9 + 5, 64 * 20 + 33])
 def test_rows_behind_a_chunk_are_never_read_as_data(hip, D, Sk):
     B, Sq, H = 2, 70, 3
     print(f"case padding D={D} Sk={Sk}", flush=True)
@@ -72,3 +72,27 @@ def test_rows_between_segments_are_never_read_as_data(hip, D):
         ro, rl = om.chunk_attention(q[:, 50 * i:50 * i + 50], k[:, b:b + n], v[:, b:b + n])
         assert (out[:, 50 * i:50 * i + 50].float().cpu() - ro).abs().max().item() <= OUT_TOL, f"segment {i}"
         assert (lse[:, :, 50 * i:50 * i + 50].cpu() - rl).abs().max().item() <= LSE_TOL, f"segment {i}"
+
+
+@pytest.mark.parametrize("D", [64, 128])
+def test_rows_behind_every_chunk_of_a_multi_chunk_job(hip, D):
+    """One job over three chunks of ragged lengths (the tile cursor moves from chunk to chunk while V still loads
+    from the previous one): NaN behind each of them."""
+    B, Sq, H = 1, 300, 2
+    g = torch.Generator().manual_seed(5 + D)
+    q = torch.randn(B, Sq, H, D, generator=g).bfloat16()
+    lens = [64 * 3 + 7, 40, 64 * 5 + 33]
+    cpu, dev = [], []
+    for n in lens:
+        (k, dk), (v, dv) = _padded(B, n, H, D, g, 80), _padded(B, n, H, D, g, 80)
+        cpu.append((k, v))
+        dev.append((dk, dv))
+    table = hip.ChunkTable([d[0] for d in dev], [d[1] for d in dev])
+    out = torch.empty(B, Sq, H, D, dtype=torch.bfloat16, device="cuda")
+    lse = torch.empty(B, H, Sq, dtype=torch.float32, device="cuda")
+    hip.attn_jobs_fwd(q.cuda(), table, [[0, 1, 2]], [out], [lse])
+    torch.cuda.synchronize()
+    ref_out, ref_lse = om.chunk_attention(q, torch.cat([c[0] for c in cpu], 1), torch.cat([c[1] for c in cpu], 1))
+    assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all(), "NaN rows behind a chunk leaked"
+    assert (out.float().cpu() - ref_out).abs().max().item() <= OUT_TOL
+    assert (lse.cpu() - ref_lse).abs().max().item() <= LSE_TOL
