@@ -218,6 +218,32 @@ def test_merge_row_mappings(hip, B, Sq, H, D, n):
     assert lse_close(dst_l.cpu().squeeze(-1).transpose(1, 2))
 
 
+@pytest.mark.parametrize("D,H", [(64, 8), (128, 4), (128, 3)])
+@pytest.mark.parametrize("order", ["ascending", "descending", "spiky"])
+def test_merge_rescales_across_batches(hip, D, H, order):
+    """States are folded in batches of 8 with a running maximum.  lse values that grow (every batch rescales what was
+    accumulated), shrink (later batches underflow to nothing) or jump by +-60 between neighbours: against the closed
+    form in fp64."""
+    B, Sq, n = 1, 41, 29
+    g = torch.Generator().manual_seed(17 + D + H)
+    outs = [torch.randn(B, Sq, H, D, generator=g).bfloat16() for _ in range(n)]
+    base = torch.randn(B, H, Sq, generator=g)
+    if order == "ascending":
+        lses = [base + 7.0 * i for i in range(n)]
+    elif order == "descending":
+        lses = [base - 7.0 * i for i in range(n)]
+    else:
+        lses = [base + (60.0 if i % 3 == 0 else -60.0 if i % 3 == 1 else 0.0) + torch.randn(B, H, Sq, generator=g) for i in range(n)]
+    lw = torch.stack([l.double() for l in lses])                       # [n,B,H,Sq]
+    ref_lse = torch.logsumexp(lw, 0)
+    w = torch.exp(lw - ref_lse).permute(0, 1, 3, 2).unsqueeze(-1)      # [n,B,Sq,H,1]
+    ref_out = (w * torch.stack([o.double() for o in outs])).sum(0)
+    o, l = hip.merge_states([x.cuda() for x in outs], [x.cuda() for x in lses])
+    torch.cuda.synchronize()
+    assert (l.cpu().double() - ref_lse).abs().max() < 1e-4 * max(1.0, float(ref_lse.abs().max()) / 16)
+    assert (o.cpu().double() - ref_out).abs().max() < 1e-5
+
+
 def test_merge_large_launch_d64(hip):
     """A D = 64 launch of more than 2^20 lane groups takes two tile passes per workgroup."""
     B, Sq, H, D, n = 1, 16400, 128, 64, 2
