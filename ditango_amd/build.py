@@ -18,6 +18,7 @@ ROOT = PKG.parent
 CSRC = PKG / "csrc"
 LIB_DIR = PKG / "lib"
 LIB_PATH = LIB_DIR / "libditango_hip.so"
+DEMO_PATH = LIB_DIR / "dt_capi_demo"
 SOURCES = ["attn_fwd.hip", "attn_f32.hip", "state_ops.hip", "producer.hip", "capi.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -52,6 +53,12 @@ def build_lib(verbose: bool = False, extra_flags=()) -> Path:
     with ThreadPoolExecutor(max_workers=min(5, len(SOURCES))) as ex:
         objs = list(ex.map(compile_one, SOURCES))
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objs), "-o", str(LIB_PATH)]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    _run(cmd)
+    # a host program that uses nothing but the C header and the HIP runtime (tests/test_capi_demo_gpu.py runs it)
+    cmd = [HIPCC, "-O2", "-std=c++17", "-Wno-unused-result", f"-I{ROOT / 'include'}", str(CSRC / "capi_demo.cpp"),
+           f"-L{LIB_DIR}", "-lditango_hip", "-Wl,-rpath,$ORIGIN", "-o", str(DEMO_PATH)]
     if verbose:
         print(" ".join(cmd), flush=True)
     _run(cmd)
