@@ -379,6 +379,23 @@ def run_workload(name, args, steps, warmup, main, reuse=None, kernels_only=False
         mfma_probe = {"tflops": round(probe_flops[0] / (kp_ms * 1e-3) / 1e12, 1), "launch_ms": round(kp_ms, 4),
                       "clock_mhz_under_load": sample_clock_mhz(probe_launch, seconds=1.5)}
     del q_folded
+    # the co-issue yardstick: one wavefront of each SIMD issues MFMAs, the other the softmax's vector instructions
+    # per MFMA at this head dimension; the MFMA rate with the softmax against the rate without is the ceiling of the
+    # attention kernel's MFMA utilisation before any LDS traffic, barrier or tile load
+    coissue = None
+    if not kernels_only:
+        co_sink = torch.zeros(1, dtype=torch.float32, device=dev)
+        co_wgs, co_iters = 256 * 8, 4096
+        co_flops = [0.0]
+
+        def co_launch(with_softmax):
+            co_flops[0] = _hip.coissue_probe(co_wgs, co_iters, D, with_softmax, co_sink)
+
+        co0_ms = time_kernel(lambda: co_launch(False), reps)
+        co1_ms = time_kernel(lambda: co_launch(True), reps)
+        coissue = {"mfma_alone_tflops": round(co_flops[0] / (co0_ms * 1e-3) / 1e12, 1),
+                   "mfma_beside_softmax_tflops": round(co_flops[0] / (co1_ms * 1e-3) / 1e12, 1),
+                   "mfma_share_beside_softmax": round(co0_ms / co1_ms, 4)}
 
     # merge of all C states of a layer into the fp32 result, rotating over the layers' arenas
     dst_n = max(1, min(8, int(1.2e9 // (rows * (4 * D + 4))) + 1))
@@ -441,6 +458,9 @@ def run_workload(name, args, steps, warmup, main, reuse=None, kernels_only=False
         roofline["mfma_probe_tflops"] = mfma_probe["tflops"]
         roofline["mfma_probe_clock_mhz"] = mfma_probe["clock_mhz_under_load"]
         roofline["frac_of_mfma_probe"] = round(k1_tflops / mfma_probe["tflops"], 4)
+    if coissue:
+        roofline["coissue_probe"] = coissue
+        roofline["frac_of_coissue_ceiling"] = round(k1_tflops / coissue["mfma_beside_softmax_tflops"], 4)
     roofline_merge = {"kernel": "merge_states_kernel<%d>" % D, "bound": "hbm", "achieved": round(k2_gbs, 1),
                       "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(k2_gbs / PEAK_HBM_GBS, 4),
                       "traffic": k2_traffic, "launch_us": round(k2_ms * 1e3, 2), "bytes_per_launch": k2_bytes,
@@ -462,7 +482,9 @@ def run_workload(name, args, steps, warmup, main, reuse=None, kernels_only=False
                "layer_attn_tflops": round(layer_tflops, 1),
                "attn": {"frac": roofline["frac"], "tflops": roofline["achieved"], "chunks_per_launch": n_typ,
                         "launch_ms": roofline["launch_ms"], "single_chunk_frac": round(k1s_tflops / PEAK_BF16_TFLOPS, 4),
-                        "q_prescaled_frac": round(k1p_tflops / PEAK_BF16_TFLOPS, 4), "traffic": k1_traffic},
+                        "q_prescaled_frac": round(k1p_tflops / PEAK_BF16_TFLOPS, 4), "traffic": k1_traffic,
+                        "coissue_probe": coissue,
+                        "frac_of_coissue_ceiling": roofline.get("frac_of_coissue_ceiling")},
                "merge": {"frac": roofline_merge["frac"], "gbs": roofline_merge["achieved"], "states": C,
                          "launch_us": roofline_merge["launch_us"], "read_probe_gbs": roofline_merge["read_probe_gbs"],
                          "traffic": k2_traffic},

@@ -75,6 +75,7 @@ _SIGNATURES = {
     "dt_build_schedule_table": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp, c_vp]),
     "dt_hbm_read_probe": (ctypes.c_int, [_P(c_vp), c_i32, c_i64, c_vp, c_vp]),
     "dt_mfma_probe": (ctypes.c_int, [c_i32, c_i32, c_vp, c_vp]),
+    "dt_coissue_probe": (ctypes.c_int, [c_i32, c_i32, c_i32, c_i32, c_vp, c_vp]),
     "dt_rel_l1_sums": (ctypes.c_int, [c_vp, c_vp, c_i64, c_vp, c_vp]),
     "dt_qk_norm_rope": (ctypes.c_int, [c_vp, c_i64, c_i64, c_i64, c_vp, c_i32, c_i32, c_i32, c_i32,
                                        c_i32, c_vp, c_vp, c_f32, c_i32, c_vp, c_vp, c_i64, c_i32, c_i32,
@@ -564,6 +565,17 @@ def mfma_probe(workgroups: int, iters: int, sink: torch.Tensor) -> float:
     rc = lib.dt_mfma_probe(int(workgroups), int(iters), sink.data_ptr(), _stream())
     _check(rc, "dt_mfma_probe")
     return float(workgroups) * 8 * 4 * iters * 32768.0
+
+
+def coissue_probe(workgroups: int, iters: int, head_dim: int, with_softmax: bool, sink: torch.Tensor) -> float:
+    """Launch the co-issue probe (one wavefront of each SIMD issues MFMAs; with ``with_softmax`` the other one
+    issues the softmax's vector instructions per MFMA at that head dimension) and return the FLOP of the
+    launch: ``workgroups * 4`` wavefronts x ``4 * iters`` bf16 MFMAs of 32 x 32 x 16."""
+    lib = load_library()
+    _require(sink.is_cuda and sink.numel() * sink.element_size() >= 4, "sink must be a device tensor of at least 4 bytes")
+    rc = lib.dt_coissue_probe(int(workgroups), int(iters), int(head_dim), int(bool(with_softmax)), sink.data_ptr(), _stream())
+    _check(rc, "dt_coissue_probe")
+    return float(workgroups) * 4 * 4 * iters * 32768.0
 
 
 def rel_l1_sums(a: torch.Tensor, b: torch.Tensor, sums: Optional[torch.Tensor] = None) -> torch.Tensor:

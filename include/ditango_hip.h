@@ -323,6 +323,21 @@ int dt_hbm_read_probe(const void* const* streams, int32_t n_streams, int64_t byt
 int dt_mfma_probe(int32_t workgroups, int32_t iters, float* sink, void* stream);
 
 /*
+ * Measurement aid, no counterpart in the reference: the same launch shape, but only ONE wavefront of each
+ * SIMD issues the 4 * iters MFMAs (a launch does workgroups * 4 * 4 * iters * 32768 FLOP); with
+ * with_softmax != 0 the other wavefront of the SIMD issues, per MFMA of its neighbour, the vector
+ * instructions that the online softmax of dt_attn_* spends per MFMA at that head dimension: at 128 one
+ * v_fma_f32, one v_exp_f32, one v_add_f32 and half a v_cvt_pk_bf16_f32; at 64 twice that.  The launch
+ * reserves the attention kernel's LDS for head_dim, so one (128) or two (64) workgroups share a CU as
+ * they do there.  The MFMA rate with the softmax against the rate without is the share of the matrix pipe
+ * that the wavefronts of a SIMD can keep busy side by side for that instruction mix: the ceiling of the
+ * attention kernel's MFMA utilisation before any LDS traffic, barrier or tile load.  sink: one device
+ * word, (almost) never written.
+ */
+int dt_coissue_probe(int32_t workgroups, int32_t iters, int32_t head_dim, int32_t with_softmax, float* sink,
+                     void* stream);
+
+/*
  * Producer side of an attention call: normalise every head row of x over D, apply the
  * rotary position embedding to the token rows [rope_begin, rope_end) and write the result
  * as bf16 [B,S,H,D] contiguous, the layout the attention entry points read -- one pass over

@@ -302,6 +302,18 @@ def test_mfma_probe_runs_and_checks_its_arguments(hip):
             hip.mfma_probe(*bad, sink)
 
 
+def test_coissue_probe_runs_and_checks_its_arguments(hip):
+    sink = torch.zeros(1, dtype=torch.float32, device="cuda")
+    for D in (64, 128):
+        for with_softmax in (False, True):
+            flop = hip.coissue_probe(64, 16, D, with_softmax, sink)
+            torch.cuda.synchronize()
+            assert flop == 64 * 4 * 4 * 16 * 32768.0 and float(sink) == 0.0
+    for bad in ((0, 16, 128), (64, 0, 128), (64, 6, 64), (64, 16, 96)):
+        with pytest.raises(hip.DitangoHipError):
+            hip.coissue_probe(*bad, True, sink)
+
+
 def test_cache_load_into_given_tensors(hip):
     B, S, H, D = 1, 70, 2, 64
     g = torch.Generator().manual_seed(9)
