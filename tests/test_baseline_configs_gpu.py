@@ -388,3 +388,59 @@ def test_stride_mode_at_full_size(env, hip):
         vs = [v + 0.01 * torch.randn(v.shape, generator=g, device="cuda") for v in vs]
         del kb, vb
     print(f"stride full-size worst: out max-abs {worst[0]:.3e} rel-l2 {worst[1]:.3e} lse {worst[2]:.3e}", flush=True)
+
+
+def test_varlen_mask_mode_at_full_size(env, hip):
+    """HunyuanVideo's real entry at its per-rank shape: a packed batch of two segments per sample (14 818 video + 64
+    text query rows; every chunk's keys split the same way), under the seeded Bernoulli(0.6) mask, three steps of one
+    layer.  The oracle evaluates each segment's sampled query rows against that segment's keys of every computed
+    chunk and keeps the cached states (rounded to bf16) for the reused ones."""
+    from ditango_amd.core.attention import proAttention
+    from ditango_amd.core.parallel_state import get_usp_group
+    from ditango_amd.core.redundancy_map import make_bernoulli_mask
+    from ditango_amd.utils import update_timestep
+
+    B, H, D, Sq, lens, T, L, p, diag, norm = CONFIGS["hunyuanvideo"]
+    C, n_txt = len(lens), 64
+    cu = [0, Sq - n_txt, Sq]
+    rm = env(C, 0, T, L)
+    mask = make_bernoulli_mask(T, L, C, p, seed=0, diag=diag)
+    rm.set_chunk_mask(mask, diag=diag)
+    q, ks, vs = _make(CONFIGS["hunyuanvideo"], seed=1)
+    g = torch.Generator().manual_seed(9)
+    rows0 = torch.sort(torch.randperm(cu[1], generator=g)[:24]).values
+    rows1 = torch.sort(torch.randperm(n_txt, generator=g)[:8]).values + cu[1]
+    rows = torch.cat([rows0, rows1])
+    layer = 7
+    group = get_usp_group()
+    attn = proAttention(layer, group)
+    cu_t = torch.tensor(cu, dtype=torch.int32)
+    cached = {}
+    for t in range(3):
+        update_timestep(t)
+        dk, dv = [k.cuda() for k in ks], [v.cuda() for v in vs]
+        group.set_kv_chunks([k[0] for k in dk], [v[0] for v in dv], cu_seqlens_kv=[cu_t] * C)
+        out = attn.varlen_attn(q[0].cuda(), dk[diag][0], dv[diag][0], cu_t, cu_t, cu[1], cu[1])
+        torch.cuda.synchronize()
+        compute, reuse = ms.build_schedule(mask[t, layer], diag)
+        n = int(rm.sched_counts_host[t, layer, 0])
+        assert rm.sched_compute_ids[t, layer, :n].tolist() == list(compute)
+        states = [cached[c] for c in reuse]
+        for c in compute:
+            o0, l0 = om.chunk_attention(q[:, rows0], ks[c][:, :cu[1]], vs[c][:, :cu[1]])
+            o1, l1 = om.chunk_attention(q[:, rows1], ks[c][:, cu[1]:], vs[c][:, cu[1]:])
+            st = (torch.cat([o0, o1], 1), torch.cat([l0, l1], 2))
+            if c != diag:
+                st = (om.bf16_round(st[0]), st[1])
+                cached[c] = st
+            states.append(st)
+        ref_out, ref_lse = om.merge_states_closed_form([s[0] for s in states], [s[1] for s in states])
+        got_out = out[rows.cuda()].cpu()[None]
+        got_lse = attn.last_lse[:, rows.cuda()].cpu().squeeze(-1).transpose(1, 2)
+        err = (got_out - ref_out).abs().max().item()
+        lerr = (got_lse - ref_lse).abs().max().item()
+        rel = (got_out - ref_out).norm().item() / ref_out.norm().item()
+        print(f"varlen full-size t={t} computed={compute} reused={reuse}: out max-abs {err:.3e} rel-l2 {rel:.3e} lse {lerr:.3e}", flush=True)
+        assert err <= OUT_TOL and lerr <= LSE_TOL and rel <= 1e-2
+        q = (q.float() + 0.01 * torch.randn(q.shape, generator=g)).bfloat16()
+        del dk, dv
