@@ -311,23 +311,27 @@ def test_attention_is_deterministic_at_full_shapes(hip, H, D, Sq, Sk, prescaled)
                     assert torch.equal(outs[j], ref[0][j]) and torch.equal(lses[j], ref[1][j]), f"run {i} job {j}"
 
 
-def test_stride_mode_at_full_size(env, hip):
-    """The reference's own mode at the HunyuanVideo per-rank shape: ring position 3 of 8, the refined dividers the
-    reference derives from the redundancy map it ships (layer 5 of `tests/golden/stride_schedules.npz`, which has
-    strides 1, 2 and 4 within its first 18 steps), 1 % input drift per step.  The lock-step oracle of all ring
-    positions evaluates attention on a seeded sample of query rows (all heads, all keys) of position 3 and applies the
-    same cache bookkeeping (cached states rounded to bf16); schedule exact, out 2e-2, lse 1e-3."""
+@pytest.mark.parametrize("name,rank,layer,T,want", [("hunyuanvideo", 3, 5, 18, {1, 2, 4}), ("cogvideox", 6, 0, 18, {1, 2, 4}),
+                                                    ("stepvideo", 0, 0, 8, {1, 2})])
+def test_stride_mode_at_full_size(env, hip, name, rank, layer, T, want):
+    """The reference's own mode at the per-rank shapes of the three models: one ring position of 8, the refined dividers
+    the reference derives from the redundancy map it ships for that model (a layer of
+    `tests/golden/stride_schedules.npz` whose first steps use several strides), 1 % input drift per step.  The
+    lock-step oracle of all ring positions evaluates attention on a seeded sample of query rows (all heads, all keys)
+    of that position and applies the same cache bookkeeping (cached states rounded to bf16); schedule exact, out
+    2e-2, lse 1e-3."""
     import os
     from oracle.state_machine import RingOracle, strides_from_dividers
     from ditango_amd.core.attention import proAttention
     from ditango_amd.core.parallel_state import get_usp_group
     from ditango_amd.utils import update_timestep
 
-    N, rank, layer, T = 8, 3, 5, 18
-    B, H, D, S = 1, 24, 128, 14882
-    div = np.load(os.path.join(os.path.dirname(__file__), "golden", "stride_schedules.npz"))["hunyuanvideo/dividers"]
+    N = 8
+    B, H, D, S = CONFIGS[name][:4]
+    div = np.load(os.path.join(os.path.dirname(__file__), "golden", "stride_schedules.npz"))[f"{name}/dividers"]
     col = [int(x) for x in div[:T, layer]]
-    assert {1, 2, 4} <= set(col)
+    assert want <= set(col)
+    print(f"case stride full-size {name}: H={H} D={D} S={S} rank={rank} dividers={col}", flush=True)
     rm = env(N, rank, T, 1)
     rm.divider_map[:, 0] = torch.tensor(col)
     curr, nxt = strides_from_dividers(N, col)
@@ -380,14 +384,14 @@ def test_stride_mode_at_full_size(env, hip):
         lerr = (got_lse - ref_lse).abs().max().item()
         rel = (got_out - ref_out).norm().item() / ref_out.norm().item()
         worst = [max(worst[0], err), max(worst[1], rel), max(worst[2], lerr)]
-        print(f"stride full-size t={t} stride {curr[t]}->{nxt[t]} computed={tr.computed} merged={tr.reuse_merged}: "
+        print(f"stride full-size {name} t={t} stride {curr[t]}->{nxt[t]} computed={tr.computed} merged={tr.reuse_merged}: "
               f"out max-abs {err:.3e} rel-l2 {rel:.3e} lse {lerr:.3e}", flush=True)
         assert err <= OUT_TOL and lerr <= LSE_TOL and rel <= 1e-2
         q = q + 0.01 * torch.randn(q.shape, generator=g, device="cuda")
         ks = [k + 0.01 * torch.randn(k.shape, generator=g, device="cuda") for k in ks]
         vs = [v + 0.01 * torch.randn(v.shape, generator=g, device="cuda") for v in vs]
         del kb, vb
-    print(f"stride full-size worst: out max-abs {worst[0]:.3e} rel-l2 {worst[1]:.3e} lse {worst[2]:.3e}", flush=True)
+    print(f"stride full-size {name} worst: out max-abs {worst[0]:.3e} rel-l2 {worst[1]:.3e} lse {worst[2]:.3e}", flush=True)
 
 
 def test_varlen_mask_mode_at_full_size(env, hip):
