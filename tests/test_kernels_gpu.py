@@ -486,3 +486,21 @@ def test_scheduled_launch_with_split_tail_and_merge_repeat_bit_exactly(hip):
             differing += (a != b).any().long()
     torch.cuda.synchronize()
     assert int(differing) == 0
+
+
+def test_rel_l1_sums_at_the_hunyuan_shape(hip):
+    """The profiling mode's reduction over two fp32 outputs of the HunyuanVideo per-rank shape (45.7 M elements each,
+    a few NaN among them) against the oracle's rel_l1 on the host."""
+    B, S, H, D = 1, 14882, 24, 128
+    g = torch.Generator(device="cuda").manual_seed(31)
+    a = torch.randn(B, S, H, D, generator=g, device="cuda")
+    b = a + 0.05 * torch.randn(B, S, H, D, generator=g, device="cuda")
+    a[0, 7, 3, 5] = float("nan")
+    b[0, 9000, 20, 100] = float("nan")
+    sums = hip.rel_l1_sums(b, a).cpu()
+    torch.cuda.synchronize()
+    d, sa, sb, cnt = [float(x) for x in sums]
+    assert cnt == a.numel() - 2
+    got = (d / cnt) / (sb / cnt + 1e-8)                 # mean|new - ori| / (mean|ori| + 1e-8), new = b, ori = a
+    want = om.rel_l1(b.cpu(), a.cpu())
+    assert abs(got - want) <= 1e-5 * want

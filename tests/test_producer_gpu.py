@@ -191,3 +191,29 @@ def test_rejects_bad_arguments(hip):
         hip.qk_norm_rope(x, norm=7)
     with pytest.raises(hip.DitangoHipError):
         hip.qk_norm_rope(x.float())
+
+
+def test_full_kv_sequence_of_the_hunyuan_shape(hip):
+    """RMSNorm + interleaved RoPE of K over the whole HunyuanVideo KV sequence (119 056 tokens x 24 heads), read in
+    place from a fused "B L (K H D)" projection, the text tokens behind rope_end left unrotated: every output row of
+    a seeded sample of 512 tokens against the oracle, and the rows in between untouched by neighbours (finite)."""
+    B, S, H, D, n_txt = 1, 119056, 24, 128, 256
+    g = torch.Generator(device=DEV).manual_seed(21)
+    qkv = (torch.randn(B, S, 3, H, D, generator=g, device=DEV) * 1.5).to(torch.bfloat16)
+    x = qkv[:, :, 1]                                   # K, strided view
+    gc = torch.Generator().manual_seed(22)
+    w = torch.rand(D, generator=gc) + 0.5
+    cos, sin = _tables(P.ROPE_INTERLEAVED, S - n_txt, D, seed=23)
+    y = hip.qk_norm_rope(x, norm=P.NORM_RMS, weight=w.to(DEV), eps=1e-6, rope=P.ROPE_INTERLEAVED, cos=cos.to(DEV),
+                         sin=sin.to(DEV), rope_begin=0, rope_end=S - n_txt)
+    torch.cuda.synchronize()
+    assert y.shape == (B, S, H, D) and y.is_contiguous() and bool(torch.isfinite(y.float()).all())
+    rows = torch.sort(torch.cat([torch.randperm(S - n_txt, generator=gc)[:448], torch.arange(S - n_txt - 32, S - n_txt + 32)])).values
+    xs = x[:, rows.to(DEV)].cpu()
+    for lo, hi, rot in ((0, int((rows < S - n_txt).sum()), True), (int((rows < S - n_txt).sum()), len(rows), False)):
+        if hi <= lo:
+            continue
+        r = rows[lo:hi]
+        o = P.qk_norm_rope(xs[:, lo:hi], P.NORM_RMS, w, None, 1e-6, P.ROPE_INTERLEAVED if rot else P.ROPE_NONE,
+                           cos[r] if rot else None, sin[r] if rot else None, 0, hi - lo, (), 0)
+        _close(y[:, r.to(DEV)], o)
