@@ -176,7 +176,7 @@ def test_reuse_sweep_shape_properties(env, hip):
         assert err <= OUT_TOL and lerr <= LSE_TOL
 
 
-@pytest.mark.parametrize("frac", [0.5, 0.9])
+@pytest.mark.parametrize("frac", [0.0, 0.25, 0.5, 0.75, 0.9])
 def test_reuse_sweep_at_full_size(env, hip, frac):
     """Configuration 5 as it stands: Q and KV are the full 119 056 tokens, KV in 32 chunks of 3721 / 3720
     keys (the reference's uneven split, utils.py:99-111, without zero padding), H = 24, D = 128, no local
