@@ -514,7 +514,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
   bf16x8 ring[kRing];
   auto v_frag = [&](int vbuf, int i) __attribute__((always_inline)) -> bf16x8 {
     // 8 consecutive keys of one d column = two transposing reads of 4 keys each
-    const int db = i >> 2, kb = (i >> 1) & 1, half = i & 1;
+    const int db = i % (D / 32), kb = (i / (D / 32)) >> 1, half = (i / (D / 32)) & 1;
     const uint8_t* p = lds + vld[db] + vbuf * T::kBytesV + (32 * kb + 16 * half) * T::kRowBytes;
     const s16x4 lo = lds_read_tr(p);
     const s16x4 hi = lds_read_tr(p + 4 * T::kRowBytes);
@@ -532,7 +532,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
     auto frag = [&](int i) -> bf16x8 {
       if (i < kPV) return v_frag(kU, i);
       const int j = i - kPV;
-      const int kb = j / (D / 16), sidx = j % (D / 16);
+      const int kb = j & 1, sidx = j >> 1;
       return *reinterpret_cast<const bf16x8*>(lds + kld[sidx] + kUK * T::kBytesK + kb * 32 * T::kRowBytes);
     };
 #pragma unroll
@@ -540,11 +540,11 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
       const bf16x8 cur = ring[i % kRing];
       if (i + kRing < kFrags) ring[i % kRing] = frag(i + kRing);
       if (i < kPV) {
-        const int db = i >> 2, kb = (i >> 1) & 1, half = i & 1;
+        const int db = i % (D / 32), kb = (i / (D / 32)) >> 1, half = (i / (D / 32)) & 1;
         o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur, p_frag[kb][half], o_acc[db], 0, 0, 0);
       } else {
         const int j = i - kPV;
-        const int kb = j / (D / 16), sidx = j % (D / 16);
+        const int kb = j & 1, sidx = j >> 1;
         if (sidx == 0) {
           f32x16 zero;
 #pragma unroll
