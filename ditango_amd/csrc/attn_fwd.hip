@@ -675,8 +675,13 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
           p.x = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[kb][r], c, -mc));
           p.y = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[kb][r + 1], c, -mc));
         }
-        rs0 += p.x;
-        rs1 += p.y;
+        if (!kPre && kb == 0 && r == 0) {   // the sums start from these two (0 + p is not folded: it would turn -0 into +0)
+          rs0 = p.x;
+          rs1 = p.y;
+        } else {
+          rs0 += p.x;
+          rs1 += p.y;
+        }
         const bf16x2 pb = __builtin_convertvector(p, bf16x2);
         p_frag[kb][r >> 3][r & 7] = pb.x;
         p_frag[kb][r >> 3][(r & 7) + 1] = pb.y;
