@@ -82,7 +82,7 @@ class proCache:
         for i, block in enumerate(self.out_block_cache):
             if block is not None:
                 active += 1
-                if self.block_size_mb is None:
+                if self.block_size_mb is None and torch.is_tensor(block):  # (dry runs keep chunk-id tuples)
                     mb = block.element_size() * block.nelement() / (1024 ** 2)
                     if self.lse_block_cache[i] is not None:
                         mb += self.lse_block_cache[i].element_size() * self.lse_block_cache[i].nelement() / (1024 ** 2)

@@ -38,13 +38,20 @@ class CacheOracle:
     """core/cache.py:9-128 (bookkeeping only; payloads are opaque)."""
 
     def __init__(self, isp_size: int, merge_fn: Callable = symbolic_merge,
-                 memory_ok: Optional[Callable[["CacheOracle", int], bool]] = None):
+                 memory_ok: Optional[Callable[["CacheOracle", int], bool]] = None,
+                 memory_probe: Optional[Callable[[], float]] = None, block_size_mb: Optional[float] = None,
+                 memory_constraint: float = float("inf")):
         self.isp_size = isp_size  # cache.py:12
         self.curr_isp_stride = isp_size  # cache.py:13
         self.curr_block_num = isp_size  # cache.py:14
         self.slots: List[Optional[Payload]] = [None] * isp_size  # cache.py:17-18
         self.merge_fn = merge_fn
         self.memory_ok = memory_ok
+        # the guard's three quantities in MB (cache.py:21-22, :89-101, :121): the device-memory
+        # reading is a callable so that a test can make the guard trip at a chosen call
+        self.memory_probe = memory_probe
+        self.block_size_mb = block_size_mb
+        self.memory_constraint = memory_constraint
 
     def _merge_blocks(self, new_block_num: int) -> None:
         # cache.py:28-46
@@ -88,12 +95,19 @@ class CacheOracle:
         self.slots[block_id] = state
 
     def pass_memory_check(self, next_isp_stride: int) -> bool:
-        # cache.py:103-128 with the device-memory probe made injectable
-        if next_isp_stride == self.isp_size:
+        # cache.py:103-128 with the device-memory reading made injectable
+        if next_isp_stride == self.isp_size:  # cache.py:104-105
             return True
-        if self.memory_ok is None:
+        if self.memory_ok is not None:  # a test's own verdict
+            return bool(self.memory_ok(self, next_isp_stride))
+        if self.memory_probe is None or self.block_size_mb is None:  # cache.py:115-116
             return True
-        return bool(self.memory_ok(self, next_isp_stride))
+        active = sum(s is not None for s in self.slots)  # cache.py:106-109
+        predicted = self.isp_size // next_isp_stride  # cache.py:117
+        if predicted <= active:  # cache.py:118-119
+            return True
+        add = self.block_size_mb * (predicted - active)  # cache.py:121
+        return not (self.memory_probe() + add > self.memory_constraint)  # cache.py:122-127
 
 
 @dataclass
@@ -125,7 +139,9 @@ class RingOracle:
     def __init__(self, isp_size: int, layer_id: int = 0, use_ditango: bool = True,
                  attn_fn: Callable = symbolic_attn, merge_fn: Callable = symbolic_merge,
                  store_fn: Callable = lambda s: s,
-                 memory_ok: Optional[Callable] = None, small_ring_stride: int = 8):
+                 memory_ok: Optional[Callable] = None, small_ring_stride: int = 8,
+                 memory_probe: Optional[Callable[[], float]] = None, block_size_mb: Optional[float] = None,
+                 memory_constraint: float = float("inf")):
         N = isp_size
         self.N = N
         self.layer_id = layer_id
@@ -136,7 +152,8 @@ class RingOracle:
         self.store_fn = store_fn
         # attention.py:27: local_chunk_id // isp_size == 0 for every rank
         self.target = [r // N for r in range(N)]
-        self.caches = [CacheOracle(N, merge_fn, memory_ok) for _ in range(N)]  # attention.py:28
+        self.caches = [CacheOracle(N, merge_fn, memory_ok, memory_probe, block_size_mb, memory_constraint)
+                       for _ in range(N)]  # attention.py:28
 
     # -- one synchronous exchange over all ranks -------------------------------------------
     def _exchange(self, held: List[int], posts: List[Optional[Tuple[int, int]]]) -> List[int]:

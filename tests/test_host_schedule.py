@@ -120,6 +120,60 @@ def test_memory_guard_falls_back_to_full_refresh(ditango_env):
     assert c.pass_memory_check(1, 0) is True
 
 
+@pytest.mark.parametrize("N,col,trip", [
+    (8, (1, 1, 1, 4, 4, 2, 2, 1, 1), {2}),          # guard trips on the step that announces stride 2
+    (8, (1, 1, 1, 4, 4, 2, 2, 1, 1), {2, 3}),       # ... and again on the next one
+    (8, (1, 1, 1, 8, 8, 4, 2, 2, 1, 1), {2}),       # stride 1 announced: 8 blocks predicted, none held
+    (8, (1, 1, 1, 2, 2, 2, 2, 2, 1, 1), {4}),       # mid-run: one of two blocks held, the other predicted
+    (4, (1, 1, 1, 2, 2, 2, 4, 4, 1, 1), {2, 5}),
+    (16, (1, 1, 1, 8, 8, 4, 4, 2, 1, 1), {2, 6}),   # two-level ring
+])
+def test_plan_with_a_tripping_memory_guard_matches_ring_oracle(ditango_env, N, col, trip):
+    """The stride-mode fallback (core/attention.py:97-98 with core/cache.py:103-128): when the predicted
+    allocation exceeds the budget, only this call's announced stride becomes N -- nothing is stored, the
+    cache is reset to N empty slots -- and the next call reads its stride from the map again, so it probes
+    block ids of an empty cache and those chunks drop out of the softmax.  The planner, fed the same three
+    quantities as the restated guard, must follow the lock-step ring step for step."""
+    from ditango_amd.core.attention import proAttention
+    from ditango_amd.core.parallel_state import get_usp_group
+    from ditango_amd.utils import update_timestep
+
+    T = len(col)
+    curr, nxt = strides_from_dividers(N, col)
+    now = {"t": 0}
+    probe = lambda: 950.0 if now["t"] in trip else 0.0      # MB allocated; budget 1000, a block is 100
+    ring = RingOracle(N, memory_probe=probe, block_size_mb=100.0, memory_constraint=1000.0)
+    oracle_traces = []
+    for t in range(T):
+        now["t"] = t
+        oracle_traces.append(ring.call(t, curr[t], nxt[t]))
+    tripped = {t for t in range(T) if oracle_traces[t][0].next_stride != nxt[t]}
+    assert tripped, "the case is meant to trip the guard"
+    dropped = 0
+    for rank in range(N):
+        rm = ditango_env(N, rank, T, 1)
+        rm.divider_map[:, 0] = torch.tensor(col)
+        attn = proAttention(0, get_usp_group(), dry_run=True)
+        attn.cache.block_size_mb, attn.cache.memory_constraint, attn.cache.memory_probe = 100.0, 1000.0, probe
+        for t in range(T):
+            now["t"] = t
+            update_timestep(t)
+            attn.attn(None, None, None)
+            p, o = attn.last_plan, oracle_traces[t][rank]
+            ctx = (col, rank, t)
+            assert (p.curr_stride, p.next_stride) == (o.curr_stride, o.next_stride), ctx
+            assert p.reuse_probed == o.reuse_probed and p.reuse_merged == o.reuse_merged, ctx
+            assert p.computed == o.computed and p.stores == o.stores and p.flushes == o.flushes, ctx
+            assert (p.target_after, p.nblk_after, p.occupancy_after) == (o.target_after, o.nblk_after, o.occupancy_after), ctx
+            if t in tripped:
+                assert p.next_stride == N and p.stores == [] and p.nblk_after == N and not any(p.occupancy_after), ctx
+            if t - 1 in tripped and curr[t] != N:
+                # the desync: blocks are probed, none is there, fewer than N chunks reach the softmax
+                assert p.reuse_probed and p.reuse_merged == [], ctx
+                dropped += N - len({c for c, _ in p.computed})
+    assert dropped > 0
+
+
 def test_mask_mode_arena_consults_the_memory_guard(ditango_env):
     """ensure_arena uses the probe and budget of pass_memory_check (core/cache.py:103-128): an arena
     that would push the allocation over the budget is refused (once, with a warning), a fitting one is
