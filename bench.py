@@ -36,6 +36,8 @@ import torch
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+import bench_probes  # noqa: E402  (the measurement aids live beside this file, outside the package)
+
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 NOMINAL_CLOCK_MHZ = 2400.0  # the shader clock the bf16 peak is quoted at
@@ -373,7 +375,7 @@ def run_workload(name, args, steps, warmup, main, reuse=None, kernels_only=False
         probe_flops = [0.0]
 
         def probe_launch():
-            probe_flops[0] = _hip.mfma_probe(probe_wgs, probe_iters, probe_sink)
+            probe_flops[0] = bench_probes.mfma_probe(probe_wgs, probe_iters, probe_sink)
 
         kp_ms = time_kernel(probe_launch, reps)
         mfma_probe = {"tflops": round(probe_flops[0] / (kp_ms * 1e-3) / 1e12, 1), "launch_ms": round(kp_ms, 4),
@@ -389,7 +391,7 @@ def run_workload(name, args, steps, warmup, main, reuse=None, kernels_only=False
         co_flops = [0.0]
 
         def co_launch(with_softmax):
-            co_flops[0] = _hip.coissue_probe(co_wgs, co_iters, D, with_softmax, co_sink)
+            co_flops[0] = bench_probes.coissue_probe(co_wgs, co_iters, D, with_softmax, co_sink)
 
         co0_ms = time_kernel(lambda: co_launch(False), reps)
         co1_ms = time_kernel(lambda: co_launch(True), reps)
@@ -434,7 +436,7 @@ def run_workload(name, args, steps, warmup, main, reuse=None, kernels_only=False
 
     def probe(i):
         cache = layers[i % L_run].cache
-        _hip.hbm_read_probe([cache.arena_out[c] for c in range(C)], sink)
+        bench_probes.hbm_read_probe([cache.arena_out[c] for c in range(C)], sink)
 
     kr_ms = time_kernel(Rotation(probe, L_run), reps)
     kr_gbs = C * probe_bytes / (kr_ms * 1e-3) / 1e9
@@ -509,15 +511,18 @@ def run_workload(name, args, steps, warmup, main, reuse=None, kernels_only=False
         # once per segment inside one launch
         pad_rows = 64
         cu = [0, Sq - pad_rows, Sq]
-        group.set_kv_chunks(ks, vs, cu_seqlens_kv=[[0, n - pad_rows, n] for n in lens])
+        # the boundaries are int32 tensors ON THE GPU, as the model makes them (hunyuan_transformer.py:789-792) and as
+        # they travel with K/V round the ring (core/attention.py:307-311); max_seqlen = the sample's length (:783-784)
+        cu_kv_ts = [torch.tensor([0, n - pad_rows, n], dtype=torch.int32, device=dev) for n in lens]
+        group.set_kv_chunks(ks, vs, cu_seqlens_kv=cu_kv_ts)
         q3, k3, v3 = q.view(B * Sq, H, D), ks[rank].view(B * lens[rank], H, D), vs[rank].view(B * lens[rank], H, D)
-        cu_t = torch.tensor(cu, dtype=torch.int32)
-        cu_kv_t = torch.tensor([0, lens[rank] - pad_rows, lens[rank]], dtype=torch.int32)
+        cu_t = torch.tensor(cu, dtype=torch.int32, device=dev)
+        cu_kv_t = cu_kv_ts[rank]
         n_var = 1 if kernels_only else min(24, len(timed))
 
         def run_varlen(t, l):
             update_timestep(t)
-            return layers[l].varlen_attn(q3, k3, v3, cu_t, cu_kv_t, Sq - pad_rows, max(lens) - pad_rows)
+            return layers[l].varlen_attn(q3, k3, v3, cu_t, cu_kv_t, Sq, max(lens))
 
         for t, l in timed[:2]:
             run_varlen(t, l)
@@ -557,6 +562,7 @@ def run_workload(name, args, steps, warmup, main, reuse=None, kernels_only=False
                          "what": "RMSNorm + interleaved RoPE of K over the whole KV sequence, strided read from a fused QKV tensor"},
             "varlen": {"what": f"proAttention.varlen_attn, two segments per sample ({Sq - pad_rows} + {pad_rows} query rows; "
                                f"{lens[0] - pad_rows} + {pad_rows} keys per chunk), same schedule rows",
+                       "cu_seqlens": "device (int32 tensors on the GPU, read by the kernel; no host sync per call)",
                        "ms_per_layer": round(var_ms, 4), "calls": n_var, "mean_chunks_computed_per_call": round(var_chunks, 3),
                        "layer_attn_tflops": round(var_flops / (var_ms * 1e-3) / 1e12, 1)},
             "rel_l1": {"kernel": "rel_l1_sums_kernel", "bound": "hbm", "achieved": round(kl_gbs, 1), "peak": PEAK_HBM_GBS,

@@ -67,15 +67,21 @@ _SIGNATURES = {
                                              c_i32, _P(c_vp), _P(c_vp), _P(c_i32), _P(c_i64), c_i64, c_i64,
                                              c_vp, c_vp, c_i32, c_vp, c_i64, c_vp, c_i64, c_i32, c_vp, c_vp,
                                              c_i32, _P(c_i32), _P(c_i32), _P(c_i32), _P(c_i32), c_f32, c_vp]),
+    "dt_attn_varlen_jobs_fwd": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i64, c_i64, c_i64,
+                                               c_i32, _P(c_vp), _P(c_vp), _P(c_i32), _P(c_i64), c_i64, c_i64,
+                                               c_i32, _P(c_i32), _P(c_i32), _P(c_i32), c_i32, c_vp, _P(c_vp), c_i32,
+                                               _P(c_vp), _P(c_vp), c_f32, c_i32, c_vp]),
+    "dt_attn_sched_varlen_fwd": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i64, c_i64, c_i64,
+                                                c_i32, _P(c_vp), _P(c_vp), _P(c_i32), _P(c_i64), c_i64, c_i64,
+                                                c_vp, c_vp, c_i32, c_vp, c_i64, c_vp, c_i64, c_i32, c_vp, c_vp,
+                                                c_i32, c_vp, _P(c_vp), c_i32, c_f32, c_i32, c_vp]),
+    "dt_zero_rows_from": (ctypes.c_int, [c_vp, c_i64, c_i64, c_vp, c_vp]),
     "dt_merge_states": (ctypes.c_int, [c_i32, _P(c_vp), _P(c_vp), _P(c_i32), _P(c_i32), c_vp, c_i32, c_vp, c_i32,
                                        c_i32, c_i32, c_i32, c_i32, c_vp]),
     "dt_cache_store": (ctypes.c_int, [c_vp, c_i32, c_vp, c_i32, c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_vp]),
     "dt_cache_load": (ctypes.c_int, [c_vp, c_vp, c_vp, c_i32, c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp]),
     "dt_build_schedule": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp, c_vp]),
     "dt_build_schedule_table": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp, c_vp]),
-    "dt_hbm_read_probe": (ctypes.c_int, [_P(c_vp), c_i32, c_i64, c_vp, c_vp]),
-    "dt_mfma_probe": (ctypes.c_int, [c_i32, c_i32, c_vp, c_vp]),
-    "dt_coissue_probe": (ctypes.c_int, [c_i32, c_i32, c_i32, c_i32, c_vp, c_vp]),
     "dt_rel_l1_sums": (ctypes.c_int, [c_vp, c_vp, c_i64, c_vp, c_vp]),
     "dt_qk_norm_rope": (ctypes.c_int, [c_vp, c_i64, c_i64, c_i64, c_vp, c_i32, c_i32, c_i32, c_i32,
                                        c_i32, c_vp, c_vp, c_f32, c_i32, c_vp, c_vp, c_i64, c_i32, c_i32,
@@ -204,21 +210,33 @@ def attn_chunk_f32_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softma
     return out, lse
 
 
-_workspaces = {}
+_workspaces: "dict" = {}   # (device type, index, stream handle) -> tensor, in order of last use
+MAX_WORKSPACES = 4         # streams per process that keep a workspace (about 102 MB each)
 
 
 def attn_workspace(device) -> torch.Tensor:
-    """The workspace of the attention launches made on the current stream of ``device`` (allocated once per
-    device and stream, ``dt_attn_workspace_bytes()`` bytes).  Launches that share a workspace must be ordered
-    on one stream; keyed by the stream, launches made on different streams never share one."""
+    """The workspace of the attention launches made on the current stream of ``device`` (``dt_attn_workspace_bytes()``
+    bytes).  Launches that share a workspace must be ordered on one stream; keyed by the stream, launches made on
+    different streams never share one.  At most ``MAX_WORKSPACES`` streams keep theirs: the least recently used
+    entry is dropped (its memory goes back to the allocator in stream order, so launches still in flight on that
+    stream are safe).  The first call on a stream allocates: make it before capturing that stream in a graph --
+    a workspace first created under capture would live in the graph's private pool -- or use the allocation-free
+    entry point (``attn_jobs_fwd(..., no_alloc=True)``)."""
     dev = torch.device(device)
     index = dev.index if dev.index is not None else torch.cuda.current_device()
     key = (dev.type, index, torch.cuda.current_stream(index).cuda_stream)
-    ws = _workspaces.get(key)
+    ws = _workspaces.pop(key, None)
     if ws is None:
+        while len(_workspaces) >= MAX_WORKSPACES:
+            _workspaces.pop(next(iter(_workspaces)))
         ws = torch.empty(int(load_library().dt_attn_workspace_bytes()), dtype=torch.uint8, device=dev)
-        _workspaces[key] = ws
+    _workspaces[key] = ws       # most recently used last
     return ws
+
+
+def release_workspaces() -> None:
+    """Drop every attention workspace (they are re-created on demand)."""
+    _workspaces.clear()
 
 
 class ChunkTable:
@@ -284,12 +302,39 @@ class ChunkTable:
         return self.whole()[3]
 
 
+class DeviceSegments:
+    """Segment boundaries of a packed variable-length batch that live in device memory, as
+    ``flash_attn_varlen_func`` takes them: ``cu_q`` int32 ``[n_seg + 1]`` for the queries and one such tensor
+    per KV chunk for its keys (``cu_kv[c]``; ``None`` for a chunk without keys).  ``max_seqlen_q`` is the
+    host-side upper bound of a segment's length that sizes the grid.  Nothing here reads device memory."""
+
+    def __init__(self, cu_q: torch.Tensor, cu_kv: Sequence[Optional[torch.Tensor]], max_seqlen_q: int):
+        for name, t in [("cu_seqlens_q", cu_q)] + [(f"cu_seqlens_kv[{i}]", t) for i, t in enumerate(cu_kv) if t is not None]:
+            _require(torch.is_tensor(t) and t.is_cuda and t.dtype == torch.int32 and t.dim() == 1 and t.is_contiguous(),
+                     f"{name} must be a contiguous int32 vector on the GPU")
+            _require(t.numel() == cu_q.numel(), f"{name} must have as many entries as cu_seqlens_q")
+        _require(cu_q.numel() >= 2, "cu_seqlens_q needs at least two entries")
+        _require(int(max_seqlen_q) > 0, "max_seqlen_q must be positive")
+        self.cu_q = cu_q
+        self.cu_kv = list(cu_kv)
+        self.n_seg = cu_q.numel() - 1
+        self.max_seqlen_q = int(max_seqlen_q)
+
+    def kv_pointers(self, ids: Sequence[int]):
+        ids = list(ids)
+        return (c_vp * len(ids))(*[self.cu_kv[i].data_ptr() if self.cu_kv[i] is not None else None for i in ids])
+
+    def window(self, w0: int, w1: int) -> "DeviceSegments":
+        return DeviceSegments(self.cu_q, self.cu_kv[w0:w1], self.max_seqlen_q)
+
+
 def attn_jobs_fwd(q: torch.Tensor, table: ChunkTable, jobs: Sequence[Sequence[int]],
                   outs: Sequence[torch.Tensor], lses: Sequence[torch.Tensor], softmax_scale: float = 0.0,
                   q_ranges: Optional[Sequence[Tuple[int, int]]] = None,
                   kv_ranges: Optional[Sequence[Sequence[Tuple[int, int]]]] = None,
                   workspace: Optional[torch.Tensor] = None, q_prescaled: bool = False,
-                  no_alloc: bool = False) -> None:
+                  no_alloc: bool = False, dev_segments: Optional["DeviceSegments"] = None,
+                  job_segments: Optional[Sequence[int]] = None) -> None:
     """One launch; job j attends q to the concatenation of chunks ``jobs[j]`` and writes (outs[j], lses[j]).
 
     ``q_ranges[j] = (begin, length)`` restricts job j to those query rows (the rest of its
@@ -301,13 +346,20 @@ def attn_jobs_fwd(q: torch.Tensor, table: ChunkTable, jobs: Sequence[Sequence[in
     ``q_prescaled``: q already carries ``softmax_scale * log2(e)`` (folded in before its rounding to
     bf16); ``softmax_scale`` is then ignored and the softmax is that of ``q k^T * ln 2``.
     ``no_alloc``: go through ``dt_attn_seg_jobs_noalloc_fwd``, which splits the tail inside the library's
-    own device array instead of a workspace (for callers that cannot allocate)."""
+    own device array instead of a workspace (for callers that cannot allocate).
+    ``dev_segments`` with ``job_segments``: the segment boundaries stay in device memory
+    (``dt_attn_varlen_jobs_fwd``); job j is segment ``job_segments[j]`` of its state and the host reads none
+    of the boundaries."""
     lib = load_library()
     _check_qkv(q, "q")
     B, Sq, H, D = q.shape
     _require((B, H, D) == (table.B, table.H, table.D), "q and KV chunks disagree on B/H/D")
     _require(not (no_alloc and workspace is not None), "no_alloc launches take no workspace")
     nj = len(jobs)
+    if dev_segments is not None:
+        _require(q_ranges is None and kv_ranges is None and not no_alloc, "device segment boundaries replace the host ranges")
+        _require(job_segments is not None and len(job_segments) == nj, "one segment index per job")
+        _require(len(dev_segments.cu_kv) == table.n, "one cu_seqlens_kv per chunk of the table")
     _require(nj == len(outs) == len(lses), "one destination per job")
     _require(q_ranges is None or len(q_ranges) == nj, "one query range per job")
     _require(kv_ranges is None or len(kv_ranges) == nj, "one list of key ranges per job")
@@ -362,7 +414,16 @@ def attn_jobs_fwd(q: torch.Tensor, table: ChunkTable, jobs: Sequence[Sequence[in
         a_ql = (c_i32 * n)(*[int(q_ranges[start + jj][1]) for jj in range(n)]) if q_ranges is not None else None
         out_ptrs = (c_vp * n)(*[outs[start + jj].data_ptr() for jj in range(n)])
         lse_ptrs = (c_vp * n)(*[lses[start + jj].data_ptr() for jj in range(n)])
-        if no_alloc:
+        if dev_segments is not None:
+            seg_ids = (c_i32 * n)(*[int(job_segments[start + jj]) for jj in range(n)])
+            cu_kv = dev_segments.kv_pointers(range(table.n) if local is None else ids)
+            rc = lib.dt_attn_varlen_jobs_fwd(q.data_ptr(), B, Sq, H, D, q.stride(0), q.stride(1), q.stride(2),
+                                             t_n, t_k, t_v, t_len, t_sb, table.ss, table.sh,
+                                             n, begin, chunks, seg_ids, dev_segments.n_seg, dev_segments.cu_q.data_ptr(),
+                                             cu_kv, int(dev_segments.max_seqlen_q), out_ptrs, lse_ptrs,
+                                             float(softmax_scale), DT_ATTN_Q_PRESCALED if q_prescaled else 0, _stream())
+            _check(rc, "dt_attn_varlen_jobs_fwd")
+        elif no_alloc:
             rc = lib.dt_attn_seg_jobs_noalloc_fwd(q.data_ptr(), B, Sq, H, D, q.stride(0), q.stride(1), q.stride(2),
                                                   t_n, t_k, t_v, t_len, t_sb, table.ss, table.sh,
                                                   n, begin, chunks, a_kvb, a_kvl, a_qb, a_ql, out_ptrs,
@@ -386,7 +447,8 @@ def attn_sched_fwd(q: torch.Tensor, table: ChunkTable, dev_compute_ids: torch.Te
                    diag_out: Optional[torch.Tensor], diag_lse: Optional[torch.Tensor],
                    softmax_scale: float = 0.0, seg_q: Optional[Sequence[Tuple[int, int]]] = None,
                    seg_kv: Optional[Sequence[Sequence[Tuple[int, int]]]] = None,
-                   workspace: Optional[torch.Tensor] = None, q_prescaled: bool = False) -> None:
+                   workspace: Optional[torch.Tensor] = None, q_prescaled: bool = False,
+                   dev_segments: Optional[DeviceSegments] = None) -> None:
     """Device-scheduled launch: chunk ids come from ``dev_compute_ids[:dev_count]`` in device memory and
     each state lands in its slot of the arena (``slot_out [C,B,Sq,H,D]`` bf16, ``slot_lse [C,B,H,Sq]`` fp32).
 
@@ -407,6 +469,21 @@ def attn_sched_fwd(q: torch.Tensor, table: ChunkTable, dev_compute_ids: torch.Te
         _require(diag_out is not None and diag_lse is not None, "a diag chunk needs (diag_out, diag_lse)")
         _require(diag_out.dtype == torch.bfloat16 and diag_out.is_contiguous() and tuple(diag_out.shape) == (B, Sq, H, D), "diag_out must be contiguous bf16 [B,Sq,H,D]")
         _require(diag_lse.dtype == torch.float32 and diag_lse.is_contiguous() and tuple(diag_lse.shape) == (B, H, Sq), "diag_lse must be contiguous fp32 [B,H,Sq]")
+    if dev_segments is not None:
+        # segment boundaries in device memory: every scheduled chunk runs once per segment, the host reads nothing
+        _require(seg_q is None and seg_kv is None, "device segment boundaries replace the host ranges")
+        _require(len(dev_segments.cu_kv) == table.n, "one cu_seqlens_kv per chunk of the table")
+        rc = lib.dt_attn_sched_varlen_fwd(q.data_ptr(), B, Sq, H, D, q.stride(0), q.stride(1), q.stride(2),
+                                          table.n, table.k_ptrs, table.v_ptrs, table.lens, table.sb, table.ss, table.sh,
+                                          dev_compute_ids.data_ptr(), dev_count.data_ptr(), int(max_jobs),
+                                          slot_out.data_ptr(), slot_out.stride(0), slot_lse.data_ptr(), slot_lse.stride(0),
+                                          int(diag), diag_out.data_ptr() if diag_out is not None else None,
+                                          diag_lse.data_ptr() if diag_lse is not None else None,
+                                          dev_segments.n_seg, dev_segments.cu_q.data_ptr(),
+                                          dev_segments.kv_pointers(range(table.n)), dev_segments.max_seqlen_q,
+                                          float(softmax_scale), DT_ATTN_Q_PRESCALED if q_prescaled else 0, _stream())
+        _check(rc, "dt_attn_sched_varlen_fwd")
+        return
     n_seg, a_qb, a_ql, a_kb, a_kl = 0, None, None, None, None
     if seg_q is not None:
         n_seg = len(seg_q)
@@ -514,6 +591,17 @@ def cache_load(slot_out: torch.Tensor, slot_lse: torch.Tensor, dst_dtype: torch.
     return dst_out, dst_lse
 
 
+def zero_rows_from(t: torch.Tensor, first_row: torch.Tensor) -> None:
+    """Zero the rows ``[first_row[0], n)`` of ``t`` (contiguous, rows along dim 0), the index read on the device."""
+    lib = load_library()
+    _require(t.is_cuda and t.is_contiguous() and t.dim() >= 1, "t must be a contiguous device tensor")
+    _require(first_row.is_cuda and first_row.dtype == torch.int32 and first_row.numel() >= 1, "first_row must be int32 on the GPU")
+    n = t.shape[0]
+    row_bytes = (t.numel() // max(n, 1)) * t.element_size()
+    rc = lib.dt_zero_rows_from(t.data_ptr(), n, row_bytes, first_row.data_ptr(), _stream())
+    _check(rc, "dt_zero_rows_from")
+
+
 # ---------------------------------------------------------------------------------------------
 # K4: schedule builder, rel-L1 sums
 # ---------------------------------------------------------------------------------------------
@@ -541,41 +629,6 @@ def build_schedule_table(mask: torch.Tensor, diag: int = -1):
     rc = lib.dt_build_schedule_table(mask.data_ptr(), T, L, C, int(diag), comp.data_ptr(), reu.data_ptr(), cnt.data_ptr(), _stream())
     _check(rc, "dt_build_schedule_table")
     return comp, reu, cnt
-
-
-def hbm_read_probe(buffers: Sequence[torch.Tensor], sink: torch.Tensor) -> None:
-    """Read ``buffers`` (equally sized, contiguous, a multiple of 256 bytes each) with the merge kernel's
-    access pattern and discard the data: the bandwidth yardstick of the HBM-bound kernels."""
-    lib = load_library()
-    n = len(buffers)
-    nbytes = buffers[0].numel() * buffers[0].element_size()
-    for b in buffers:
-        _require(b.is_cuda and b.is_contiguous() and b.numel() * b.element_size() == nbytes, "probe buffers must be equally sized contiguous device tensors")
-    _require(sink.is_cuda and sink.numel() * sink.element_size() >= 4, "sink must be a device tensor of at least 4 bytes")
-    ptrs = (c_vp * n)(*[b.data_ptr() for b in buffers])
-    rc = lib.dt_hbm_read_probe(ptrs, n, nbytes // 256 * 256, sink.data_ptr(), _stream())
-    _check(rc, "dt_hbm_read_probe")
-
-
-def mfma_probe(workgroups: int, iters: int, sink: torch.Tensor) -> float:
-    """Launch the register-only MFMA loop (the sustained-rate yardstick of the attention kernel) and return
-    the FLOP the launch performs: ``workgroups * 8`` wavefronts x ``4 * iters`` bf16 MFMAs of 32 x 32 x 16."""
-    lib = load_library()
-    _require(sink.is_cuda and sink.numel() * sink.element_size() >= 4, "sink must be a device tensor of at least 4 bytes")
-    rc = lib.dt_mfma_probe(int(workgroups), int(iters), sink.data_ptr(), _stream())
-    _check(rc, "dt_mfma_probe")
-    return float(workgroups) * 8 * 4 * iters * 32768.0
-
-
-def coissue_probe(workgroups: int, iters: int, head_dim: int, with_softmax: bool, sink: torch.Tensor) -> float:
-    """Launch the co-issue probe (one wavefront of each SIMD issues MFMAs; with ``with_softmax`` the other one
-    issues the softmax's vector instructions per MFMA at that head dimension) and return the FLOP of the
-    launch: ``workgroups * 4`` wavefronts x ``4 * iters`` bf16 MFMAs of 32 x 32 x 16."""
-    lib = load_library()
-    _require(sink.is_cuda and sink.numel() * sink.element_size() >= 4, "sink must be a device tensor of at least 4 bytes")
-    rc = lib.dt_coissue_probe(int(workgroups), int(iters), int(head_dim), int(bool(with_softmax)), sink.data_ptr(), _stream())
-    _check(rc, "dt_coissue_probe")
-    return float(workgroups) * 4 * 4 * iters * 32768.0
 
 
 def rel_l1_sums(a: torch.Tensor, b: torch.Tensor, sums: Optional[torch.Tensor] = None) -> torch.Tensor:

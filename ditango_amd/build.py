@@ -1,7 +1,9 @@
 """Build libditango_hip.so (gfx950) in-tree with hipcc.
 
 ``python -m ditango_amd.build`` compiles every translation unit under
-``ditango_amd/csrc`` and links ``ditango_amd/lib/libditango_hip.so``.  hipcc
+``ditango_amd/csrc`` and links ``ditango_amd/lib/libditango_hip.so`` (the drop-in
+library) and ``ditango_amd/lib/libditango_probes.so`` (the benchmark's measurement
+aids, a library of its own that only ``bench.py`` loads).  hipcc
 cross-compiles for gfx950 without a GPU.  Packed-FP32 instruction selection is
 switched off for all device code (``-target-feature -packed-fp32-ops``).
 """
@@ -18,8 +20,10 @@ ROOT = PKG.parent
 CSRC = PKG / "csrc"
 LIB_DIR = PKG / "lib"
 LIB_PATH = LIB_DIR / "libditango_hip.so"
+PROBES_PATH = LIB_DIR / "libditango_probes.so"
 DEMO_PATH = LIB_DIR / "dt_capi_demo"
 SOURCES = ["attn_fwd.hip", "attn_f32.hip", "state_ops.hip", "producer.hip", "capi.hip"]
+PROBE_SOURCES = ["probes.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 COMMON = [
@@ -50,12 +54,16 @@ def build_lib(verbose: bool = False, extra_flags=()) -> Path:
         _run(cmd)
         return obj
 
-    with ThreadPoolExecutor(max_workers=min(5, len(SOURCES))) as ex:
-        objs = list(ex.map(compile_one, SOURCES))
-    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objs), "-o", str(LIB_PATH)]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    _run(cmd)
+    with ThreadPoolExecutor(max_workers=6) as ex:
+        all_objs = list(ex.map(compile_one, SOURCES + PROBE_SOURCES))
+    objs, probe_objs = all_objs[:len(SOURCES)], all_objs[len(SOURCES):]
+    # a version script keeps everything but the C entry points out of the dynamic symbol table
+    for out, members, exports in ((LIB_PATH, objs, "exports_hip.map"), (PROBES_PATH, probe_objs, "exports_probes.map")):
+        cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", f"-Wl,--version-script={CSRC / exports}",
+               *map(str, members), "-o", str(out)]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        _run(cmd)
     # a host program that uses nothing but the C header and the HIP runtime (tests/test_capi_demo_gpu.py runs it)
     cmd = [HIPCC, "-O2", "-std=c++17", "-Wno-unused-result", f"-I{ROOT / 'include'}", str(CSRC / "capi_demo.cpp"),
            f"-L{LIB_DIR}", "-lditango_hip", "-Wl,-rpath,$ORIGIN", "-o", str(DEMO_PATH)]

@@ -203,7 +203,9 @@ class proAttention:
         # plain vector-ALU kernel for small problems) and only cached states are rounded to bf16.
         self.fp32_inputs = "round"
         self._exact_f32 = False
-        self._segments = None  # (cu_seqlens_q, chunk -> cu_seqlens_kv) while a variable-length call runs
+        # while a variable-length call runs: (cu_seqlens_q, chunk -> cu_seqlens_kv) as host lists, or a
+        # _DeviceSegmentSource when the boundaries are device tensors that the host never reads
+        self._segments = None
         if self.layer_id == 0:
             logger.info(f"R{self.global_rank}L{layer_id} | cached block attention on HIP kernels (gfx950)")
 
@@ -230,7 +232,9 @@ class proAttention:
         curr, nxt = self._strides(timestep)
         if timestep == 0 and value is not None:
             self.cache.set_block_size_mb(value)  # :93-94
-        if not self.dry_run and not self.cache.pass_memory_check(nxt, self.layer_id):  # :97-98
+        # :97-98: an over-budget prediction turns the announced stride into N for this call only -- the next
+        # call reads its stride from the map again and probes a cache that was reset to N empty slots
+        if not self.cache.pass_memory_check(nxt, self.layer_id):
             nxt = N
         if self._ring_targets[r] != self.target_chunk_id:  # the pointer was set from outside: same offset everywhere
             shift = (self.target_chunk_id - self._ring_targets[r]) % N
@@ -343,7 +347,9 @@ class proAttention:
         # (local + own) is computed once and merged twice
         job_lists, dests, seen = [], [], {}
         pieced = []  # states computed in pieces: [(o, l) of the first piece = destination, the others...]
-        q_ranges, kv_ranges = ([], []) if segments is not None else (None, None)
+        dev_seg = segments if isinstance(segments, _DeviceSegmentSource) else None
+        q_ranges, kv_ranges = ([], []) if segments is not None and dev_seg is None else (None, None)
+        job_segs = [] if dev_seg is not None else None
         states = []
         for job in plan.jobs:
             if job.chunks in seen and job.store_slot is None:
@@ -366,6 +372,12 @@ class proAttention:
             elif len(pieces) > 1:
                 raise NotImplementedError("variable-length calls with blocks of more than "
                                           f"{self._MAX_JOB_CHUNKS} chunks are not supported")
+            elif dev_seg is not None:
+                # one kernel job per segment; the kernel reads the segment's rows and keys from device memory
+                for i in range(dev_seg.n_seg):
+                    job_lists.append([index[c] for c in job.chunks])
+                    dests.append((o, l))
+                    job_segs.append(i)
             else:
                 # one kernel job per segment: its query rows against its key rows of every chunk
                 cu_q, cu_kv_of = segments
@@ -378,9 +390,13 @@ class proAttention:
             states.append((o, l))
         if job_lists:
             table = _hip.ChunkTable(ks, vs)
-            _hip.attn_jobs_fwd(query, table, job_lists, [d[0] for d in dests], [d[1] for d in dests],
-                               q_ranges=q_ranges, kv_ranges=kv_ranges, workspace=_hip.attn_workspace(dev),
-                               q_prescaled=self.q_prescaled)
+            if dev_seg is not None:
+                _hip.attn_jobs_fwd(query, table, job_lists, [d[0] for d in dests], [d[1] for d in dests],
+                                   q_prescaled=self.q_prescaled, dev_segments=dev_seg.over(needed), job_segments=job_segs)
+            else:
+                _hip.attn_jobs_fwd(query, table, job_lists, [d[0] for d in dests], [d[1] for d in dests],
+                                   q_ranges=q_ranges, kv_ranges=kv_ranges, workspace=_hip.attn_workspace(dev),
+                                   q_prescaled=self.q_prescaled)
         for piece_states in pieced:
             _hip.merge_states([s[0] for s in piece_states], [s[1] for s in piece_states],
                               dst_out=piece_states[0][0], dst_lse=piece_states[0][1])
@@ -415,8 +431,10 @@ class proAttention:
         for c in range(C):
             if c != diag and row[c] != 0 and not cache.arena_valid[c]:
                 raise RuntimeError(f"T{t}L{l}: mask asks to reuse chunk {c} but no state was ever stored for it")
-        seg_q = seg_kv = None
-        if self._segments is not None:
+        seg_q = seg_kv = dev_seg = None
+        if isinstance(self._segments, _DeviceSegmentSource):
+            dev_seg = self._segments.over(range(C))
+        elif self._segments is not None:
             # packed variable-length batch: every scheduled chunk runs once per segment
             cu_q, cu_kv_of = self._segments
             seg_q = [(cu_q[i], cu_q[i + 1] - cu_q[i]) for i in range(len(cu_q) - 1)]
@@ -427,18 +445,31 @@ class proAttention:
             n_comp = int(rm.sched_counts_host[t, l, 0])
             _hip.attn_sched_fwd(query, _hip.ChunkTable(ks, vs), rm.sched_compute_ids[t, l], rm.sched_counts[t, l, 0:1],
                                 n_comp, cache.arena_out, cache.arena_lse, diag, cache.diag_out, cache.diag_lse,
-                                seg_q=seg_q, seg_kv=seg_kv, workspace=ws, q_prescaled=self.q_prescaled)
+                                seg_q=seg_q, seg_kv=seg_kv, workspace=ws, q_prescaled=self.q_prescaled,
+                                dev_segments=dev_seg)
         else:
             # more chunks than one launch addresses: one launch per window of chunk ids (ordered on the
             # stream, so they can share the workspace)
             for w0, w1, d_w, comp_w, cnt_w, cnt_host_w in rm.sched_windows:
                 n_comp = int(cnt_host_w[t, l, 0])
-                if n_comp == 0 or all(k.shape[1] == 0 for k in ks[w0:w1]):
+                if n_comp == 0:
+                    continue
+                if all(k.shape[1] == 0 for k in ks[w0:w1]):
+                    # a window without a single key is not launched (a chunk table needs one): the states its
+                    # scheduled chunks would have got -- out = 0, lse = -inf, neutral in the merge -- are written here
+                    for c in range(w0, w1):
+                        if c == diag:
+                            cache.diag_out.zero_()
+                            cache.diag_lse.fill_(float("-inf"))
+                        elif row[c] == 0:
+                            cache.arena_out[c].zero_()
+                            cache.arena_lse[c].fill_(float("-inf"))
                     continue
                 _hip.attn_sched_fwd(query, _hip.ChunkTable(ks[w0:w1], vs[w0:w1]), comp_w[t, l], cnt_w[t, l, 0:1],
                                     n_comp, cache.arena_out[w0:w1], cache.arena_lse[w0:w1], d_w, cache.diag_out,
                                     cache.diag_lse, seg_q=seg_q, seg_kv=None if seg_kv is None else seg_kv[w0:w1],
-                                    workspace=ws, q_prescaled=self.q_prescaled)
+                                    workspace=ws, q_prescaled=self.q_prescaled,
+                                    dev_segments=None if dev_seg is None else dev_seg.window(w0, w1))
         outs, lses = [], []
         for c in range(C):
             if c == diag:
@@ -489,11 +520,28 @@ class proAttention:
         B, Sq, H, D = query.shape
         dev = query.device
         ids = [c for c in range(len(ks)) if ks[c].shape[1] > 0]
+        if not ids:  # no key anywhere: the empty attention state
+            self.last_lse = torch.full((B, Sq, H, 1), float("-inf"), dtype=torch.float32, device=dev)
+            return torch.zeros((B, Sq, H, D), dtype=self.out_dtype, device=dev)
         pieces = [ids[i:i + self._MAX_JOB_CHUNKS] for i in range(0, len(ids), self._MAX_JOB_CHUNKS)]
         outs = [torch.empty((B, Sq, H, D), dtype=torch.bfloat16, device=dev) for _ in pieces]
         lses = [torch.empty((B, H, Sq), dtype=torch.float32, device=dev) for _ in pieces]
         q_ranges = kv_ranges = None
         jobs, d_out, d_lse = pieces, outs, lses
+        if isinstance(self._segments, _DeviceSegmentSource):
+            src = self._segments
+            jobs, d_out, d_lse, job_segs = [], [], [], []
+            for piece, o, l_ in zip(pieces, outs, lses):
+                for i in range(src.n_seg):
+                    jobs.append(piece)
+                    d_out.append(o)
+                    d_lse.append(l_)
+                    job_segs.append(i)
+            _hip.attn_jobs_fwd(query, _hip.ChunkTable(ks, vs), jobs, d_out, d_lse, q_prescaled=self.q_prescaled,
+                               dev_segments=src.over(range(len(ks))), job_segments=job_segs)
+            out, lse = _hip.merge_states(outs, lses, dst_dtype=self.out_dtype, dst_lse_bsh=True)
+            self.last_lse = lse
+            return out
         if self._segments is not None:
             cu_q, cu_kv_of = self._segments
             jobs, d_out, d_lse, q_ranges, kv_ranges = [], [], [], [], []
@@ -528,20 +576,60 @@ class proAttention:
             logger.warning("cu_seqlens_q not provided, using normal attention instead.")
             return self.attn(query, key, value)
         total_q, H, D = query.shape
-        cu_q = [int(x) for x in (cu_seqlens_q.tolist() if hasattr(cu_seqlens_q, "tolist") else cu_seqlens_q)]
-        local_cu = [int(x) for x in (cu_seqlens_kv.tolist() if hasattr(cu_seqlens_kv, "tolist") else cu_seqlens_kv)]
-        assert cu_q[0] == 0 and cu_q[-1] <= total_q and len(local_cu) == len(cu_q), "malformed cu_seqlens"
         r = self.local_chunk_id
+        on_device = torch.is_tensor(cu_seqlens_q) and cu_seqlens_q.is_cuda
+        if on_device and not self.dry_run:
+            # the reference's calling convention: int32 cu_seqlens on the GPU.  They stay there -- the kernels read
+            # them (dt_attn_varlen_jobs_fwd / dt_attn_sched_varlen_fwd), the host reads none, nothing synchronises
+            self._segments = _DeviceSegmentSource(self, cu_seqlens_q, cu_seqlens_kv, max_seqlen_q, total_q)
+            cu_q = None
+        else:
+            cu_q = [int(x) for x in (cu_seqlens_q.tolist() if hasattr(cu_seqlens_q, "tolist") else cu_seqlens_q)]
+            local_cu = [int(x) for x in (cu_seqlens_kv.tolist() if hasattr(cu_seqlens_kv, "tolist") else cu_seqlens_kv)]
+            assert cu_q[0] == 0 and cu_q[-1] <= total_q and len(local_cu) == len(cu_q), "malformed cu_seqlens"
 
-        def cu_kv_of(c):
-            return local_cu if c == r else self.group.kv_cu_seqlens(c)
+            def cu_kv_of(c):
+                if c == r:
+                    return local_cu
+                cu = self.group.kv_cu_seqlens(c)
+                # (boundaries that were handed over on the GPU beside host-side cu_seqlens_q: one blocking read)
+                return [int(x) for x in cu.tolist()] if torch.is_tensor(cu) else cu
 
-        self._segments = (cu_q, cu_kv_of)
+            self._segments = (cu_q, cu_kv_of)
         try:
             out = self.attn(query.view(1, total_q, H, D), key.view(1, key.shape[0], H, D),
                             value.view(1, value.shape[0], H, D))
         finally:
             self._segments = None
-        if cu_q[-1] < total_q:
-            out[:, cu_q[-1]:] = 0  # rows outside every segment: flash_attn_varlen_func leaves zeros
+        # rows outside every segment: flash_attn_varlen_func leaves zeros
+        if cu_q is None:
+            _hip.zero_rows_from(out.view(total_q, H * D), cu_seqlens_q[-1:])
+        elif cu_q[-1] < total_q:
+            out[:, cu_q[-1]:] = 0
         return out.view(total_q, H, D)
+
+
+class _DeviceSegmentSource:
+    """The segment boundaries of one variable-length call while they stay in device memory: hands the
+    launches a ``_hip.DeviceSegments`` over the chunks they address."""
+
+    def __init__(self, attn: "proAttention", cu_q, local_cu_kv, max_seqlen_q, total_q: int):
+        if not (torch.is_tensor(local_cu_kv) and local_cu_kv.is_cuda):
+            raise TypeError("cu_seqlens_q is on the GPU, so cu_seqlens_kv must be as well")
+        self.attn = attn
+        self.cu_q = cu_q.to(torch.int32).contiguous()            # (no-ops for the int32 vectors the callers pass)
+        self.local = local_cu_kv.to(torch.int32).contiguous()
+        self.max_seqlen_q = int(max_seqlen_q) if max_seqlen_q else int(total_q)
+        self.n_seg = self.cu_q.numel() - 1
+
+    def cu_kv(self, c: int):
+        if c == self.attn.local_chunk_id:
+            return self.local
+        cu = self.attn.group.kv_cu_seqlens(c)
+        if not torch.is_tensor(cu):                              # a host list beside device boundaries: one small upload
+            cu = torch.tensor(list(cu), dtype=torch.int32, device=self.cu_q.device)
+        return cu.to(torch.int32).contiguous()
+
+    def over(self, chunk_ids) -> "_hip.DeviceSegments":
+        """Boundaries of the chunks ``chunk_ids`` in that order (the local chunk's are the call's ``cu_seqlens_kv``)."""
+        return _hip.DeviceSegments(self.cu_q, [self.cu_kv(c) for c in chunk_ids], self.max_seqlen_q)

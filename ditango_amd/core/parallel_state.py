@@ -31,18 +31,22 @@ class LocalRingGroup:
         [total_c,H,D] for the variable-length entry).  The entry at ``rank_in_group`` may be
         None: the local chunk is the (key, value) passed to ``attn`` itself.
         ``cu_seqlens_kv[c]`` are the segment boundaries of chunk ``c`` (they travel with K/V on
-        the reference's ring, core/attention.py:307-311)."""
+        the reference's ring, core/attention.py:307-311): int32 device tensors as the reference's
+        callers make them (hunyuan_transformer.py:789-792) are kept as they are -- nothing is copied to
+        the host -- and lists / CPU tensors as lists of ints."""
         assert len(k_chunks) == self.world_size and len(v_chunks) == self.world_size
         self._k = list(k_chunks)
         self._v = list(v_chunks)
         if cu_seqlens_kv is not None:
             assert len(cu_seqlens_kv) == self.world_size
-            self._cu = [None if c is None else [int(x) for x in (c.tolist() if hasattr(c, "tolist") else c)]
+            self._cu = [c if c is None or (torch.is_tensor(c) and c.is_cuda)
+                        else [int(x) for x in (c.tolist() if hasattr(c, "tolist") else c)]
                         for c in cu_seqlens_kv]
         else:
             self._cu = [None] * self.world_size
 
-    def kv_cu_seqlens(self, chunk_id: int) -> Sequence[int]:
+    def kv_cu_seqlens(self, chunk_id: int):
+        """Segment boundaries of chunk ``chunk_id``: a list of ints, or the int32 device tensor that was handed in."""
         cu = self._cu[chunk_id]
         if cu is None:
             raise RuntimeError(f"segment boundaries of KV chunk {chunk_id} were not provided (set_kv_chunks)")

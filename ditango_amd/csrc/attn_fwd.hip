@@ -253,6 +253,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
   __bf16* out_ptr;
   float* lse_ptr;
   int vseg = -1;  // segment of a packed variable-length batch (device-listed jobs only)
+  int dseg = -1;  // segment whose boundaries are read from device memory (a.cu_q != nullptr)
   if (a.dev_ids != nullptr) {
     int slot = job;
     if (a.n_seg > 0) {
@@ -272,25 +273,49 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
       lse_ptr = a.slot_lse + (int64_t)single * a.slot_lse_stride;
     }
     if (vseg >= 0) {
-      q_begin = a.seg_q_begin[vseg];
-      q_end = q_begin + a.seg_q_len[vseg];
-      if (qt * kBQ >= q_end - q_begin) return;  // the grid is sized for the longest segment
+      if (a.cu_q != nullptr) {
+        dseg = vseg;
+      } else {
+        q_begin = a.seg_q_begin[vseg];
+        q_end = q_begin + a.seg_q_len[vseg];
+      }
     }
   } else {
     seg_begin = a.job_begin[job];
     seg_end = a.job_begin[job + 1];
     out_ptr = a.job_out[job];
     lse_ptr = a.job_lse[job];
-    q_begin = a.job_q_begin[job];
-    q_end = q_begin + a.job_q_len[job];
-    if (qt * kBQ >= q_end - q_begin) return;  // the grid is sized for the longest job
+    if (a.cu_q != nullptr) {
+      dseg = a.job_q_begin[job];
+    } else {
+      q_begin = a.job_q_begin[job];
+      q_end = q_begin + a.job_q_len[job];
+    }
   }
+  if (dseg >= 0) {
+    // boundaries from device memory: nothing on the host has looked at them, so they are clamped
+    // to the rows that exist (a malformed list then yields wrong rows, never a stray access)
+    q_begin = min(max(__builtin_amdgcn_readfirstlane(a.cu_q[dseg]), 0), a.Sq);
+    q_end = min(max(__builtin_amdgcn_readfirstlane(a.cu_q[dseg + 1]), q_begin), a.Sq);
+  }
+  if (qt * kBQ >= q_end - q_begin) return;  // the grid is sized for the longest job / segment
   auto chunk_of = [&](int seg) -> int { return single >= 0 ? single : a.job_chunks[seg]; };
+  // keys [begin, begin + len) of chunk reference `seg`
   auto kv_begin_of = [&](int seg) -> int {
+    if (dseg >= 0) {
+      const int cid = chunk_of(seg);
+      return min(max(__builtin_amdgcn_readfirstlane(a.cu_kv[cid][dseg]), 0), a.kv_len[cid]);
+    }
     if (single < 0) return a.entry_kv_begin[seg];
     return vseg >= 0 ? a.entry_kv_begin[single * a.n_seg + vseg] : 0;
   };
   auto kv_len_of = [&](int seg) -> int {
+    if (dseg >= 0) {
+      const int cid = chunk_of(seg);
+      const int lo = min(max(__builtin_amdgcn_readfirstlane(a.cu_kv[cid][dseg]), 0), a.kv_len[cid]);
+      const int hi = min(max(__builtin_amdgcn_readfirstlane(a.cu_kv[cid][dseg + 1]), lo), a.kv_len[cid]);
+      return hi - lo;
+    }
     if (single < 0) return a.entry_kv_len[seg];
     return vseg >= 0 ? a.entry_kv_len[single * a.n_seg + vseg] : a.kv_len[single];
   };
@@ -889,109 +914,8 @@ __global__ __launch_bounds__(256) void attn_tail_fold_kernel(const AttnArgs a) {
   }
 }
 
-// Measurement aid: back-to-back bf16 MFMAs on registers, nothing else -- the rate (and the shader
-// clock) this part sustains when only the matrix pipes work, i.e. what the power limit leaves of the
-// nominal peak.  Same launch shape as the attention kernel (512 threads, two wavefronts per SIMD).
-// Four accumulators keep four independent MFMAs in flight; the operands rotate through four register
-// sets of pseudo-random values so that the operand buses toggle as they do on real data.
-__global__ __launch_bounds__(kThreads, 2) void mfma_probe_kernel(float* sink, int iters) {
-  const uint32_t lane = threadIdx.x;
-  bf16x8 av[4], bv[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j)
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      uint32_t ha = (lane * 8u + e + 1u) * 2654435761u + j * 40503u;
-      uint32_t hb = (lane * 8u + e + 7u) * 2246822519u + j * 9973u;
-      ha ^= ha >> 15;
-      hb ^= hb >> 13;
-      av[j][e] = (__bf16)((float)(int)(ha & 255u) * (1.f / 128.f) - 1.f);
-      bv[j][e] = (__bf16)((float)(int)(hb & 255u) * (1.f / 128.f) - 1.f);
-    }
-  f32x16 acc[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) acc[j][r] = 0.f;
-  for (int i = 0; i < iters; i += 4) {   // iters is rounded up to a multiple of 4; register indices stay static
-#pragma unroll
-    for (int u = 0; u < 4; ++u)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[j], bv[(j + u) & 3], acc[j], 0, 0, 0);
-  }
-  float total = 0.f;
-#pragma unroll
-  for (int j = 0; j < 4; ++j)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) total += acc[j][r];
-  if (total == 12345.678f) sink[0] = total;   // keeps the MFMAs alive; (almost) never true
-}
-
-// Measurement aid: what two wavefronts of a SIMD can issue side by side.  Wavefronts 0-3 of a workgroup (one
-// per SIMD) issue 4 * iters back-to-back MFMAs as above; wavefronts 4-7 (the other wavefront of each SIMD)
-// issue, per MFMA of their neighbour, the vector instructions the online softmax spends per MFMA of the
-// attention kernel: kMix = 1 (head dimension 128: 32 MFMAs per 64-key tile against 32 fma, 32 exp, 32 add
-// and 16 cvt) one v_fma_f32, one v_exp_f32, one v_add_f32 and half a v_cvt_pk_bf16_f32; kMix = 2 (head
-// dimension 64, half the MFMAs per softmax element) twice that; kMix = 0 nothing (the MFMA wavefronts alone).
-// The launch reserves the attention kernel's LDS for that head dimension, so one (128) or two (64) workgroups share a CU as there.
-// The instructions are written out so that the mix is exactly this; their values do not matter.
-template <int kMix>
-__global__ __launch_bounds__(kThreads, 2) void coissue_probe_kernel(float* sink, int iters) {
-  extern __shared__ __attribute__((aligned(16))) uint8_t probe_lds[];   // unused: sized by the launch to set the occupancy
-  const uint32_t lane = threadIdx.x;
-  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-  float total = 0.f;
-  if (wave < 4) {
-    bf16x8 av[4], bv[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        uint32_t ha = (lane * 8u + e + 1u) * 2654435761u + j * 40503u;
-        uint32_t hb = (lane * 8u + e + 7u) * 2246822519u + j * 9973u;
-        ha ^= ha >> 15;
-        hb ^= hb >> 13;
-        av[j][e] = (__bf16)((float)(int)(ha & 255u) * (1.f / 128.f) - 1.f);
-        bv[j][e] = (__bf16)((float)(int)(hb & 255u) * (1.f / 128.f) - 1.f);
-      }
-    f32x16 acc[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[j][r] = 0.f;
-    for (int i = 0; i < iters; i += 4) {
-#pragma unroll
-      for (int u = 0; u < 4; ++u)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[j], bv[(j + u) & 3], acc[j], 0, 0, 0);
-    }
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) total += acc[j][r];
-  } else if (kMix > 0) {
-    float s[8], t[8], rs0 = 0.f, rs1 = 0.f;
-    const float c = 0.18f, m = -0.25f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) s[e] = (float)(int)((lane * 8u + e) & 63u) * 0.05f - 1.6f;
-    uint32_t pk = 0;
-    for (int i = 0; i < iters; ++i) {   // one trip = the vector work beside 4 MFMAs
-#pragma unroll
-      for (int e = 0; e < 4 * kMix; ++e) {
-        asm volatile("v_fma_f32 %0, %1, %2, %3" : "=v"(t[e]) : "v"(s[e]), "v"(c), "v"(m));
-        asm volatile("v_exp_f32 %0, %0" : "+v"(t[e]));
-      }
-#pragma unroll
-      for (int e = 0; e < 4 * kMix; e += 2) {
-        asm volatile("v_add_f32 %0, %1, %0" : "+v"(rs0) : "v"(t[e]));
-        asm volatile("v_add_f32 %0, %1, %0" : "+v"(rs1) : "v"(t[e + 1]));
-        asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(pk) : "v"(t[e]), "v"(t[e + 1]));
-      }
-    }
-    total = rs0 + rs1 + (float)pk;
-  }
-  if (total == 12345.678f) sink[0] = total;   // keeps the work alive; (almost) never true
-}
+static_assert(Tile<128>::kLdsBytes == kAttnLdsBytes128 && Tile<64>::kLdsBytes == kAttnLdsBytes64,
+              "dt_common.h states the LDS footprint of the attention kernel");
 
 template <int D, bool kPre>
 static int launch_one(const AttnArgs& a, dim3 grid, hipStream_t stream) {
@@ -1117,8 +1041,9 @@ int launch_attn(const AttnArgs& a_in, int D, int n_jobs, hipStream_t stream, voi
     }
   }
   if (tail == 0) return launch_dim(a, D, dim3((unsigned)slots_per_job, (unsigned)n_jobs, 1), stream);
+  // (the planner only considers splits of at most `cap` slots, so this cannot fire; it guards later edits to it)
   if ((int64_t)tail * ways * slot_bytes > workspace_bytes) {
-    set_error("tail split of %d items x %d parts needs %lld bytes of scratch, %lld are there", tail, ways,
+    set_error("internal: tail split of %d items x %d parts needs %lld bytes of scratch, %lld are there", tail, ways,
               (long long)((int64_t)tail * ways * slot_bytes), (long long)workspace_bytes);
     return DT_ERR_INVALID;
   }
@@ -1139,42 +1064,3 @@ int launch_attn(const AttnArgs& a_in, int D, int n_jobs, hipStream_t stream, voi
 }
 
 }  // namespace dt
-
-template <int kMix>
-static int launch_coissue(int workgroups, int iters, size_t lds_bytes, float* sink, hipStream_t stream) {
-  // more than 64 KB of dynamic LDS has to be allowed once per kernel and device
-  static thread_local int allowed_dev = -1;
-  int dev = 0;
-  if (int rc = dt::hip_fail(hipGetDevice(&dev), "hipGetDevice")) return rc;
-  if (allowed_dev != dev) {
-    if (int rc = dt::hip_fail(hipFuncSetAttribute(reinterpret_cast<const void*>(&dt::coissue_probe_kernel<kMix>),
-                                                  hipFuncAttributeMaxDynamicSharedMemorySize, dt::Tile<128>::kLdsBytes),
-                              "hipFuncSetAttribute"))
-      return rc;
-    allowed_dev = dev;
-  }
-  hipLaunchKernelGGL(dt::coissue_probe_kernel<kMix>, dim3((unsigned)workgroups), dim3(dt::kThreads), lds_bytes, stream, sink, iters);
-  return dt::hip_fail(hipGetLastError(), "coissue_probe launch");
-}
-
-extern "C" int dt_coissue_probe(int32_t workgroups, int32_t iters, int32_t head_dim, int32_t with_softmax, float* sink,
-                                void* stream) {
-  if (workgroups <= 0 || iters <= 0 || iters % 4 != 0 || !sink || (head_dim != 64 && head_dim != 128)) {
-    dt::set_error("co-issue probe: workgroups and iters must be positive, iters a multiple of 4, head_dim 64 or 128, and sink non-null");
-    return DT_ERR_INVALID;
-  }
-  // the attention kernel's LDS footprint decides how many workgroups share a CU, as it does there
-  const size_t lds = head_dim == 128 ? dt::Tile<128>::kLdsBytes : dt::Tile<64>::kLdsBytes;
-  if (!with_softmax) return launch_coissue<0>(workgroups, iters, lds, sink, (hipStream_t)stream);
-  if (head_dim == 128) return launch_coissue<1>(workgroups, iters, lds, sink, (hipStream_t)stream);
-  return launch_coissue<2>(workgroups, iters, lds, sink, (hipStream_t)stream);
-}
-
-extern "C" int dt_mfma_probe(int32_t workgroups, int32_t iters, float* sink, void* stream) {
-  if (workgroups <= 0 || iters <= 0 || iters % 4 != 0 || !sink) {
-    dt::set_error("mfma probe: workgroups and iters must be positive, iters a multiple of 4, and sink non-null");
-    return DT_ERR_INVALID;
-  }
-  hipLaunchKernelGGL(dt::mfma_probe_kernel, dim3((unsigned)workgroups), dim3(dt::kThreads), 0, (hipStream_t)stream, sink, iters);
-  return dt::hip_fail(hipGetLastError(), "mfma_probe launch");
-}

@@ -193,6 +193,93 @@ extern "C" int dt_attn_seg_jobs_ws_fwd(const void* q, int32_t B, int32_t Sq, int
   return launch_attn(a, D, n_jobs, (hipStream_t)stream, workspace, workspace_bytes, job_q_begin == nullptr);
 }
 
+// Device-resident segment boundaries: shared checks of the two varlen entry points.
+static int fill_device_segments(AttnArgs& a, int32_t n_chunks, const int32_t* kv_lens, int32_t n_seg,
+                                const int32_t* cu_seqlens_q, const int32_t* const* cu_seqlens_kv, int32_t max_seqlen_q,
+                                int32_t B, int32_t Sq, int32_t H) {
+  if (n_seg <= 0 || !cu_seqlens_q || !cu_seqlens_kv) {
+    set_error("device segment boundaries: need n_seg > 0, cu_seqlens_q and the per-chunk cu_seqlens_kv table");
+    return DT_ERR_INVALID;
+  }
+  if (max_seqlen_q <= 0) {
+    set_error("max_seqlen_q must be positive (got %d): it sizes the grid, the boundaries themselves are never read on the host", max_seqlen_q);
+    return DT_ERR_INVALID;
+  }
+  if ((reinterpret_cast<uintptr_t>(cu_seqlens_q) & 3) != 0) {
+    set_error("cu_seqlens_q must be 4-byte aligned");
+    return DT_ERR_INVALID;
+  }
+  for (int c = 0; c < n_chunks; ++c) {
+    if (kv_lens[c] > 0 && (!cu_seqlens_kv[c] || (reinterpret_cast<uintptr_t>(cu_seqlens_kv[c]) & 3) != 0)) {
+      set_error("chunk %d: null or misaligned cu_seqlens_kv", c);
+      return DT_ERR_INVALID;
+    }
+    // an empty chunk is never dereferenced for keys, but the kernel still reads its boundaries: point it at the queries'
+    a.cu_kv[c] = cu_seqlens_kv[c] ? cu_seqlens_kv[c] : cu_seqlens_q;
+  }
+  a.cu_q = cu_seqlens_q;
+  // size the grid for the longest segment the caller promises; shorter ones leave their surplus workgroups at once
+  a.nqt = ((max_seqlen_q < Sq ? max_seqlen_q : Sq) + 255) / 256;
+  a.total = B * H * a.nqt;
+  a.per_xcd = (a.total + 7) / 8;
+  return DT_OK;
+}
+
+extern "C" int dt_attn_varlen_jobs_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D, int64_t q_sb,
+                                       int64_t q_ss, int64_t q_sh, int32_t n_chunks, const void* const* k_ptrs,
+                                       const void* const* v_ptrs, const int32_t* kv_lens, const int64_t* kv_sb,
+                                       int64_t kv_ss, int64_t kv_sh, int32_t n_jobs, const int32_t* job_begin,
+                                       const int32_t* job_chunks, const int32_t* job_segment, int32_t n_seg,
+                                       const int32_t* cu_seqlens_q, const int32_t* const* cu_seqlens_kv,
+                                       int32_t max_seqlen_q, void* const* out_ptrs, float* const* lse_ptrs,
+                                       float softmax_scale, int32_t flags, void* stream) {
+  AttnArgs a{};
+  if (int rc = fill_common(a, q, B, Sq, H, D, q_sb, q_ss, q_sh, n_chunks, k_ptrs, v_ptrs, kv_lens, kv_sb, kv_ss, kv_sh,
+                           softmax_scale))
+    return rc;
+  if (int rc = apply_flags(a, flags)) return rc;
+  if (n_jobs == 0) return DT_OK;
+  if (n_jobs < 0 || n_jobs > DT_MAX_JOBS || !job_begin || !job_chunks || !job_segment || !out_ptrs || !lse_ptrs) {
+    set_error("%d jobs: need 0..%d and non-null job tables", n_jobs, DT_MAX_JOBS);
+    return DT_ERR_INVALID;
+  }
+  if (job_begin[0] != 0 || job_begin[n_jobs] > DT_MAX_JOB_ENTRIES) {
+    set_error("job_begin must start at 0 and end at most at %d", DT_MAX_JOB_ENTRIES);
+    return DT_ERR_INVALID;
+  }
+  if (int rc = fill_device_segments(a, n_chunks, kv_lens, n_seg, cu_seqlens_q, cu_seqlens_kv, max_seqlen_q, B, Sq, H))
+    return rc;
+  for (int j = 0; j < n_jobs; ++j) {
+    if (job_begin[j + 1] < job_begin[j]) {
+      set_error("job_begin is not monotone at job %d", j);
+      return DT_ERR_INVALID;
+    }
+    if (!out_ptrs[j] || !lse_ptrs[j] || !aligned16(out_ptrs[j])) {
+      set_error("job %d: null or misaligned destination", j);
+      return DT_ERR_INVALID;
+    }
+    if (job_segment[j] < 0 || job_segment[j] >= n_seg) {
+      set_error("job %d: segment %d outside 0..%d", j, job_segment[j], n_seg - 1);
+      return DT_ERR_INVALID;
+    }
+    a.job_out[j] = static_cast<__bf16*>(out_ptrs[j]);
+    a.job_lse[j] = lse_ptrs[j];
+    a.job_begin[j] = job_begin[j];
+    a.job_q_begin[j] = job_segment[j];   // with device boundaries this field names the segment
+    a.job_q_len[j] = 0;
+  }
+  a.job_begin[n_jobs] = job_begin[n_jobs];
+  for (int e = 0; e < job_begin[n_jobs]; ++e) {
+    const int32_t c = job_chunks[e];
+    if (c < 0 || c >= n_chunks) {
+      set_error("job chunk reference %d is outside the chunk table", c);
+      return DT_ERR_INVALID;
+    }
+    a.job_chunks[e] = c;
+  }
+  return launch_attn(a, D, n_jobs, (hipStream_t)stream, nullptr, 0, false);
+}
+
 // The same launch for callers that cannot allocate: the tail is split inside the library's own
 // device array instead of a caller's workspace.
 extern "C" int dt_attn_seg_jobs_noalloc_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D, int64_t q_sb,
@@ -203,6 +290,19 @@ extern "C" int dt_attn_seg_jobs_noalloc_fwd(const void* q, int32_t B, int32_t Sq
                                             const int32_t* entry_kv_len, const int32_t* job_q_begin,
                                             const int32_t* job_q_len, void* const* out_ptrs, float* const* lse_ptrs,
                                             float softmax_scale, int32_t flags, void* stream) {
+  // The scratch array has one copy per GPU, at that GPU's own address, and the lookup below answers for the
+  // CURRENT device: it must be the one that owns the tensors (and the stream), or the kernel would be handed
+  // another GPU's array.
+  if (q) {
+    hipPointerAttribute_t attr{};
+    int dev = -1;
+    if (hipPointerGetAttributes(&attr, q) == hipSuccess && hipGetDevice(&dev) == hipSuccess &&
+        attr.type == hipMemoryTypeDevice && attr.device != dev) {
+      set_error("q lives on device %d but device %d is current: make the tensors' device current for this call", attr.device, dev);
+      return DT_ERR_INVALID;
+    }
+    (void)hipGetLastError();  // a pointer the runtime does not know leaves an error behind; the checks below report it properly
+  }
   void* scratch = nullptr;
   int64_t scratch_bytes = 0;
   if (int rc = static_tail_scratch(&scratch, &scratch_bytes)) return rc;
@@ -249,23 +349,11 @@ extern "C" int dt_attn_chunk_fwd(const void* q, const void* k, const void* v, vo
                           lses, softmax_scale, stream);
 }
 
-extern "C" int dt_attn_sched_seg_ws_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D, int64_t q_sb,
-                                        int64_t q_ss, int64_t q_sh, int32_t n_chunks, const void* const* k_ptrs,
-                                        const void* const* v_ptrs, const int32_t* kv_lens, const int64_t* kv_sb,
-                                        int64_t kv_ss, int64_t kv_sh, const int32_t* dev_compute_ids,
-                                        const int32_t* dev_count, int32_t max_jobs, void* slot_out,
-                                        int64_t slot_out_stride, float* slot_lse, int64_t slot_lse_stride,
-                                        int32_t diag, void* diag_out, float* diag_lse, int32_t n_seg,
-                                        const int32_t* seg_q_begin, const int32_t* seg_q_len,
-                                        const int32_t* seg_kv_begin, const int32_t* seg_kv_len, float softmax_scale,
-                                        int32_t flags, void* workspace, int64_t workspace_bytes, void* stream) {
-  if (int rc = check_workspace(workspace, workspace_bytes)) return rc;
-  AttnArgs a{};
-  if (int rc = fill_common(a, q, B, Sq, H, D, q_sb, q_ss, q_sh, n_chunks, k_ptrs, v_ptrs, kv_lens, kv_sb, kv_ss, kv_sh,
-                           softmax_scale))
-    return rc;
-  if (int rc = apply_flags(a, flags)) return rc;
-  if (max_jobs == 0) return DT_OK;
+// Checks and fields every device-scheduled launch shares.
+static int fill_sched(AttnArgs& a, int32_t n_chunks, const void* const* k_ptrs, const void* const* v_ptrs,
+                      const int32_t* kv_lens, const int32_t* dev_compute_ids, const int32_t* dev_count, int32_t max_jobs,
+                      void* slot_out, int64_t slot_out_stride, float* slot_lse, int64_t slot_lse_stride, int32_t diag,
+                      void* diag_out, float* diag_lse) {
   if (max_jobs < 0 || max_jobs > n_chunks) {
     set_error("max_jobs %d must be in 0..n_chunks (%d)", max_jobs, n_chunks);
     return DT_ERR_INVALID;
@@ -284,6 +372,38 @@ extern "C" int dt_attn_sched_seg_ws_fwd(const void* q, int32_t B, int32_t Sq, in
     set_error("diag chunk %d needs a destination outside the cache", diag);
     return DT_ERR_INVALID;
   }
+  a.dev_ids = dev_compute_ids;
+  a.dev_count = dev_count;
+  a.slot_out = static_cast<__bf16*>(slot_out);
+  a.slot_lse = slot_lse;
+  a.slot_out_stride = slot_out_stride;
+  a.slot_lse_stride = slot_lse_stride;
+  a.diag = diag;
+  a.diag_out = static_cast<__bf16*>(diag_out);
+  a.diag_lse = diag_lse;
+  return DT_OK;
+}
+
+extern "C" int dt_attn_sched_seg_ws_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D, int64_t q_sb,
+                                        int64_t q_ss, int64_t q_sh, int32_t n_chunks, const void* const* k_ptrs,
+                                        const void* const* v_ptrs, const int32_t* kv_lens, const int64_t* kv_sb,
+                                        int64_t kv_ss, int64_t kv_sh, const int32_t* dev_compute_ids,
+                                        const int32_t* dev_count, int32_t max_jobs, void* slot_out,
+                                        int64_t slot_out_stride, float* slot_lse, int64_t slot_lse_stride,
+                                        int32_t diag, void* diag_out, float* diag_lse, int32_t n_seg,
+                                        const int32_t* seg_q_begin, const int32_t* seg_q_len,
+                                        const int32_t* seg_kv_begin, const int32_t* seg_kv_len, float softmax_scale,
+                                        int32_t flags, void* workspace, int64_t workspace_bytes, void* stream) {
+  if (int rc = check_workspace(workspace, workspace_bytes)) return rc;
+  AttnArgs a{};
+  if (int rc = fill_common(a, q, B, Sq, H, D, q_sb, q_ss, q_sh, n_chunks, k_ptrs, v_ptrs, kv_lens, kv_sb, kv_ss, kv_sh,
+                           softmax_scale))
+    return rc;
+  if (int rc = apply_flags(a, flags)) return rc;
+  if (max_jobs == 0) return DT_OK;
+  if (int rc = fill_sched(a, n_chunks, k_ptrs, v_ptrs, kv_lens, dev_compute_ids, dev_count, max_jobs, slot_out,
+                          slot_out_stride, slot_lse, slot_lse_stride, diag, diag_out, diag_lse))
+    return rc;
   int32_t jobs = max_jobs;
   if (n_seg != 0) {
     if (n_seg < 0 || n_seg > DT_MAX_SEGMENTS || (int64_t)n_seg * n_chunks > DT_MAX_JOB_ENTRIES) {
@@ -324,16 +444,35 @@ extern "C" int dt_attn_sched_seg_ws_fwd(const void* q, int32_t B, int32_t Sq, in
     a.per_xcd = (a.total + 7) / 8;
     jobs = max_jobs * n_seg;
   }
-  a.dev_ids = dev_compute_ids;
-  a.dev_count = dev_count;
-  a.slot_out = static_cast<__bf16*>(slot_out);
-  a.slot_lse = slot_lse;
-  a.slot_out_stride = slot_out_stride;
-  a.slot_lse_stride = slot_lse_stride;
-  a.diag = diag;
-  a.diag_out = static_cast<__bf16*>(diag_out);
-  a.diag_lse = diag_lse;
   return launch_attn(a, D, jobs, (hipStream_t)stream, workspace, workspace_bytes, n_seg == 0);
+}
+
+extern "C" int dt_attn_sched_varlen_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D, int64_t q_sb,
+                                        int64_t q_ss, int64_t q_sh, int32_t n_chunks, const void* const* k_ptrs,
+                                        const void* const* v_ptrs, const int32_t* kv_lens, const int64_t* kv_sb,
+                                        int64_t kv_ss, int64_t kv_sh, const int32_t* dev_compute_ids,
+                                        const int32_t* dev_count, int32_t max_jobs, void* slot_out,
+                                        int64_t slot_out_stride, float* slot_lse, int64_t slot_lse_stride,
+                                        int32_t diag, void* diag_out, float* diag_lse, int32_t n_seg,
+                                        const int32_t* cu_seqlens_q, const int32_t* const* cu_seqlens_kv,
+                                        int32_t max_seqlen_q, float softmax_scale, int32_t flags, void* stream) {
+  AttnArgs a{};
+  if (int rc = fill_common(a, q, B, Sq, H, D, q_sb, q_ss, q_sh, n_chunks, k_ptrs, v_ptrs, kv_lens, kv_sb, kv_ss, kv_sh,
+                           softmax_scale))
+    return rc;
+  if (int rc = apply_flags(a, flags)) return rc;
+  if (max_jobs == 0) return DT_OK;
+  if (int rc = fill_sched(a, n_chunks, k_ptrs, v_ptrs, kv_lens, dev_compute_ids, dev_count, max_jobs, slot_out,
+                          slot_out_stride, slot_lse, slot_lse_stride, diag, diag_out, diag_lse))
+    return rc;
+  if (n_seg <= 0 || (int64_t)n_seg * max_jobs > 65535) {
+    set_error("%d segments x %d scheduled chunks: need at least one segment and at most 65535 launch planes", n_seg, max_jobs);
+    return DT_ERR_INVALID;
+  }
+  if (int rc = fill_device_segments(a, n_chunks, kv_lens, n_seg, cu_seqlens_q, cu_seqlens_kv, max_seqlen_q, B, Sq, H))
+    return rc;
+  a.n_seg = n_seg;
+  return launch_attn(a, D, max_jobs * n_seg, (hipStream_t)stream, nullptr, 0, false);
 }
 
 extern "C" int dt_attn_sched_seg_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D, int64_t q_sb,

@@ -54,6 +54,13 @@ struct AttnArgs {
   int32_t n_seg;
   int32_t seg_q_begin[DT_MAX_SEGMENTS];
   int32_t seg_q_len[DT_MAX_SEGMENTS];
+  // Segment boundaries that live in DEVICE memory (cu_q != nullptr), the calling convention of
+  // flash_attn_varlen_func: cu_q[s], cu_q[s + 1] bound the query rows of segment s and cu_kv[c][s],
+  // cu_kv[c][s + 1] its keys inside chunk c (every chunk brings its own boundaries).  The host never
+  // reads them; the kernel clamps them to the tensors' extents.  A host-listed job then names its
+  // segment in job_q_begin[job]; a device-listed job is segment job % n_seg as above.
+  const int32_t* cu_q;
+  const int32_t* cu_kv[DT_MAX_CHUNKS];
   // Tail balancing (workspace launches only).  The workgroups of a launch are equal pieces of
   // work, so its last round usually fills only part of the chip.  The main launch then leaves
   // the work items with index >= tail_idx0 of job tail_job alone (tail_job < 0: nothing is left);
@@ -70,6 +77,11 @@ struct AttnArgs {
   float* ws_lse;    // [slot][256]
 };
 
+// Dynamic LDS of one attention workgroup by head dimension (four 64-key buffers per operand).  The
+// occupancy of a CU follows from it: one workgroup at 128, two at 64.
+constexpr int kAttnLdsBytes128 = 131072;
+constexpr int kAttnLdsBytes64 = 65536;
+
 // Workspace bytes the tail balancing can use at most (what dt_attn_workspace_bytes reports).
 constexpr int64_t kMaxTailSlots = 1536;
 
@@ -79,6 +91,8 @@ constexpr int64_t kStaticTailSlots = DT_NOALLOC_TAIL_SLOTS;
 constexpr int64_t kStaticTailBytes = kStaticTailSlots * (256 * 128 * 2 + 256 * 4);
 // Device address and size of that array on the current device (looked up once per device).
 int static_tail_scratch(void** ptr, int64_t* bytes);
+
+static_assert(sizeof(AttnArgs) <= 4096, "the kernel arguments travel in the 4 KB kernarg segment");
 
 int launch_attn(const AttnArgs& a, int D, int n_jobs, hipStream_t stream, void* workspace = nullptr,
                 int64_t workspace_bytes = 0, bool balance = false);

@@ -698,37 +698,16 @@ __global__ __launch_bounds__(kThreads) void rel_l1_sums_kernel(const float* a, c
   }
 }
 
-// Yardstick for the kernels above: reads n streams the way the merge kernel reads its states
-// (a workgroup takes 32 consecutive 256-byte rows of every stream, 16 bytes per lane, all streams of
-// a batch of 8 in flight before the first use) and discards the data.
-struct ProbeArgs {
-  const uint8_t* stream[DT_MAX_MERGE];
-  int32_t n;
-  int64_t rows;  // 256-byte rows per stream
-  uint32_t* sink;
-};
-
-__global__ __launch_bounds__(kThreads) void hbm_read_probe_kernel(const ProbeArgs a) {
-  const int64_t row = (int64_t)blockIdx.x * 32 + threadIdx.x / 16;
-  const int c = threadIdx.x % 16;
-  uint32_t acc = 0;
-  for (int s0 = 0; s0 < a.n; s0 += kBatch) {
-    u32x4 v[kBatch][2];
-#pragma unroll
-    for (int s = 0; s < kBatch; ++s)
-#pragma unroll
-      for (int p = 0; p < 2; ++p) {
-        const int64_t r = row + 16 * p;
-        v[s][p] = u32x4{0u, 0u, 0u, 0u};
-        if (s0 + s < a.n && r < a.rows) v[s][p] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(a.stream[s0 + s] + r * 256 + 16 * c));
-      }
-#pragma unroll
-    for (int s = 0; s < kBatch; ++s)
-#pragma unroll
-      for (int p = 0; p < 2; ++p) acc ^= v[s][p].x ^ v[s][p].y ^ v[s][p].z ^ v[s][p].w;
-  }
-  // keeps the loads alive; a real store happens only for one bit pattern in 2^32 per lane
-  if (acc == 0x9e3779b9u) a.sink[0] = acc;
+// Zeroes the 16-byte units behind row *first_row of a dense [n_rows, row_bytes] tensor (the rows of a packed
+// batch that belong to no segment).  A fixed, small grid walks the range; with nothing to clear -- the usual
+// case -- every lane leaves after one scalar load.
+__global__ __launch_bounds__(kThreads) void zero_rows_from_kernel(u32x4* dst, int64_t n_rows, int64_t units_per_row,
+                                                                 const int32_t* first_row) {
+  int64_t first = *first_row;
+  first = first < 0 ? 0 : (first > n_rows ? n_rows : first);
+  const int64_t begin = first * units_per_row, end = n_rows * units_per_row;
+  for (int64_t i = begin + (int64_t)blockIdx.x * kThreads + threadIdx.x; i < end; i += (int64_t)gridDim.x * kThreads)
+    dst[i] = u32x4{0u, 0u, 0u, 0u};
 }
 
 // ---- host-side launchers ---------------------------------------------------------------
@@ -976,30 +955,15 @@ extern "C" int dt_build_schedule_table(const uint8_t* mask, int32_t T, int32_t L
   return hip_fail(hipGetLastError(), "build_schedule_table launch");
 }
 
-extern "C" int dt_hbm_read_probe(const void* const* streams, int32_t n_streams, int64_t bytes, uint32_t* sink,
-                                 void* stream) {
-  if (!streams || !sink || n_streams <= 0 || n_streams > DT_MAX_MERGE || bytes <= 0 || (bytes % 256)) {
-    set_error("read probe: need 1..%d streams of a positive multiple of 256 bytes and a sink", DT_MAX_MERGE);
+extern "C" int dt_zero_rows_from(void* dst, int64_t n_rows, int64_t row_bytes, const int32_t* first_row, void* stream) {
+  if (!dst || !first_row || !aligned16(dst) || n_rows < 0 || row_bytes <= 0 || (row_bytes % 16)) {
+    set_error("zero_rows_from: need a 16-byte aligned tensor, rows of a positive multiple of 16 bytes and a device row index");
     return DT_ERR_INVALID;
   }
-  ProbeArgs a{};
-  for (int i = 0; i < n_streams; ++i) {
-    if (!streams[i] || !aligned16(streams[i])) {
-      set_error("read probe: stream %d is null or misaligned", i);
-      return DT_ERR_INVALID;
-    }
-    a.stream[i] = static_cast<const uint8_t*>(streams[i]);
-  }
-  a.n = n_streams;
-  a.rows = bytes / 256;
-  a.sink = sink;
-  const int64_t wgs = (a.rows + 31) / 32;
-  if (wgs > 0x7fffffffLL) {
-    set_error("read probe grid too large");
-    return DT_ERR_INVALID;
-  }
-  hipLaunchKernelGGL(hbm_read_probe_kernel, dim3((unsigned)wgs), dim3(kThreads), 0, (hipStream_t)stream, a);
-  return hip_fail(hipGetLastError(), "hbm_read_probe launch");
+  if (n_rows == 0) return DT_OK;
+  hipLaunchKernelGGL(zero_rows_from_kernel, dim3(512), dim3(kThreads), 0, (hipStream_t)stream, static_cast<u32x4*>(dst),
+                     n_rows, row_bytes / 16, first_row);
+  return hip_fail(hipGetLastError(), "zero_rows_from launch");
 }
 
 extern "C" int dt_rel_l1_sums(const float* a, const float* b, int64_t n, double* sums, void* stream) {

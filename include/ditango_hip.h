@@ -75,8 +75,9 @@ int dt_attn_chunk_fwd(const void* q, const void* k, const void* v, void* out, fl
                       float softmax_scale, void* stream);
 
 /*
- * The same for fp32 tensors, computed in fp32 throughout (vector ALU, expf / logf): the attention
- * of the fp32 numbers themselves, not of their bf16 roundings.  flash_attn_func takes no fp32; the
+ * The same call site (core/attention.py:185-191) for fp32 tensors, computed in fp32 throughout (vector
+ * ALU, expf / logf): the attention of the fp32 numbers themselves, not of their bf16 roundings.
+ * flash_attn_func takes no fp32; the
  * reference runs its CPU-runnable configuration (fp32, B=1, H=4, d=64, 512 queries x 4 chunks of
  * 512 keys) on its torch math path, and this entry point is that path's counterpart here.  q / k / v
  * fp32 with element strides and a contiguous last dimension; out fp32 [B,Sq,H,D] contiguous, lse
@@ -176,7 +177,57 @@ int dt_attn_sched_seg_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32
                           float softmax_scale, void* stream);
 
 /*
- * The two launches above with a workspace (device memory, 16-byte aligned, at most
+ * The two variable-length launches with the segment boundaries in DEVICE memory -- the calling
+ * convention of
+ *   flash_attn_varlen_func(q, k, v, cu_seqlens_q, cu_seqlens_kv, max_seqlen_q, max_seqlen_kv, ...)
+ * at core/attention.py:314-324 and :366-376, whose cu_seqlens are int32 device tensors
+ * (executor/hunyuanvideo/hunyuan_transformer.py:789-792) and, for the other chunks, arrive with K/V
+ * over the ring (core/attention.py:307-311).  The host never reads them: no copy, no synchronisation,
+ * and the launch can be captured in a HIP graph while the boundaries change between replays.
+ *   cu_seqlens_q   device int32 [n_seg + 1]: segment s covers query rows [cu_q[s], cu_q[s+1])
+ *   cu_seqlens_kv  HOST array of n_chunks device pointers, each int32 [n_seg + 1]: the keys of segment
+ *                  s inside chunk c are [cu_kv[c][s], cu_kv[c][s+1]) (NULL allowed for an empty chunk)
+ *   max_seqlen_q   host upper bound of the segment lengths; it sizes the grid, so rows of a longer
+ *                  segment would be left uncomputed (flash-attn's contract for the same argument)
+ * The kernel clamps every boundary it reads to the rows / keys that exist, so a malformed list gives
+ * wrong rows but no stray access.  n_seg is not limited by DT_MAX_SEGMENTS (n_seg * max_jobs <= 65535).
+ * dt_attn_varlen_jobs_fwd: job j is segment job_segment[j] (HOST array) of the state (out_ptrs[j],
+ * lse_ptrs[j]) over its chunk list; the segments of one state are separate jobs with one destination.
+ * dt_attn_sched_varlen_fwd: every scheduled chunk runs once per segment, as in dt_attn_sched_seg_fwd.
+ * No tail balancing (the jobs cover row sub-ranges), hence no workspace.
+ */
+int dt_attn_varlen_jobs_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D,
+                            int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
+                            int32_t n_chunks, const void* const* k_ptrs, const void* const* v_ptrs,
+                            const int32_t* kv_lens, const int64_t* kv_stride_b,
+                            int64_t kv_stride_s, int64_t kv_stride_h,
+                            int32_t n_jobs, const int32_t* job_begin, const int32_t* job_chunks,
+                            const int32_t* job_segment, int32_t n_seg,
+                            const int32_t* cu_seqlens_q, const int32_t* const* cu_seqlens_kv, int32_t max_seqlen_q,
+                            void* const* out_ptrs, float* const* lse_ptrs,
+                            float softmax_scale, int32_t flags, void* stream);
+int dt_attn_sched_varlen_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D,
+                             int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
+                             int32_t n_chunks, const void* const* k_ptrs, const void* const* v_ptrs,
+                             const int32_t* kv_lens, const int64_t* kv_stride_b,
+                             int64_t kv_stride_s, int64_t kv_stride_h,
+                             const int32_t* dev_compute_ids, const int32_t* dev_count, int32_t max_jobs,
+                             void* slot_out, int64_t slot_out_stride, float* slot_lse, int64_t slot_lse_stride,
+                             int32_t diag, void* diag_out, float* diag_lse,
+                             int32_t n_seg, const int32_t* cu_seqlens_q, const int32_t* const* cu_seqlens_kv,
+                             int32_t max_seqlen_q, float softmax_scale, int32_t flags, void* stream);
+
+/*
+ * Zeroes the rows [*first_row, n_rows) of a dense [n_rows, row_bytes] tensor, first_row read from
+ * DEVICE memory (clamped to 0..n_rows): rows of a packed batch that belong to no segment
+ * (cu_seqlens_q[n_seg] < total) come out of flash_attn_varlen_func as zeros, and with the boundaries
+ * on the device the host cannot slice them off.  row_bytes a multiple of 16, dst 16-byte aligned.
+ * Stands in for that part of the call at core/attention.py:314-324.
+ */
+int dt_zero_rows_from(void* dst, int64_t n_rows, int64_t row_bytes, const int32_t* first_row, void* stream);
+
+/*
+ * dt_attn_seg_jobs_fwd and dt_attn_sched_seg_fwd with a workspace (device memory, 16-byte aligned, at most
  * dt_attn_workspace_bytes() are used; NULL or too small: plain launch).  All workgroups of an
  * attention launch are equal pieces of work, so its last round usually fills only part of the
  * chip; with a workspace the work items of that round are each cut into several ranges of key
@@ -225,12 +276,14 @@ int dt_attn_sched_seg_ws_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, in
  * library runs on until the process ends).  No counterpart in the reference.  Arguments, limits,
  * errors and results are those of dt_attn_seg_jobs_ws_fwd called with a workspace of exactly that
  * size: the split is planned to fit the array (a tail that would need more parts gets fewer), so the
- * scratch need does not grow with the input and no shape is turned away on its account; a plan
- * that does not fit is refused with DT_ERR_INVALID instead of being launched.  The call makes no
- * hipMalloc / hipFree; the array's device address is looked up once per device on the first call
- * there (hipGetSymbolAddress: make that first call outside a graph capture).  All calls on one GPU share the array: calls that overlap in time on one GPU (different
- * streams or threads) race on it; order them on one stream.  Nothing in the array has to start at
- * zero (every partial state that is read was written by the same call).
+ * scratch need does not grow with the input and no shape is turned away on its account.  The call
+ * makes no hipMalloc / hipFree; the array's device address is looked up once per device on the first
+ * call there (hipGetSymbolAddress: make that first call outside a graph capture).  Every GPU holds
+ * its own copy of the array and the lookup answers for the CURRENT device, so the device that owns
+ * q / out (and the stream) must be current when the call is made; a q that lives on another device
+ * is refused with DT_ERR_INVALID.  All calls on one GPU share the array: calls that overlap in time
+ * on one GPU (different streams or threads) race on it; order them on one stream.  Nothing in the
+ * array has to start at zero (every partial state that is read was written by the same call).
  */
 #define DT_NOALLOC_TAIL_SLOTS 512
 int dt_attn_seg_jobs_noalloc_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D,
@@ -302,40 +355,6 @@ int dt_build_schedule_table(const uint8_t* mask, int32_t T, int32_t L, int32_t C
  * (core/redundancy_map.py:174-197).  a, b are fp32, n elements.
  */
 int dt_rel_l1_sums(const float* a, const float* b, int64_t n, double* sums, void* stream);
-
-/*
- * Measurement aid, no counterpart in the reference: reads n_streams device buffers of `bytes` bytes
- * each (a multiple of 256) with the access pattern of dt_merge_states (a workgroup takes 32
- * consecutive 256-byte rows of every stream, eight streams in flight at a time) and discards the
- * data.  Its rate is what this part's memory system delivers to that pattern, the yardstick next to
- * the nominal HBM peak for the merge and cache kernels.  sink: one device word, (almost) never written.
- */
-int dt_hbm_read_probe(const void* const* streams, int32_t n_streams, int64_t bytes, uint32_t* sink, void* stream);
-
-/*
- * Measurement aid, no counterpart in the reference: `workgroups` workgroups of 8 wavefronts (two per
- * SIMD, the attention kernel's launch shape) each issue 4 * iters (iters a multiple of 4) back-to-back
- * v_mfma_f32_32x32x16_bf16 on registers -- 32768 FLOP apiece, so a launch does
- * workgroups * 8 * 4 * iters * 32768 FLOP -- and nothing else.  Its rate is what the part sustains
- * when only the matrix pipes work (the power limit holds the shader clock below nominal): the
- * yardstick next to the nominal MFMA peak for dt_attn_*.  sink: one device word, (almost) never written.
- */
-int dt_mfma_probe(int32_t workgroups, int32_t iters, float* sink, void* stream);
-
-/*
- * Measurement aid, no counterpart in the reference: the same launch shape, but only ONE wavefront of each
- * SIMD issues the 4 * iters MFMAs (a launch does workgroups * 4 * 4 * iters * 32768 FLOP); with
- * with_softmax != 0 the other wavefront of the SIMD issues, per MFMA of its neighbour, the vector
- * instructions that the online softmax of dt_attn_* spends per MFMA at that head dimension: at 128 one
- * v_fma_f32, one v_exp_f32, one v_add_f32 and half a v_cvt_pk_bf16_f32; at 64 twice that.  The launch
- * reserves the attention kernel's LDS for head_dim, so one (128) or two (64) workgroups share a CU as
- * they do there.  The MFMA rate with the softmax against the rate without is the share of the matrix pipe
- * that the wavefronts of a SIMD can keep busy side by side for that instruction mix: the ceiling of the
- * attention kernel's MFMA utilisation before any LDS traffic, barrier or tile load.  sink: one device
- * word, (almost) never written.
- */
-int dt_coissue_probe(int32_t workgroups, int32_t iters, int32_t head_dim, int32_t with_softmax, float* sink,
-                     void* stream);
 
 /*
  * Producer side of an attention call: normalise every head row of x over D, apply the

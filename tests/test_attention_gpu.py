@@ -125,12 +125,87 @@ def test_stride_mode_matches_numeric_oracle(env, N, rank, D, col, max_job_chunks
         q, ks, vs = _perturb(q, g), [_perturb(k, g) for k in ks], [_perturb(v, g) for v in vs]
 
 
+@pytest.mark.parametrize("N,rank,D,col,trip", [
+    (8, 3, 128, (1, 1, 1, 4, 4, 2, 2, 1, 1), {2}),        # trips on the step that announces stride 2
+    (8, 0, 64, (1, 1, 1, 2, 2, 2, 2, 2, 1, 1), {4}),      # mid-run: one of two blocks held, the other predicted
+    (4, 2, 128, (1, 1, 1, 2, 2, 2, 4, 4, 1, 1), {2, 5}),
+])
+def test_stride_mode_memory_guard_fallback_matches_numeric_oracle(env, N, rank, D, col, trip):
+    """The stride-mode fallback of the memory guard (core/attention.py:97-98 with core/cache.py:103-128),
+    run on the kernels with an injected memory reading against the lock-step ring with the same reading:
+    on the tripping call the announced stride becomes N, nothing is stored and the cache is reset to N
+    empty slots; the NEXT call reads its stride from the map again, probes blocks of the empty cache and
+    computes only its target block, so the other chunks are missing from its softmax -- schedule and
+    numbers (out, lse of the partial softmax) must equal the oracle's."""
+    from ditango_amd.core.attention import proAttention
+    from ditango_amd.core.parallel_state import get_usp_group
+    from ditango_amd.utils import update_timestep
+
+    T, B, H, S = len(col), 1, 2, 100
+    rm = env(N, rank, T, 1)
+    rm.divider_map[:, 0] = torch.tensor(col)
+    curr, nxt = strides_from_dividers(N, col)
+    g = torch.Generator().manual_seed(29)
+    q, ks, vs = _inputs(B, S, [S] * N, H, D, seed=N * 7 + rank)
+    state, now = {}, {"t": 0}
+    probe = lambda: 950.0 if now["t"] in trip else 0.0       # MB allocated; budget 1000 MB, one block 100 MB
+
+    def attn_fn(r, c):
+        if r != rank:
+            return (c,)
+        return om.chunk_attention(state["q"], state["ks"][c], state["vs"][c])
+
+    def merge_fn(a, b):
+        if isinstance(b[0], int):
+            return tuple(b) if a is None else tuple(a) + tuple(b)
+        return om.update_out_and_lse(None if a is None else a[0], None if a is None else a[1], b[0], b[1])
+
+    def store_fn(s):
+        return s if isinstance(s[0], int) else (om.bf16_round(s[0]), s[1])
+
+    ring = RingOracle(N, attn_fn=attn_fn, merge_fn=merge_fn, store_fn=store_fn,
+                      memory_probe=probe, block_size_mb=100.0, memory_constraint=1000.0)
+    group = get_usp_group()
+    attn = proAttention(0, group)
+    attn.cache.block_size_mb, attn.cache.memory_constraint, attn.cache.memory_probe = 100.0, 1000.0, probe
+    tripped, dropped = set(), 0
+    for t in range(T):
+        print(f"case guard N={N} rank={rank} D={D} t={t} curr={curr[t]} next={nxt[t]} trip={t in trip}", flush=True)
+        now["t"] = t
+        qb, kb, vb = q.bfloat16(), [k.bfloat16() for k in ks], [v.bfloat16() for v in vs]
+        state.update(q=qb, ks=kb, vs=vb)
+        tr = ring.call(t, curr[t], nxt[t])[rank]
+        update_timestep(t)
+        dk, dv = [k.cuda() for k in kb], [v.cuda() for v in vb]
+        group.set_kv_chunks(dk, dv)
+        out = attn.attn(qb.cuda(), dk[rank], dv[rank])
+        torch.cuda.synchronize()
+        p = attn.last_plan
+        assert (p.curr_stride, p.next_stride) == (tr.curr_stride, tr.next_stride)
+        assert p.computed == tr.computed and p.reuse_probed == tr.reuse_probed and p.reuse_merged == tr.reuse_merged
+        assert p.stores == tr.stores and p.flushes == tr.flushes
+        assert (p.target_after, p.nblk_after, p.occupancy_after) == (tr.target_after, tr.nblk_after, tr.occupancy_after)
+        if tr.next_stride != nxt[t]:
+            tripped.add(t)
+            assert p.next_stride == N and p.stores == [] and attn.cache.curr_block_num == N
+            assert all(o is None for o in attn.cache.out_block_cache) and all(l is None for l in attn.cache.lse_block_cache)
+        if t - 1 in tripped and curr[t] != N:
+            assert p.reuse_probed and p.reuse_merged == []
+            dropped += N - len({c for c, _ in p.computed})
+        ref_out, ref_lse = tr.out
+        _cmp(out, attn.last_lse, ref_out, ref_lse.squeeze(-1).transpose(1, 2), f"guard t={t}")
+        q, ks, vs = _perturb(q, g), [_perturb(k, g) for k in ks], [_perturb(v, g) for v in vs]
+    assert tripped == trip and dropped > 0
+
+
 @pytest.mark.parametrize("C,diag,D,p,lens", [
     (8, 0, 128, 0.5, None),
     (8, 5, 64, 0.6, None),
     (6, -1, 128, 0.75, [70, 69, 69, 70, 1, 64]),     # ragged chunks, no local chunk
     (48, 5, 128, 0.5, None),                         # more chunks than one launch addresses: two windows
     (70, 43, 64, 0.6, None),                         # local chunk in the second window; 70-way merge
+    (48, 5, 128, 0.5, [90] * 40 + [0] * 8),          # the second window holds no key at all: it is not launched,
+                                                     # its scheduled chunks get the empty state (out 0, lse -inf)
 ])
 def test_mask_mode_matches_numeric_oracle(env, C, diag, D, p, lens):
     from ditango_amd.core.attention import proAttention
@@ -167,6 +242,71 @@ def test_mask_mode_matches_numeric_oracle(env, C, diag, D, p, lens):
             torch.cuda.synchronize()
             _cmp(out, layers[l].last_lse, ref_out, ref_lse, f"t={t} l={l}")
             q, ks, vs = _perturb(q, g), [_perturb(k, g) for k in ks], [_perturb(v, g) for v in vs]
+
+
+@pytest.mark.parametrize("N,rank,S_total,D", [(8, 7, 8 * 90 - 3, 128), (4, 3, 4 * 130 - 1, 64)])
+def test_zero_padded_shards_of_an_uneven_sequence(env, N, rank, S_total, D):
+    """The callers shard an uneven sequence with ``split_tensor_uneven`` (utils.py:86-136): the last shards
+    carry a zero-padded row, and the dense path does not mask it (utils.py:120-127) -- a padded key takes
+    part in the softmax with score 0, a padded query row is computed like any other.  Shards built by the
+    drop-in ``split_tensor_uneven`` go through ``attn`` (a full-stride call and a cached one) and must equal
+    the oracle on those same zero-padded chunks; and against attention over the UNPADDED sequence the merged
+    lse must be off by exactly the padded keys: exp(lse) = exp(lse_unpadded) + number of padded keys."""
+    from ditango_amd.core.attention import proAttention
+    from ditango_amd.core.parallel_state import get_usp_group
+    from ditango_amd.utils import get_padding_dict, split_tensor_uneven, update_timestep
+
+    B, H = 1, 3
+    col = (1, 1, 2, 2, 1)
+    T = len(col)
+    rm = env(N, rank, T, 1)
+    rm.divider_map[:, 0] = torch.tensor(col)
+    curr, nxt = strides_from_dividers(N, col)
+    g = torch.Generator().manual_seed(S_total)
+    q_full = torch.randn(B, S_total, H, D, generator=g).bfloat16()
+    k_full = torch.randn(B, S_total, H, D, generator=g).bfloat16()
+    v_full = torch.randn(B, S_total, H, D, generator=g).bfloat16()
+    qs = split_tensor_uneven(q_full, N, dim=1, tensor_name="q")
+    ks = split_tensor_uneven(k_full, N, dim=1, tensor_name="k")
+    vs = split_tensor_uneven(v_full, N, dim=1, tensor_name="v")
+    pads = get_padding_dict()["k"]
+    n_pad = sum(pads)
+    assert n_pad == N - S_total % N and pads[rank] == 1 and all(k.shape[1] == -(-S_total // N) for k in ks)
+    state = dict(q=qs[rank], ks=ks, vs=vs)
+
+    def attn_fn(r, c):
+        return (c,) if r != rank else om.chunk_attention(state["q"], state["ks"][c], state["vs"][c])
+
+    def merge_fn(a, b):
+        if isinstance(b[0], int):
+            return tuple(b) if a is None else tuple(a) + tuple(b)
+        return om.update_out_and_lse(None if a is None else a[0], None if a is None else a[1], b[0], b[1])
+
+    ring = RingOracle(N, attn_fn=attn_fn, merge_fn=merge_fn,
+                      store_fn=lambda s: s if isinstance(s[0], int) else (om.bf16_round(s[0]), s[1]))
+    group = get_usp_group()
+    attn = proAttention(0, group)
+    dk, dv = [k.cuda() for k in ks], [v.cuda() for v in vs]
+    group.set_kv_chunks(dk, dv)
+    # attention of the local queries over the unpadded sequence (the padded query row attends like a zero query)
+    ex_out, ex_lse = om.chunk_attention(qs[rank], k_full, v_full)
+    for t in range(T):
+        print(f"case padded shards N={N} rank={rank} D={D} t={t} curr={curr[t]}", flush=True)
+        tr = ring.call(t, curr[t], nxt[t])[rank]
+        update_timestep(t)
+        out = attn.attn(qs[rank].cuda(), dk[rank], dv[rank])
+        torch.cuda.synchronize()
+        assert attn.last_plan.computed == tr.computed and attn.last_plan.stores == tr.stores
+        ref_out, ref_lse = tr.out
+        _cmp(out, attn.last_lse, ref_out, ref_lse.squeeze(-1).transpose(1, 2), f"padded t={t}")
+        # inputs do not change between the steps, so every step sees all N chunks: padded keys add exactly n_pad
+        lse = attn.last_lse.cpu().squeeze(-1).transpose(1, 2).double()
+        assert torch.allclose(lse.exp(), ex_lse.double().exp() + n_pad, rtol=2e-3)
+        w = (ex_lse.double().exp() / (ex_lse.double().exp() + n_pad)).transpose(1, 2).unsqueeze(-1)
+        assert (out.cpu().double() - ex_out.double() * w).abs().max() <= OUT_TOL
+    # the padded query row (a zero query: uniform attention over all keys, padded ones included)
+    mean_v = torch.cat(vs, dim=1).float().sum(1) / (N * ks[0].shape[1])
+    assert (out.cpu()[:, -1] - mean_v).abs().max() <= OUT_TOL
 
 
 def test_mask_mode_cold_reuse_is_an_error(env):
@@ -392,6 +532,33 @@ def test_mask_mode_memory_guard_recomputes_without_arena(env):
         _cmp(out, tight.last_lse, ref_out, ref_lse, f"no arena t={t}")
         q, ks, vs = _perturb(q, g), [_perturb(k, g) for k in ks], [_perturb(v, g) for v in vs]
     assert tight.cache.arena_out is None and roomy.cache.arena_out is not None
+
+
+def test_fp16_inputs_are_rounded_to_bf16_once(env):
+    """flash_attn_func takes fp16 as well as bf16; the kernels here read bf16, so fp16 tensors are rounded to bf16
+    at the kernel boundary (3 mantissa bits fewer than an fp16 flash-attn run would carry; parity with that run is
+    unpinned -- the wheel is absent and the reference holds no fp16 vectors).  What is checked: the result is the
+    attention of the ROUNDED inputs to the usual bar, and its distance to fp32 attention of the fp16 inputs stays
+    within the price of that rounding (2^-9 relative per element; the test allows 5e-3 / 5e-3)."""
+    from ditango_amd.core.attention import proAttention
+    from ditango_amd.core.parallel_state import get_usp_group
+    B, H, D, S, N = 1, 2, 128, 200, 2
+    env(N, 0, 1, 1)
+    g = torch.Generator().manual_seed(12)
+    q = torch.randn(B, S, H, D, generator=g).half()
+    ks = [torch.randn(B, S, H, D, generator=g).half() for _ in range(N)]
+    vs = [torch.randn(B, S, H, D, generator=g).half() for _ in range(N)]
+    group = get_usp_group()
+    group.set_kv_chunks([k.cuda() for k in ks], [v.cuda() for v in vs])
+    attn = proAttention(0, group)
+    out = attn.attn(q.cuda(), ks[0].cuda(), vs[0].cuda())
+    torch.cuda.synchronize()
+    assert out.dtype == torch.float32
+    r_out, r_lse = om.full_attention(q.bfloat16(), [k.bfloat16() for k in ks], [v.bfloat16() for v in vs])
+    _cmp(out, attn.last_lse, r_out, r_lse, "fp16 inputs vs attention of their bf16 roundings")
+    f_out, f_lse = om.full_attention(q.float(), [k.float() for k in ks], [v.float() for v in vs])
+    lse = attn.last_lse.cpu().squeeze(-1).transpose(1, 2)
+    assert (out.cpu() - f_out).abs().max() <= 5e-3 and (lse - f_lse).abs().max() <= 5e-3
 
 
 def test_update_out_and_lse_dropin(hip):

@@ -418,13 +418,15 @@ def test_varlen_mask_mode_at_full_size(env, hip):
     layer = 7
     group = get_usp_group()
     attn = proAttention(layer, group)
-    cu_t = torch.tensor(cu, dtype=torch.int32)
+    # int32 boundaries on the GPU and max_seqlen = the sample's length, as the model passes them
+    # (executor/hunyuanvideo/hunyuan_transformer.py:783-792)
+    cu_t = torch.tensor(cu, dtype=torch.int32, device="cuda")
     cached = {}
     for t in range(3):
         update_timestep(t)
         dk, dv = [k.cuda() for k in ks], [v.cuda() for v in vs]
         group.set_kv_chunks([k[0] for k in dk], [v[0] for v in dv], cu_seqlens_kv=[cu_t] * C)
-        out = attn.varlen_attn(q[0].cuda(), dk[diag][0], dv[diag][0], cu_t, cu_t, cu[1], cu[1])
+        out = attn.varlen_attn(q[0].cuda(), dk[diag][0], dv[diag][0], cu_t, cu_t, Sq, Sq)
         torch.cuda.synchronize()
         compute, reuse = ms.build_schedule(mask[t, layer], diag)
         n = int(rm.sched_counts_host[t, layer, 0])

@@ -35,6 +35,50 @@ def test_library_exports_every_declared_symbol():
     assert isinstance(lib.dt_last_error(), bytes)
 
 
+def test_dynamic_symbol_table_holds_the_c_abi_and_nothing_else():
+    """``nm -D``: the defined dynamic symbols of the drop-in library are exactly the header's functions (no C++
+    internals, no kernel stubs, no measurement aids), and those of the probes library exactly ditango_probes.h's."""
+    import shutil
+    import subprocess
+    from ditango_amd import _hip
+    if shutil.which("nm") is None:
+        pytest.skip("no nm")
+    if not _hip.LIB_PATH.exists():
+        from ditango_amd.build import build_lib
+        build_lib()
+
+    def defined(path):
+        out = subprocess.run(["nm", "-D", "--defined-only", str(path)], capture_output=True, text=True, check=True).stdout
+        return sorted(line.split()[-1] for line in out.splitlines() if line.split()[-2] in ("T", "t", "D", "B", "W"))
+
+    assert defined(_hip.LIB_PATH) == _declared()
+    assert not any("probe" in n for n in _declared())
+    import bench_probes
+    text = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", "ditango_probes.h")).read(), flags=re.S)
+    probe_names = sorted(set(re.findall(r"\b(dtp_[a-z0-9_]+)\s*\(", text)))
+    assert defined(bench_probes.PROBES_PATH) == probe_names == sorted(bench_probes.EXPORTED_SYMBOLS)
+    lib = bench_probes.load_library()
+    assert lib.dtp_mfma_probe(0, 4, None, None) == -1 and b"mfma probe" in lib.dtp_last_error()     # refused on the host
+
+
+def test_every_entry_point_names_what_it_replaces():
+    """Each declaration's comment cites the reference call site it stands in for (file.py:line) or says that
+    the reference has no counterpart."""
+    text = open(os.path.join(ROOT, "include", "ditango_hip.h")).read()
+    body = text[text.index("int dt_version"):]
+    blocks = re.findall(r"/\*(.*?)\*/(.*?)(?=/\*|#ifdef __cplusplus)", body, flags=re.S)
+    seen = set()
+    for comment, decls in blocks:
+        names = re.findall(r"\b(dt_[a-z0-9_]+)\s*\(", decls)
+        if not names:
+            continue
+        cites = re.search(r"[a-z_/]+\.py:\d+", comment) or "No counterpart in the reference" in comment \
+            or "no counterpart in the reference" in comment
+        assert cites, f"{names}: the comment names neither a reference call site nor the absence of one"
+        seen.update(names)
+    assert seen | {"dt_version", "dt_last_error"} == set(_declared())
+
+
 def test_missing_library_fails_loudly(tmp_path):
     from ditango_amd import _hip
     with pytest.raises(_hip.DitangoHipError):

@@ -65,6 +65,51 @@ def test_sched_attention_and_merge_replay_in_a_graph(hip):
     assert np.array_equal(comp.cpu().numpy(), ms.build_schedule_table(mask, diag)[0])
 
 
+def test_varlen_launch_with_device_boundaries_replays_in_a_graph(hip):
+    """The variable-length launch with its cu_seqlens in device memory, captured once and replayed while the
+    BOUNDARIES (and K/V) change on the device: every replay equals the eager launch on the same boundaries,
+    which a launch that had read them on the host at capture time could not do."""
+    B, H, D, total, lens = 1, 4, 128, 700, [500, 420]
+    dev = "cuda"
+    g = torch.Generator(device=dev).manual_seed(8)
+    q = torch.randn(B, total, H, D, generator=g, device=dev).bfloat16()
+    ks = [torch.randn(B, n, H, D, generator=g, device=dev).bfloat16() for n in lens]
+    vs = [torch.randn(B, n, H, D, generator=g, device=dev).bfloat16() for n in lens]
+    table = hip.ChunkTable(ks, vs)
+    cu_q = torch.tensor([0, 600, 700], dtype=torch.int32, device=dev)
+    cu_k = [torch.tensor([0, 400, 500], dtype=torch.int32, device=dev), torch.tensor([0, 300, 420], dtype=torch.int32, device=dev)]
+    seg = hip.DeviceSegments(cu_q, cu_k, total)
+    jobs, job_segs = [[0, 1], [0, 1]], [0, 1]
+
+    def buffers():
+        return dict(o=torch.zeros(B, total, H, D, dtype=torch.bfloat16, device=dev), l=torch.zeros(B, H, total, device=dev))
+
+    def call(b):
+        hip.attn_jobs_fwd(q, table, jobs, [b["o"]] * 2, [b["l"]] * 2, dev_segments=seg, job_segments=job_segs)
+
+    eager, graphed = buffers(), buffers()
+    call(graphed)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(graphed)
+    splits = [(600, 400, 300), (512, 100, 420), (64, 500, 0), (700, 250, 250), (333, 1, 419)]
+    seen = []
+    for step, (sq, s0, s1) in enumerate(splits):
+        cu_q.copy_(torch.tensor([0, sq, total], dtype=torch.int32))
+        cu_k[0].copy_(torch.tensor([0, s0, lens[0]], dtype=torch.int32))
+        cu_k[1].copy_(torch.tensor([0, s1, lens[1]], dtype=torch.int32))
+        for k in ks + vs:
+            k.add_(0.01 * torch.randn_like(k))
+        call(eager)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(graphed["o"], eager["o"]) and torch.equal(graphed["l"], eager["l"]), f"replay {step}"
+        seen.append(graphed["o"].clone())
+    assert not torch.equal(seen[0], seen[1])
+
+
 def test_noalloc_attention_replays_in_a_graph(hip):
     """The allocation-free entry point under capture: the attention launch (with its tail split inside the
     library's own scratch array and the fold kernel behind it) plus the merge, replayed four times

@@ -267,19 +267,6 @@ def test_tail_balancing_random_launches_match_plain(hip, seed):
         assert (res[0][1][j] - res[1][1][j]).abs().max() <= 1e-5
 
 
-def test_read_probe_and_its_argument_checks(hip):
-    """The bandwidth yardstick reads its streams and writes nothing; bad arguments are refused without a launch."""
-    bufs = [torch.full((1000, 64), 3, dtype=torch.int32, device="cuda") for _ in range(11)]    # 256 000 bytes each
-    sink = torch.zeros(1, dtype=torch.int32, device="cuda")
-    hip.hbm_read_probe(bufs, sink)
-    torch.cuda.synchronize()
-    assert int(sink.item()) == 0 and all(int(b.sum().item()) == 3 * 64000 for b in bufs)
-    with pytest.raises(hip.DitangoHipError):
-        hip.hbm_read_probe(bufs + [bufs[0][:500]], sink)
-    with pytest.raises(hip.DitangoHipError):
-        hip.hbm_read_probe(bufs * 6, sink)                     # 66 streams: more than one launch takes
-
-
 def test_attention_workspace_is_per_stream(hip):
     """Launches on different streams must not share the tail-balancing workspace (they would race on it)."""
     a = hip.attn_workspace("cuda")
@@ -290,28 +277,19 @@ def test_attention_workspace_is_per_stream(hip):
         assert hip.attn_workspace("cuda").data_ptr() == b.data_ptr()
     assert a.data_ptr() != b.data_ptr() and a.numel() == b.numel()
     assert hip.attn_workspace("cuda").data_ptr() == a.data_ptr()
-
-
-def test_mfma_probe_runs_and_checks_its_arguments(hip):
-    sink = torch.zeros(1, dtype=torch.float32, device="cuda")
-    flop = hip.mfma_probe(64, 16, sink)
-    torch.cuda.synchronize()
-    assert flop == 64 * 8 * 4 * 16 * 32768.0 and float(sink) == 0.0
-    for bad in ((0, 16), (64, 0), (-1, 4), (64, 6)):
-        with pytest.raises(hip.DitangoHipError):
-            hip.mfma_probe(*bad, sink)
-
-
-def test_coissue_probe_runs_and_checks_its_arguments(hip):
-    sink = torch.zeros(1, dtype=torch.float32, device="cuda")
-    for D in (64, 128):
-        for with_softmax in (False, True):
-            flop = hip.coissue_probe(64, 16, D, with_softmax, sink)
-            torch.cuda.synchronize()
-            assert flop == 64 * 4 * 4 * 16 * 32768.0 and float(sink) == 0.0
-    for bad in ((0, 16, 128), (64, 0, 128), (64, 6, 64), (64, 16, 96)):
-        with pytest.raises(hip.DitangoHipError):
-            hip.coissue_probe(*bad, True, sink)
+    # the table is bounded: streams beyond MAX_WORKSPACES push the least recently used entry out
+    streams = [torch.cuda.Stream() for _ in range(hip.MAX_WORKSPACES + 2)]
+    for st in streams:
+        with torch.cuda.stream(st):
+            hip.attn_workspace("cuda")
+            hip.attn_workspace("cuda")          # a repeated request must not grow the table
+        assert len(hip._workspaces) <= hip.MAX_WORKSPACES
+    assert len(hip._workspaces) == hip.MAX_WORKSPACES
+    with torch.cuda.stream(streams[-1]):
+        last = hip.attn_workspace("cuda")
+    assert hip.attn_workspace("cuda").data_ptr() != last.data_ptr()     # the default stream's entry was re-created
+    hip.release_workspaces()
+    assert len(hip._workspaces) == 0
 
 
 def test_cache_load_into_given_tensors(hip):

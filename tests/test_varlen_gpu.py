@@ -58,6 +58,93 @@ def test_segment_jobs_match_varlen_oracle(hip, D, cu_q, cu_k):
     assert (got[finite] - ref[finite]).abs().max() <= LSE_TOL
 
 
+@pytest.mark.parametrize("D,cu_q,cu_k", [
+    (128, [0, 300], [0, 333]),
+    (128, [0, 257, 300], [0, 300, 333]),
+    (64, [0, 100, 100, 290], [0, 64, 200, 333]),      # an empty query segment; rows 290.. in no segment
+    (128, [0, 10, 280], [0, 0, 333]),                 # a segment without keys
+    (64, [0, 40, 80, 120, 160, 200, 240, 250, 260, 270, 300], [0, 30, 60, 90, 120, 150, 180, 210, 240, 270, 333]),  # 10 segments
+])
+def test_segment_jobs_with_device_boundaries_equal_host_boundaries(hip, D, cu_q, cu_k):
+    """dt_attn_varlen_jobs_fwd (cu_seqlens read by the kernel from device memory, flash_attn_varlen_func's calling
+    convention) against dt_attn_seg_jobs_fwd (the same boundaries as host ranges): bit-identical states, and both
+    within tolerance of the varlen oracle."""
+    H = 3
+    g = torch.Generator().manual_seed(len(cu_q) + D)
+    q = torch.randn(300, H, D, generator=g).bfloat16()
+    k = torch.randn(333, H, D, generator=g).bfloat16()
+    v = torch.randn(333, H, D, generator=g).bfloat16()
+    ref_out, ref_lse = om.varlen_chunk_attention(q, k, v, cu_q, cu_k)
+    dq, dk, dv = q.cuda()[None], k.cuda()[None], v.cuda()[None]
+    table = hip.ChunkTable([dk], [dv])
+    nseg = len(cu_q) - 1
+    res = []
+    for on_device in (False, True):
+        out = torch.zeros(1, 300, H, D, dtype=torch.bfloat16, device="cuda")
+        lse = torch.full((1, H, 300), float("-inf"), device="cuda")
+        if on_device:
+            seg = hip.DeviceSegments(torch.tensor(cu_q, dtype=torch.int32, device="cuda"),
+                                     [torch.tensor(cu_k, dtype=torch.int32, device="cuda")], max(b - a for a, b in zip(cu_q, cu_q[1:])))
+            hip.attn_jobs_fwd(dq, table, [[0]] * nseg, [out] * nseg, [lse] * nseg, dev_segments=seg, job_segments=list(range(nseg)))
+        else:
+            hip.attn_jobs_fwd(dq, table, [[0]] * nseg, [out] * nseg, [lse] * nseg,
+                              q_ranges=[(cu_q[i], cu_q[i + 1] - cu_q[i]) for i in range(nseg)],
+                              kv_ranges=[[(cu_k[i], cu_k[i + 1] - cu_k[i])] for i in range(nseg)])
+        torch.cuda.synchronize()
+        res.append((out, lse))
+    assert torch.equal(res[0][0], res[1][0]) and torch.equal(res[0][1], res[1][1])
+    out, lse = res[1]
+    assert (out[0].float().cpu() - ref_out).abs().max() <= OUT_TOL
+    got, finite = lse[0].cpu(), torch.isfinite(ref_lse)
+    assert torch.equal(torch.isfinite(got), finite) and (got[finite] - ref_lse[finite]).abs().max() <= LSE_TOL
+
+
+def test_device_boundaries_are_clamped_and_checked(hip):
+    """Nothing on the host reads device-resident boundaries, so the kernel clamps them to the rows and keys that
+    exist: a list that overshoots both ends yields the full-range result, never a stray access.  What the host can
+    check (dtype, placement, segment index, max_seqlen_q) is refused before any launch."""
+    H, D = 2, 64
+    g = torch.Generator().manual_seed(77)
+    q = torch.randn(1, 200, H, D, generator=g).bfloat16().cuda()
+    k = torch.randn(1, 150, H, D, generator=g).bfloat16().cuda()
+    v = torch.randn(1, 150, H, D, generator=g).bfloat16().cuda()
+    table = hip.ChunkTable([k], [v])
+    full_o, full_l = hip.attn_chunk_fwd(q, k, v)
+    out = torch.zeros_like(full_o)
+    lse = torch.zeros_like(full_l)
+    seg = hip.DeviceSegments(torch.tensor([-7, 100000], dtype=torch.int32, device="cuda"),
+                             [torch.tensor([-3, 2 ** 30], dtype=torch.int32, device="cuda")], 200)
+    hip.attn_jobs_fwd(q, table, [[0]], [out], [lse], dev_segments=seg, job_segments=[0])
+    torch.cuda.synchronize()
+    assert torch.equal(out, full_o) and torch.equal(lse, full_l)
+    # decreasing boundaries: an empty segment (nothing written), no fault
+    out.zero_()
+    seg = hip.DeviceSegments(torch.tensor([150, 20], dtype=torch.int32, device="cuda"),
+                             [torch.tensor([0, 150], dtype=torch.int32, device="cuda")], 200)
+    hip.attn_jobs_fwd(q, table, [[0]], [out], [lse], dev_segments=seg, job_segments=[0])
+    torch.cuda.synchronize()
+    assert int(torch.count_nonzero(out)) == 0
+    with pytest.raises(hip.DitangoHipError):
+        hip.DeviceSegments(torch.tensor([0, 200], dtype=torch.int32), [torch.tensor([0, 150], dtype=torch.int32, device="cuda")], 200)
+    with pytest.raises(hip.DitangoHipError):
+        hip.DeviceSegments(torch.tensor([0, 200], dtype=torch.int64, device="cuda"), [None], 200)
+    ok = hip.DeviceSegments(torch.tensor([0, 200], dtype=torch.int32, device="cuda"),
+                            [torch.tensor([0, 150], dtype=torch.int32, device="cuda")], 200)
+    with pytest.raises(hip.DitangoHipError):
+        hip.attn_jobs_fwd(q, table, [[0]], [out], [lse], dev_segments=ok, job_segments=[1])      # segment index out of range
+    with pytest.raises(hip.DitangoHipError):
+        hip.DeviceSegments(ok.cu_q, ok.cu_kv, 0)
+
+
+def test_zero_rows_from_a_device_index(hip):
+    for first, n in ((0, 37), (20, 37), (37, 37), (-4, 10), (99, 10)):
+        t = torch.ones(n, 3, 8, dtype=torch.float32, device="cuda")
+        hip.zero_rows_from(t, torch.tensor([first], dtype=torch.int32, device="cuda"))
+        torch.cuda.synchronize()
+        lo = min(max(first, 0), n)
+        assert bool((t[:lo] == 1).all()) and bool((t[lo:] == 0).all()), (first, n)
+
+
 def test_single_segment_reduces_to_the_dense_path(env, hip):
     from ditango_amd.core.attention import proAttention
     from ditango_amd.core.parallel_state import get_usp_group
@@ -80,9 +167,32 @@ def test_single_segment_reduces_to_the_dense_path(env, hip):
     assert torch.equal(c, b)
 
 
-def test_varlen_stride_mode_matches_numeric_oracle(env, hip):
+def _cu(values, on_device):
+    """cu_seqlens as the callers make them: int32, on the GPU (hunyuan_transformer.py:789-792) or on the host."""
+    return torch.tensor(values, dtype=torch.int32, device="cuda" if on_device else "cpu")
+
+
+class _no_host_sync:
+    """Inside: any torch operation that blocks the host on the GPU raises (reading a device tensor's values,
+    a pageable copy...).  The calling convention with device-resident boundaries promises there is none."""
+
+    def __init__(self, on):
+        self.on = on
+
+    def __enter__(self):
+        if self.on:
+            torch.cuda.set_sync_debug_mode("error")
+
+    def __exit__(self, *exc):
+        torch.cuda.set_sync_debug_mode("default")
+        return False
+
+
+@pytest.mark.parametrize("cu_on_device", [False, True])
+def test_varlen_stride_mode_matches_numeric_oracle(env, hip, cu_on_device):
     """Two segments per sample (valid tokens | padding), different boundaries in every chunk,
-    over a divider sequence with reuse, coarsening and a full refresh."""
+    over a divider sequence with reuse, coarsening and a full refresh.  With the boundaries on the GPU
+    (the reference's calling convention) the call must not synchronise with the device."""
     from ditango_amd.core.attention import proAttention
     from ditango_amd.core.parallel_state import get_usp_group
     from ditango_amd.utils import update_timestep
@@ -126,9 +236,11 @@ def test_varlen_stride_mode_matches_numeric_oracle(env, hip):
         tr = ring.call(t, curr[t], nxt[t])[rank]
         update_timestep(t)
         dk, dv = [k.cuda() for k in kb], [v.cuda() for v in vb]
-        group.set_kv_chunks(dk, dv, cu_seqlens_kv=[torch.tensor(c, dtype=torch.int32) for c in cu_k])
-        out = attn.varlen_attn(qb.cuda(), dk[rank], dv[rank], torch.tensor(cu_q, dtype=torch.int32),
-                               torch.tensor(cu_k[rank], dtype=torch.int32), max(150, 30), max(lens))
+        dq, d_cu_q, d_cu_k = qb.cuda(), _cu(cu_q, cu_on_device), [_cu(c, cu_on_device) for c in cu_k]
+        group.set_kv_chunks(dk, dv, cu_seqlens_kv=d_cu_k)
+        torch.cuda.synchronize()
+        with _no_host_sync(cu_on_device and t > 0):     # (the first call sets kernel attributes and allocates the workspace)
+            out = attn.varlen_attn(dq, dk[rank], dv[rank], d_cu_q, d_cu_k[rank], max(150, 30), max(lens))
         torch.cuda.synchronize()
         assert attn.last_plan.computed == tr.computed and attn.last_plan.stores == tr.stores
         ref_out, ref_lse = tr.out
@@ -141,9 +253,11 @@ def test_varlen_stride_mode_matches_numeric_oracle(env, hip):
         vs = [v + 0.01 * torch.randn(v.shape, generator=g) for v in vs]
 
 
-def test_varlen_mask_mode_matches_numeric_oracle(env, hip):
+@pytest.mark.parametrize("cu_on_device", [False, True])
+def test_varlen_mask_mode_matches_numeric_oracle(env, hip, cu_on_device):
     """The packed entry under a per-chunk reuse mask: every scheduled chunk runs once per segment
-    (dt_attn_sched_seg_fwd) into its cache slot; a trailing pad region belongs to no segment."""
+    (dt_attn_sched_seg_fwd, or dt_attn_sched_varlen_fwd when the boundaries are device tensors) into its
+    cache slot; a trailing pad region belongs to no segment."""
     import numpy as np
     from oracle import mask_schedule as ms
     from ditango_amd.core.attention import proAttention
@@ -173,9 +287,11 @@ def test_varlen_mask_mode_matches_numeric_oracle(env, hip):
         print(f"case varlen mask t={t} computes {c_ids} reuses {r_ids}", flush=True)
         update_timestep(t)
         dk, dv = [k.cuda() for k in kb], [v.cuda() for v in vb]
-        group.set_kv_chunks(dk, dv, cu_seqlens_kv=[torch.tensor(c, dtype=torch.int32) for c in cu_k])
-        out = attn.varlen_attn(qb.cuda(), dk[diag], dv[diag], torch.tensor(cu_q, dtype=torch.int32),
-                               torch.tensor(cu_k[diag], dtype=torch.int32), 260, 300)
+        dq, d_cu_q, d_cu_k = qb.cuda(), _cu(cu_q, cu_on_device), [_cu(c, cu_on_device) for c in cu_k]
+        group.set_kv_chunks(dk, dv, cu_seqlens_kv=d_cu_k)
+        torch.cuda.synchronize()
+        with _no_host_sync(cu_on_device and t > 0):
+            out = attn.varlen_attn(dq, dk[diag], dv[diag], d_cu_q, d_cu_k[diag], 260, 300)
         torch.cuda.synchronize()
         n = int(rm.sched_counts_host[t, 0, 0])
         assert rm.sched_compute_ids[t, 0, :n].tolist() == list(c_ids)
