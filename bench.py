@@ -202,18 +202,18 @@ def cpu_baseline(B, H, D, Sq, lens, mean_computed, n_chunks, norm, budget_s=20.0
     }
 
 
-def bench_stride_schedule(args):
-    """One full pass of the reference's stride schedule: 50 steps x ``--layers`` layers (default 12) of
-    ``proAttention.attn`` at the HunyuanVideo per-rank shape as ring rank 0 of 8, with the divider map
-    generated from the redundancy map the reference ships for HunyuanVideo (percentiles [0,40,90],
-    dividers [8,4,2,1], configs/hunyuanvideo/config.yaml).  Every call is timed, the full-stride
-    steps included."""
+def stride_schedule_record(n_layers):
+    """One full pass of the reference's own schedule (core/attention.py:100-216, core/cache.py:28-72): 50 steps x
+    ``n_layers`` layers of ``proAttention.attn`` at the HunyuanVideo per-rank shape as ring rank 0 of 8, with the
+    divider map generated from the redundancy map the reference ships for HunyuanVideo (percentiles [0,40,90],
+    dividers [8,4,2,1], configs/hunyuanvideo/config.yaml).  Every call is timed, the full-stride steps included.
+    The in-place cache coarsening (``proCache._merge_blocks``) is bracketed by events of its own."""
     from ditango_amd.core import config, parallel_state, redundancy_map as rmod
     from ditango_amd.core.attention import proAttention
     from ditango_amd.utils import update_timestep
     label, B, H, D, Sq, lens, T, L, _, _, norm = WORKLOADS["hunyuanvideo"]
     N, rank = len(lens), 0
-    L_run = min(L, args.layers or 12)
+    L_run = min(L, n_layers)
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     parallel_state.init_local_groups(N, rank)
@@ -225,26 +225,66 @@ def bench_stride_schedule(args):
     group = parallel_state.get_usp_group()
     group.set_kv_chunks(ks, vs)
     layers = [proAttention(l, group) for l in range(L_run)]
-    computed = 0
+    coarsen_events = []
+
+    def bracketed(merge_blocks):
+        def run(new_block_num):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            merge_blocks(new_block_num)
+            e1.record()
+            coarsen_events.append((e0, e1))
+        return run
+
+    for layer in layers:
+        layer.cache._merge_blocks = bracketed(layer.cache._merge_blocks)
+    computed = reused = double_counted = 0
+    strides = {}
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for t in range(T):
         update_timestep(t)
         for l in range(L_run):
             layers[l].attn(q, ks[rank], vs[rank])
-            computed += len(layers[l].last_plan.computed)
+            plan = layers[l].last_plan
+            computed += len(plan.computed)
+            reused += len(plan.reuse_merged)
+            double_counted += len(plan.computed) - len({c for c, _ in plan.computed})
+            strides[plan.curr_stride] = strides.get(plan.curr_stride, 0) + 1
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    coarsen_ms = sum(e0.elapsed_time(e1) for e0, e1 in coarsen_events)
     calls = T * L_run
     flops = 4.0 * B * H * Sq * lens[0] * D * computed
-    print(json.dumps({
-        "metric": "ms/layer", "value": round(1e3 * elapsed / calls, 4), "unit": "ms", "n_gpus": 1, "steps": calls, "warmup": 0,
-        "ms_per_step": round(1e3 * elapsed / calls, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": label + ", stride schedule of the shipped redundancy map, ring rank 0 of 8", "B": B, "H": H,
-                   "D": D, "Sq": Sq, "kv_chunks": N, "Sk": lens[0], "layers_instantiated": L_run, "steps_per_layer": T,
-                   "mean_chunks_computed_per_call": round(computed / calls, 3)},
+    rmod.destroy_redundancy_map()
+    parallel_state.destroy_local_groups()
+    update_timestep(0)
+    for layer in layers:
+        layer.cache.release()
+    del layers, q, ks, vs
+    torch.cuda.empty_cache()
+    return {
+        "config": {"workload": label + ", stride schedule of the shipped redundancy map (refined dividers), ring rank 0 of 8",
+                   "B": B, "H": H, "D": D, "Sq": Sq, "kv_chunks": N, "Sk": lens[0], "layers_instantiated": L_run,
+                   "steps_per_layer": T, "calls_by_stride": {str(k): v for k, v in sorted(strides.items())}},
+        "ms_per_layer": round(1e3 * elapsed / calls, 4), "calls": calls,
+        "mean_chunks_computed_per_call": round(computed / calls, 3),
+        "mean_cached_blocks_merged_per_call": round(reused / calls, 3),
+        "calls_with_the_local_chunk_merged_twice": double_counted,
         "layer_attn_tflops": round(flops / elapsed / 1e12, 1),
+        "coarsening": {"what": "in-place merges of proCache._merge_blocks, device time between events",
+                       "launch_groups": len(coarsen_events), "ms_total": round(coarsen_ms, 3),
+                       "share_of_run": round(coarsen_ms / (1e3 * elapsed), 5)},
+    }
+
+
+def bench_stride_schedule(args):
+    """``--schedule stride``: the stride-schedule pass as a report of its own (default 12 layers)."""
+    rec = stride_schedule_record(args.layers or 12)
+    print(json.dumps({
+        "metric": "ms/layer", "value": rec["ms_per_layer"], "unit": "ms", "n_gpus": 1, "steps": rec["calls"], "warmup": 0,
+        "ms_per_step": rec["ms_per_layer"], "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic", **{k: v for k, v in rec.items() if k not in ("ms_per_layer", "calls")},
     }), flush=True)
 
 
@@ -633,6 +673,8 @@ def main():
             rec = run_workload(name, args, steps, 4 if name != "sweep" else 2, main=False, reuse=reuse)
             rec.pop("_mean_computed")
             others[name if name != "sweep" else f"sweep_reuse_{reuse}"] = rec
+        # the reference's own mode: the stride schedule of the redundancy map it ships, every call timed
+        others["stride_schedule"] = stride_schedule_record(args.layers or 6)
         result["other_configs"] = others
     if not args.no_cpu_baseline and not args.kernels_only:
         label, B, H, D, Sq, lens, T, L, p, diag, norm = WORKLOADS[args.workload]

@@ -9,7 +9,9 @@ switched off for all device code (``-target-feature -packed-fp32-ops``).
 """
 from __future__ import annotations
 
+import json
 import os
+import re
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -22,6 +24,7 @@ LIB_DIR = PKG / "lib"
 LIB_PATH = LIB_DIR / "libditango_hip.so"
 PROBES_PATH = LIB_DIR / "libditango_probes.so"
 DEMO_PATH = LIB_DIR / "dt_capi_demo"
+RESOURCES_PATH = LIB_DIR / "kernel_resources.json"   # per-kernel registers / scratch / occupancy of the last build
 SOURCES = ["attn_fwd.hip", "attn_f32.hip", "state_ops.hip", "producer.hip", "capi.hip"]
 PROBE_SOURCES = ["probes.hip"]
 
@@ -41,17 +44,35 @@ def _run(cmd):
     return res
 
 
+def parse_resource_remarks(text: str) -> dict:
+    """``{kernel symbol: {"VGPRs": n, "ScratchSize [bytes/lane]": n, ...}}`` from the compiler's
+    ``-Rpass-analysis=kernel-resource-usage`` remarks."""
+    out, cur = {}, None
+    for line in text.splitlines():
+        m = re.search(r"remark:\s+Function Name: (\S+)", line)
+        if m:
+            cur = out.setdefault(m.group(1), {})
+            continue
+        m = re.search(r"remark:\s+([A-Za-z][^:]*): (-?\d+)", line)
+        if m and cur is not None:
+            cur[m.group(1).strip()] = int(m.group(2))
+    return out
+
+
 def build_lib(verbose: bool = False, extra_flags=()) -> Path:
     """Compile and link the library unconditionally; returns its path."""
     LIB_DIR.mkdir(exist_ok=True)
     objs = []
 
+    resources = {}
+
     def compile_one(src):
         obj = LIB_DIR / (Path(src).stem + ".o")
-        cmd = [HIPCC, *COMMON, *extra_flags, "-c", str(CSRC / src), "-o", str(obj)]
+        # the resource remarks (registers, scratch, occupancy per kernel) come with the compilation at no cost
+        cmd = [HIPCC, *COMMON, *extra_flags, "-Rpass-analysis=kernel-resource-usage", "-c", str(CSRC / src), "-o", str(obj)]
         if verbose:
             print(" ".join(cmd), flush=True)
-        _run(cmd)
+        resources[src] = parse_resource_remarks(_run(cmd).stderr)
         return obj
 
     with ThreadPoolExecutor(max_workers=6) as ex:
@@ -64,6 +85,7 @@ def build_lib(verbose: bool = False, extra_flags=()) -> Path:
         if verbose:
             print(" ".join(cmd), flush=True)
         _run(cmd)
+    RESOURCES_PATH.write_text(json.dumps(resources, indent=1, sort_keys=True) + "\n")
     # a host program that uses nothing but the C header and the HIP runtime (tests/test_capi_demo_gpu.py runs it)
     cmd = [HIPCC, "-O2", "-std=c++17", "-Wno-unused-result", f"-I{ROOT / 'include'}", str(CSRC / "capi_demo.cpp"),
            f"-L{LIB_DIR}", "-lditango_hip", "-Wl,-rpath,$ORIGIN", "-o", str(DEMO_PATH)]

@@ -219,8 +219,16 @@ __device__ __forceinline__ void load_block_to_lds(u32x4 rsrc, uint32_t lane_off,
 #define DT_D64_WAVES 4
 #endif
 template <int D, bool kPre>
-__global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd_kernel(const AttnArgs args_by_value) {
   using T = Tile<D>;
+  // The arguments are read where they arrive: in the kernarg segment (constant address space, scalar loads),
+  // through its base pointer -- AttnArgs is the kernel's only parameter, so it sits at offset 0.  Going through the
+  // by-value parameter instead leaves it to the optimiser to prove that its private copy of the 3.6 KB struct is
+  // never needed; with the tables indexed at run time from several branches it sometimes cannot, and every lane
+  // then copies the whole struct into scratch memory before it starts (seven times the run time of a short launch).
+  typedef const AttnArgs __attribute__((address_space(4))) KernArgs;
+  KernArgs& a = *(KernArgs*)__builtin_amdgcn_kernarg_segment_ptr();
+  (void)args_by_value;
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
   // ---- which (job, batch, head, query tile) ------------------------------------------
@@ -299,9 +307,9 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
     q_end = min(max(__builtin_amdgcn_readfirstlane(a.cu_q[dseg + 1]), q_begin), a.Sq);
   }
   if (qt * kBQ >= q_end - q_begin) return;  // the grid is sized for the longest job / segment
-  auto chunk_of = [&](int seg) -> int { return single >= 0 ? single : a.job_chunks[seg]; };
+  auto chunk_of = [&](int seg) __attribute__((always_inline)) -> int { return single >= 0 ? single : a.job_chunks[seg]; };
   // keys [begin, begin + len) of chunk reference `seg`
-  auto kv_begin_of = [&](int seg) -> int {
+  auto kv_begin_of = [&](int seg) __attribute__((always_inline)) -> int {
     if (dseg >= 0) {
       const int cid = chunk_of(seg);
       return min(max(__builtin_amdgcn_readfirstlane(a.cu_kv[cid][dseg]), 0), a.kv_len[cid]);
@@ -309,7 +317,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
     if (single < 0) return a.entry_kv_begin[seg];
     return vseg >= 0 ? a.entry_kv_begin[single * a.n_seg + vseg] : 0;
   };
-  auto kv_len_of = [&](int seg) -> int {
+  auto kv_len_of = [&](int seg) __attribute__((always_inline)) -> int {
     if (dseg >= 0) {
       const int cid = chunk_of(seg);
       const int lo = min(max(__builtin_amdgcn_readfirstlane(a.cu_kv[cid][dseg]), 0), a.kv_len[cid]);
@@ -378,7 +386,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
       rv = rk;
     }
   };
-  auto cp_next_chunk = [&]() {
+  auto cp_next_chunk = [&]() __attribute__((always_inline)) {
     do { ++cp_seg; } while (cp_seg < seg_end && kv_len_of(cp_seg) == 0);
     if (cp_seg < seg_end) cp_left = kv_len_of(cp_seg);
   };
