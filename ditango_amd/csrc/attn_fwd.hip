@@ -50,6 +50,7 @@
 #include <mutex>
 #include <type_traits>
 
+#include "attn_schedule.h"
 #include "dt_common.h"
 
 namespace dt {
@@ -66,7 +67,8 @@ constexpr int kThreads = kWaves * 64;
 constexpr int kBQ = kWaves * 32;  // queries per workgroup
 constexpr int kBK = 64;           // keys per tile
 constexpr int kXcds = 8;
-constexpr int kNumBuf = 4;        // LDS buffers per operand; a tile uses buffer (tile & 3)
+constexpr int kNumBuf = DT_SCHED_NUM_BUF;  // LDS buffers per operand; a tile uses buffer (tile & 3)
+static_assert(kNumBuf == 4, "buffer indices are computed with & 3 and the loop is unrolled by four");
 #ifndef DT_RING
 #define DT_RING 4
 #endif
@@ -84,6 +86,22 @@ __device__ __forceinline__ void phase_barrier() {
   __builtin_amdgcn_sched_barrier(0);
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
   __builtin_amdgcn_sched_barrier(0);
+}
+// Waits until at most N of this wavefront's tile loads are still in flight.  N comes from attn_schedule.h.
+template <int N>
+__device__ __forceinline__ void wait_tile_loads() {
+#define DT_WAIT_VMCNT(K) asm volatile("s_waitcnt vmcnt(" #K ")" ::: "memory")
+  if constexpr (N == 0) DT_WAIT_VMCNT(0);
+  else if constexpr (N == 3) DT_WAIT_VMCNT(3);
+  else if constexpr (N == 4) DT_WAIT_VMCNT(4);
+  else if constexpr (N == 5) DT_WAIT_VMCNT(5);
+  else if constexpr (N == 6) DT_WAIT_VMCNT(6);
+  else if constexpr (N == 8) DT_WAIT_VMCNT(8);
+  else {
+    static_assert(N == 10, "add the immediate for this wait count");
+    DT_WAIT_VMCNT(10);
+  }
+#undef DT_WAIT_VMCNT
 }
 // The same barrier with the results of the finished phase routed through it as in/out
 // operands.  Register-only code may otherwise migrate across an asm statement; tied to it,
@@ -539,7 +557,13 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
   // MFMAs of its matrix phase (one phase later, and then awaited one call earlier).  At D = 64
   // the vector phase is the longer one (half the MFMAs per softmax element) and the matrix
   // phase has the room (measured +16 %); at D = 128 it is the other way round (+1.5 %).
-  constexpr bool kLoadAfterMatrix = D == 64;
+  constexpr bool kLoadAfterMatrix = (D == 64 ? DT_SCHED_LOAD_AFTER_MATRIX_D64 : DT_SCHED_LOAD_AFTER_MATRIX_D128) != 0;
+  static_assert(T::kLoads == (D == 64 ? DT_SCHED_LOADS_D64 : DT_SCHED_LOADS_D128),
+                "attn_schedule.h states how many load instructions a wavefront issues per tile and operand");
+  // shares of tile loads that may stay in flight across the barrier that ends a vector phase
+  constexpr int kVectorInFlight = D == 64 ? DT_SCHED_VECTOR_BARRIER_INFLIGHT_D64 : DT_SCHED_VECTOR_BARRIER_INFLIGHT_D128;
+  static_assert(DT_SCHED_PROLOGUE_CALLS_LEADING == DT_SCHED_CALL_AHEAD && DT_SCHED_PROLOGUE_CALLS_TRAILING == DT_SCHED_CALL_AHEAD + 1,
+                "the prologue issues exactly the calls the loop's first phase pair assumes: tiles 0 .. 2 + group");
   // The operand ring lives across the barrier in front of a matrix phase: its first kRing
   // fragments (V fragments of a tile completed at least a phase ago) are read at the END of the
   // preceding vector phase, so their LDS latency passes while the wavefront waits at the barrier
@@ -627,18 +651,15 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
   using U1 = std::integral_constant<int, 1>;
   using U2 = std::integral_constant<int, 2>;
   using U3 = std::integral_constant<int, 3>;
-  load_tile(0);
-  load_tile(1);
-  load_tile(2);
-  if (group == 1) load_tile(3);
-  // in flight behind this wait: K of tile 1 and the calls after it (kLoads + 2 kLoads (1 + g) loads)
-  if (group == 0) {
-    if constexpr (T::kLoads == 2) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
-  } else {
-    if constexpr (T::kLoads == 2) asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+#pragma unroll
+  for (int y = 0; y < DT_SCHED_PROLOGUE_CALLS_LEADING; ++y) load_tile(y);
+  if (group == 1) {
+#pragma unroll
+    for (int y = DT_SCHED_PROLOGUE_CALLS_LEADING; y < DT_SCHED_PROLOGUE_CALLS_TRAILING; ++y) load_tile(y);
   }
+  // in flight behind this wait: K of tile 1 and the calls after it (kLoads + 2 kLoads (1 + g) loads)
+  if (group == 0) wait_tile_loads<DT_SCHED_PROLOGUE_INFLIGHT_LEADING * T::kLoads>();
+  else wait_tile_loads<DT_SCHED_PROLOGUE_INFLIGHT_TRAILING * T::kLoads>();
   phase_barrier();
   if (group == 1) phase_barrier();
   // first matrix phase: scores of tile 0
@@ -654,10 +675,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
   // so it waits for its share now (of its 8 kLoads loads, the 4 kLoads oldest: V(-1), K0, V0, K1).
   // From tile 2 on, the wait that ends a group's vector phase covers the tile the other group
   // reads next.
-  if (group == 1) {
-    if constexpr (T::kLoads == 2) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-  }
+  if (group == 1) wait_tile_loads<DT_SCHED_TRAILING_K1_INFLIGHT * T::kLoads>();
   phase_barrier_after_matrix(s_acc, o_acc);
 
   // one iteration = vector phase of tile t, then matrix phase (P V of tile t, scores of t+1)
@@ -671,7 +689,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
     // (D = 64: four wavefronts of two workgroups share the SIMD and the raised priority only gets in
     // the way of the other workgroup's matrix phase: measured -3 %, so it is left at 0 there)
     __builtin_amdgcn_s_setprio(D == 64 ? 0 : 1);
-    if constexpr (!kLoadAfterMatrix) load_tile((kU + 3 + group) & (kNumBuf - 1));
+    if constexpr (!kLoadAfterMatrix) load_tile((kU + DT_SCHED_CALL_AHEAD + group) & (kNumBuf - 1));
     // (kPre: the same rare branch takes the reference off the scores of a wavefront in which some
     // row has left the band; everywhere else the reference is 0 and there is nothing to subtract)
     if (__builtin_expect(cp_valid < kBK || (kPre && any_off), 0)) {
@@ -768,12 +786,12 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
     }
     l_run += rs0 + rs1;
     ring_prefill(u_tag);
-    phase_barrier_after_vector<(kLoadAfterMatrix ? 1 : 3) * T::kLoads>(p_frag);
+    phase_barrier_after_vector<kVectorInFlight * T::kLoads>(p_frag);
 
     // ======== matrix phase: O^T += V^T P^T (tile t), S^T = K Q^T (tile t+1) ========
     __builtin_amdgcn_s_setprio(0);
     matrix_phase(u_tag);
-    if constexpr (kLoadAfterMatrix) load_tile((kU + 3 + group) & (kNumBuf - 1));
+    if constexpr (kLoadAfterMatrix) load_tile((kU + DT_SCHED_CALL_AHEAD + group) & (kNumBuf - 1));
     // the tile after the last one of this workgroup's range has no keys for it (its scores are
     // computed on whatever the buffer holds and never used; it may belong to the next part of a
     // split item)
@@ -795,7 +813,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
   }
   // tile loads issued for tiles past the end are still on their way (they store zeros): let them
   // land before the epilogue reuses the tile buffers
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  wait_tile_loads<0>();
   // the leading group waits out the phase it is ahead
   if (group == 0) phase_barrier();
 
