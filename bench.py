@@ -481,6 +481,19 @@ def run_workload(name, args, steps, warmup, main, reuse=None, kernels_only=False
     kr_ms = time_kernel(Rotation(probe, L_run), reps)
     kr_gbs = C * probe_bytes / (kr_ms * 1e-3) / 1e9
 
+    # what launches of these grids cost before they move a byte: an empty kernel of the merge's grid (16 units of 128
+    # elements per 256-thread workgroup and pass; two passes for 6 and more states at D = 128 and for launches of 2^20
+    # units and more at D = 64) and of the flat copy's (8 KB per 512-thread workgroup)
+    units = rows * D // 128
+    merge_passes = 2 if ((D == 128 and C >= 6) or (D == 64 and units >= (1 << 20))) else 1
+    merge_wgs = -(-units // (16 * merge_passes))
+    copy_wgs = -(-(rows * (2 * D + 4)) // 8192)
+    floor_merge_ms = time_kernel(lambda: bench_probes.empty_launch(merge_wgs, 256), reps)
+    floor_copy_ms = time_kernel(lambda: bench_probes.empty_launch(copy_wgs, 512), reps)
+    launch_floor = {"merge_grid": [merge_wgs, 256], "merge_grid_us": round(floor_merge_ms * 1e3, 2),
+                    "copy_grid": [copy_wgs, 512], "copy_grid_us": round(floor_copy_ms * 1e3, 2),
+                    "what": "an empty kernel of the same grid, launched back to back: the part of a short launch that is not bandwidth"}
+
     traffic = load_traffic(name)   # per launch shape: the same whatever reuse fraction drew the mask
     # counter bytes of exactly the launch shape that is timed next to them, or nothing
     k1_traffic = traffic.get("attn_fwd", {}).get(str(n_typ)) if isinstance(traffic.get("attn_fwd"), dict) else None
@@ -530,7 +543,9 @@ def run_workload(name, args, steps, warmup, main, reuse=None, kernels_only=False
                "merge": {"frac": roofline_merge["frac"], "gbs": roofline_merge["achieved"], "states": C,
                          "launch_us": roofline_merge["launch_us"], "read_probe_gbs": roofline_merge["read_probe_gbs"],
                          "traffic": k2_traffic},
-               "cache_gbs": {"store_bf16_to_slot": cache_gbs["store_bf16_to_slot"], "load_slot_to_fp32": cache_gbs["load_slot_to_fp32"]}}
+               "cache_gbs": {"store_bf16_to_slot": cache_gbs["store_bf16_to_slot"], "load_slot_to_fp32": cache_gbs["load_slot_to_fp32"],
+                             "store_bf16_launch_us": round(k3c_ms * 1e3, 2), "load_launch_us": round(k3l_ms * 1e3, 2)},
+               "launch_floor": launch_floor}
     else:
         # producer step of the callers: RMSNorm + interleaved RoPE of K over the whole KV sequence, read in
         # place from a fused QKV projection ("B L (K H D)"), written as the [B,S,H,D] bf16 the attention reads
@@ -595,7 +610,7 @@ def run_workload(name, args, steps, warmup, main, reuse=None, kernels_only=False
             "ms_per_layer_schedule_mean": round(schedule_mean_ms, 4),
             "ms_by_chunks_computed": {str(k): round(float(np.mean(v)), 4) for k, v in sorted(per_count.items())},
             "layer_attn_tflops": round(layer_tflops, 1),
-            "roofline": roofline, "roofline_merge": roofline_merge, "cache_gbs": cache_gbs,
+            "roofline": roofline, "roofline_merge": roofline_merge, "cache_gbs": cache_gbs, "launch_floor": launch_floor,
             "producer": {"kernel": "qk_norm_rope_kernel<%d>" % D, "bound": "hbm", "achieved": round(kp_gbs, 1),
                          "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(kp_gbs / PEAK_HBM_GBS, 4),
                          "launch_us": round(kp_ms * 1e3, 2), "bytes_per_launch": kp_bytes, "tokens": S_all,

@@ -18,6 +18,7 @@ _SIGNATURES = {
     "dtp_hbm_read_probe": (ctypes.c_int, [ctypes.POINTER(c_vp), c_i32, c_i64, c_vp, c_vp]),
     "dtp_mfma_probe": (ctypes.c_int, [c_i32, c_i32, c_vp, c_vp]),
     "dtp_coissue_probe": (ctypes.c_int, [c_i32, c_i32, c_i32, c_i32, c_vp, c_vp]),
+    "dtp_empty_launch": (ctypes.c_int, [c_i32, c_i32, c_vp]),
 }
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 _lib: Optional[ctypes.CDLL] = None
@@ -86,3 +87,8 @@ def coissue_probe(workgroups: int, iters: int, head_dim: int, with_softmax: bool
     _check(lib.dtp_coissue_probe(int(workgroups), int(iters), int(head_dim), int(bool(with_softmax)), sink.data_ptr(),
                                  _stream()), "dtp_coissue_probe")
     return float(workgroups) * 4 * 4 * iters * 32768.0
+
+
+def empty_launch(workgroups: int, threads: int) -> None:
+    """Launch a kernel of that grid that does nothing (the floor of a launch)."""
+    _check(load_library().dtp_empty_launch(int(workgroups), int(threads), _stream()), "dtp_empty_launch")

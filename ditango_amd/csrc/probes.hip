@@ -175,6 +175,9 @@ __global__ __launch_bounds__(kReadThreads) void hbm_read_probe_kernel(const Prob
   if (acc == 0x9e3779b9u) a.sink[0] = acc;
 }
 
+// A kernel that does nothing: what a launch of a given grid costs before it moves a byte.
+__global__ void empty_kernel() {}
+
 }  // namespace dt
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
@@ -242,4 +245,13 @@ extern "C" int dtp_hbm_read_probe(const void* const* streams, int32_t n_streams,
   }
   hipLaunchKernelGGL(dt::hbm_read_probe_kernel, dim3((unsigned)wgs), dim3(dt::kReadThreads), 0, (hipStream_t)stream, a);
   return probe_fail(hipGetLastError(), "hbm_read_probe launch");
+}
+
+extern "C" int dtp_empty_launch(int32_t workgroups, int32_t threads, void* stream) {
+  if (workgroups <= 0 || threads <= 0 || threads > 1024 || threads % 64 != 0) {
+    probe_error("empty launch: need a positive grid and 64..1024 threads in multiples of 64");
+    return DTP_ERR_INVALID;
+  }
+  hipLaunchKernelGGL(dt::empty_kernel, dim3((unsigned)workgroups), dim3((unsigned)threads), 0, (hipStream_t)stream);
+  return probe_fail(hipGetLastError(), "empty launch");
 }

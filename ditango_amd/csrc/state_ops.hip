@@ -788,7 +788,12 @@ int launch_copy(const CopyArgs& a, int D, hipStream_t stream) {
     const int64_t rows = (int64_t)a.B * a.Sq * a.H;
     const int64_t groups = rows * D / 4;
     const int64_t w_out = (groups + kConvThreads - 1) / kConvThreads;
-    const int lse_run = a.H <= 256 ? 64 : std::max(1, 16384 / a.H);   // at most 64 KB of LDS
+    // Query positions per lse workgroup.  Runs of 64 floats per head read whole 256-byte lines of a [H][S] source,
+    // but on a small state the few workgroups that result each walk a dozen dependent rounds of loads and finish
+    // long after the streaming part (2222 x 48 heads: 35 workgroups of 3072 values, 16.6 us for a 42 MB launch
+    // against 10 us with runs of 16); so a workgroup takes about 1024 values, in runs of at least 16 floats.
+    int lse_run = a.H <= 256 ? 64 : std::max(1, 16384 / a.H);   // at most 64 KB of LDS
+    if ((int64_t)a.B * a.Sq * a.H < (1 << 18)) lse_run = std::min(lse_run, std::max(16, 1024 / a.H / 16 * 16));
     const int64_t w_lse = with_lse ? (int64_t)a.B * ((a.Sq + lse_run - 1) / lse_run) : 0;
     if (w_out + w_lse <= 0) return DT_OK;
     if (w_out + w_lse > 0x7fffffffLL || (int64_t)lse_run * a.H * 4 > 65536) {

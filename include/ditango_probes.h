@@ -55,6 +55,13 @@ int dtp_mfma_probe(int32_t workgroups, int32_t iters, float* sink, void* stream)
 int dtp_coissue_probe(int32_t workgroups, int32_t iters, int32_t head_dim, int32_t with_softmax, float* sink,
                       void* stream);
 
+/*
+ * Launches a kernel of `workgroups` x `threads` that does nothing.  Timed back to back it gives the floor of a
+ * launch of that grid (dispatch of the workgroups included) -- what a short HBM-bound launch (a merge or a
+ * cache copy of a few MB) pays before it moves a byte.
+ */
+int dtp_empty_launch(int32_t workgroups, int32_t threads, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -450,3 +450,45 @@ def test_varlen_mask_mode_at_full_size(env, hip):
         assert err <= OUT_TOL and lerr <= LSE_TOL and rel <= 1e-2
         q = (q.float() + 0.01 * torch.randn(q.shape, generator=g)).bfloat16()
         del dk, dv
+
+
+@pytest.mark.parametrize("name", ["cogvideox", "hunyuanvideo", "stepvideo", "sweep_chunk"])
+def test_every_row_at_full_size_against_the_fp32_kernel(hip, name):
+    """The oracle runs on the host, so at full size it covers a sample of the query rows.  The rows in between are
+    covered here: one chunk state of every configuration's real shape, ALL rows, heads and keys, computed by the
+    bf16 MFMA kernel (plain launch and tail-balanced launch) against the fp32 vector-ALU kernel
+    ``dt_attn_chunk_f32_fwd`` on the same (bf16-valued) numbers -- an independent implementation (no MFMA, no LDS
+    prefetch schedule, expf / logf) that the small-shape tests pin against the oracle.  Bar as everywhere:
+    out <= 2e-2, lse <= 1e-3; observed two orders below."""
+    if name == "sweep_chunk":
+        B, H, D, Sq, Sk, norm = 1, 24, 128, 119056, 3721, "rms"
+    else:
+        B, H, D, Sq, lens, _, _, _, _, norm = CONFIGS[name]
+        Sk = lens[0]
+    dev = "cuda"
+    g = torch.Generator(device=dev).manual_seed(11)
+
+    def draw(n, normalise):
+        x = torch.randn(B, n, H, D, generator=g, device=dev)
+        if normalise == "rms":
+            x = x / x.pow(2).mean(-1, keepdim=True).sqrt()
+        elif normalise == "layer":
+            x = torch.nn.functional.layer_norm(x, (D,))
+        return x.bfloat16()
+
+    q, k, v = draw(Sq, norm), draw(Sk, norm), draw(Sk, None)
+    print(f"case all rows {name}: H={H} D={D} Sq={Sq} Sk={Sk}", flush=True)
+    ref_o, ref_l = hip.attn_chunk_f32_fwd(q.float(), k.float(), v.float())
+    torch.cuda.synchronize()
+    table = hip.ChunkTable([k], [v])
+    for how, ws in (("plain", None), ("tail-balanced", hip.attn_workspace(dev))):
+        out = torch.empty(B, Sq, H, D, dtype=torch.bfloat16, device=dev)
+        lse = torch.empty(B, H, Sq, dtype=torch.float32, device=dev)
+        hip.attn_jobs_fwd(q, table, [[0]], [out], [lse], workspace=ws)
+        torch.cuda.synchronize()
+        err = (out.float() - ref_o).abs().max().item()
+        lerr = (lse - ref_l).abs().max().item()
+        rel = ((out.float() - ref_o).norm() / ref_o.norm()).item()
+        print(f"  {how}: out max-abs {err:.3e} rel-l2 {rel:.3e} lse max-abs {lerr:.3e} over {B * Sq * H} rows", flush=True)
+        assert torch.isfinite(out).all() and torch.isfinite(lse).all()
+        assert err <= OUT_TOL and lerr <= LSE_TOL and rel <= 1e-2, (name, how)

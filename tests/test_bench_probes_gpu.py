@@ -48,3 +48,11 @@ def test_coissue_probe_runs_and_checks_its_arguments(probes):
     for bad in ((0, 16, 128), (64, 0, 128), (64, 6, 64), (64, 16, 96)):
         with pytest.raises(probes.ProbeError):
             probes.coissue_probe(*bad, True, sink)
+
+
+def test_empty_launch_runs_and_checks_its_arguments(probes):
+    probes.empty_launch(3333, 256)
+    torch.cuda.synchronize()
+    for bad in ((0, 256), (10, 0), (10, 100), (10, 2048)):
+        with pytest.raises(probes.ProbeError):
+            probes.empty_launch(*bad)
