@@ -5,8 +5,9 @@ The reference's call sites import the hot path as ``ditango.*``
 executor/step/attentions.py:6-12).  With this directory on ``sys.path`` those imports work
 unchanged: every name below is the SAME module object as its ``ditango_amd`` counterpart (one
 step counter, one redundancy map, one set of groups), not a copy.  Only the modules of the
-cached block attention path exist; ``ditango.executor``, ``ditango.baseline`` and
-``ditango.core.initialize`` of the reference are not part of this build and raise ImportError.
+cached block attention path and its three call-site adapters (``ditango.executor.*``: the attention
+processors only, not the model forks) exist; ``ditango.baseline`` and ``ditango.core.initialize`` of the
+reference are not part of this build and raise ImportError.
 """
 import importlib
 import sys
@@ -14,7 +15,9 @@ import sys
 import ditango_amd as _impl
 
 _ALIASED = ("logger", "timer", "utils", "producer", "core", "core.config", "core.parallel_state",
-            "core.redundancy_map", "core.cache", "core.attention")
+            "core.redundancy_map", "core.cache", "core.attention", "executor", "executor.cogvideox",
+            "executor.cogvideox.attention_processor", "executor.hunyuanvideo", "executor.hunyuanvideo.attention_hunyuan",
+            "executor.step", "executor.step.attentions")
 
 for _name in _ALIASED:
     _mod = importlib.import_module("ditango_amd." + _name)
@@ -23,4 +26,4 @@ for _name in _ALIASED:
         globals()[_name] = _mod
 
 __version__ = _impl.__version__
-__all__ = ["logger", "timer", "utils", "producer", "core"]
+__all__ = ["logger", "timer", "utils", "producer", "core", "executor"]

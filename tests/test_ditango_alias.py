@@ -30,7 +30,15 @@ def test_reference_import_lines_resolve_to_the_same_modules():
     assert impl_utils.get_timestep() == 7 == get_timestep()
     update_timestep(0)
     assert callable(get_timer("x").__enter__) and init_logger("t") is not None
-    for missing in ("ditango.executor", "ditango.baseline", "ditango.core.initialize"):
+    # the three attention adapters resolve under the reference's paths; the model forks, the comparison
+    # baselines and the multi-process bootstrap are not part of the package
+    from ditango.executor.cogvideox.attention_processor import CVX_oCacheAttnProcessor
+    from ditango.executor.hunyuanvideo.attention_hunyuan import Hunyuan_DiTangoProcessor, MEMORY_LAYOUT
+    from ditango.executor.step.attentions import Attention
+    import ditango_amd.executor.step.attentions as impl_step
+    assert Attention is impl_step.Attention and callable(CVX_oCacheAttnProcessor) and callable(Hunyuan_DiTangoProcessor)
+    assert set(MEMORY_LAYOUT) == {"flash", "torch", "vanilla", "oAttn"}
+    for missing in ("ditango.baseline", "ditango.core.initialize", "ditango.executor.cogvideox.pipeline_cogvideox"):
         with pytest.raises(ImportError):
             __import__(missing)
 
