@@ -288,6 +288,46 @@ def bench_stride_schedule(args):
     }), flush=True)
 
 
+def bench_item_model(args):
+    """``--item-model``: what a work item of the attention kernel costs on top of its key tiles.  Launches whose
+    items exactly fill the chip's workgroup slots (256 at D = 128, 512 at D = 64: 8 query tiles x 32 / 64 heads), with
+    1, 2 and 4 rounds of such items (the same chunk as several jobs) and 8 ... 233 key tiles per item; prints the
+    launches and the least-squares fit  round time = item cost + tile time x tiles  over the rounds after the first."""
+    from ditango_amd import _hip
+    dev = torch.device("cuda", 0)
+    out = {"metric": "attention work-item cost model", "unit": "us", "n_gpus": 1, "dtype": "bf16", "data": "synthetic", "fits": {}}
+    for D, heads, tiles_list in ((64, 64, (8, 16, 35, 70)), (128, 32, (8, 16, 59, 117, 233))):
+        B, Sq = 1, 2048
+        q = torch.randn(B, Sq, heads, D, device=dev).bfloat16()
+        rows = []
+        for tiles in tiles_list:
+            Sk = tiles * 64
+            k = torch.randn(B, Sk, heads, D, device=dev).bfloat16()
+            v = torch.randn(B, Sk, heads, D, device=dev).bfloat16()
+            table = _hip.ChunkTable([k], [v])
+            o = torch.empty_like(q)
+            l = torch.empty(B, heads, Sq, device=dev)
+            per_rounds = {}
+            for rounds in (1, 2, 4):
+                ms = min(time_kernel(lambda: _hip.attn_jobs_fwd(q, table, [[0]] * rounds, [o] * rounds, [l] * rounds),
+                                     args.kernel_reps) for _ in range(3))
+                per_rounds[rounds] = ms * 1e3
+            later = (per_rounds[4] - per_rounds[1]) / 3.0         # one round behind the first
+            rows.append({"tiles": tiles, "us_1_round": round(per_rounds[1], 1), "us_2_rounds": round(per_rounds[2], 1),
+                         "us_4_rounds": round(per_rounds[4], 1), "us_per_later_round": round(later, 2),
+                         "first_round_extra_us": round(per_rounds[1] - later, 2)})
+        x = np.array([r["tiles"] for r in rows], dtype=np.float64)
+        y = np.array([r["us_per_later_round"] for r in rows], dtype=np.float64)
+        slope, icpt = np.polyfit(x, y, 1)
+        items = heads * (Sq // 256)
+        flop_tile_round = 4.0 * items * 256 * 64 * D
+        out["fits"][f"D{D}"] = {"items_per_round": items, "launches": rows, "tile_us": round(float(slope), 3),
+                                "item_cost_us": round(float(icpt), 2), "item_cost_tiles": round(float(icpt / slope), 2),
+                                "steady_state_tflops": round(flop_tile_round / (slope * 1e-6) / 1e12, 1),
+                                "max_fit_error": round(float(np.max(np.abs(slope * x + icpt - y) / y)), 4)}
+    print(json.dumps(out), flush=True)
+
+
 def load_traffic(workload):
     """HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE runs, committed under profiles/
     (``{"attn_fwd": {"<chunks per launch>": bytes, ...}, "merge_states": {"<states>": bytes}}``)."""
@@ -653,6 +693,9 @@ def main():
     ap.add_argument("--schedule", default="mask", choices=["mask", "stride"],
                     help="mask: the seeded Bernoulli reuse mask (the headline metric); stride: the reference's own stride "
                          "schedule from the HunyuanVideo redundancy map it ships (a separate, shorter report)")
+    ap.add_argument("--item-model", action="store_true",
+                    help="a separate report: the attention kernel's time per key tile and per work item, fitted from launches "
+                         "that exactly fill the chip (both head dimensions)")
     ap.add_argument("--kernels-only", action="store_true",
                     help="run only the per-kernel roofline launches (short; for rocprofv3 counter passes)")
     args = ap.parse_args()
@@ -676,6 +719,8 @@ def main():
     global PROFILING
     PROFILING = args.kernels_only
 
+    if args.item_model:
+        return bench_item_model(args)
     if args.schedule == "stride":
         return bench_stride_schedule(args)
     result = run_workload(args.workload, args, args.steps, args.warmup, main=True, reuse=args.reuse,
