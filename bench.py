@@ -15,8 +15,11 @@ Prints ONE JSON line: ms per layer call plus
   * ``roofline``        the fresh-chunk attention kernel against the bf16 dense MFMA peak,
   * ``roofline_merge``  the fused LSE-merge kernel against the HBM peak,
   * ``cache_gbs``       cache store / load copies against the HBM peak,
+  * ``launch_floor``    empty kernels of the merge's and the copy's grids (what a short launch pays before it moves a byte),
+  * ``varlen``          the variable-length entry with its cu_seqlens on the GPU, as the model passes them,
   * ``other_configs``   compact records of the other single-GPU configurations (CogVideoX share,
-                        Step-Video share, the 32-chunk reuse sweep),
+                        Step-Video share, the 32-chunk reuse sweep) and ``stride_schedule``: one full pass of the
+                        reference's own stride schedule from the HunyuanVideo redundancy map it ships,
   * ``cpu_baseline``    the torch-math oracle timed on this box's host cores on a bounded sample.
 The HBM-bound kernels are timed over a rotation of distinct buffers of more than 1 GB in total,
 so the figures are those of HBM and not of the 256 MB memory-side cache.
