@@ -1,7 +1,8 @@
 // A caller of libditango_hip.so that knows nothing but the C header and the HIP runtime: two KV chunks of
 // attention (dt_attn_jobs_fwd), their merge (dt_merge_states), a trip through a cache slot
-// (dt_cache_store / dt_cache_load) and a device-built schedule (dt_build_schedule), each checked against
-// plain host loops in double precision.  Exit status 0 = everything within the library's stated bounds
+// (dt_cache_store / dt_cache_load), a device-built schedule (dt_build_schedule) and a packed variable-length
+// batch whose segment boundaries live in device memory (dt_attn_varlen_jobs_fwd, dt_zero_rows_from), each checked
+// against plain host loops in double precision.  Exit status 0 = everything within the library's stated bounds
 // (out 2e-2, lse 1e-3, integer results exact).
 #include <hip/hip_runtime.h>
 
@@ -147,6 +148,27 @@ int main() {
   HIP_OK(hipMalloc((void**)&dcnt, 2 * 4));
   const int t = 1, l = 2, diag = 3;
   DT_CHECK(dt_build_schedule(dmask, T, L, C, t, l, diag, dcomp, dreu, dcnt, stream));
+  // ---- a packed batch of two segments against chunk 0, boundaries in device memory (never read on the host) ----
+  const int32_t cu_q[3] = {0, 50, 64}, cu_k[3] = {0, 60, 100};      // rows 64..69 belong to no segment
+  int32_t *d_cu_q, *d_cu_k;
+  void* dvar_o;
+  float* dvar_l;
+  HIP_OK(hipMalloc((void**)&d_cu_q, sizeof cu_q));
+  HIP_OK(hipMalloc((void**)&d_cu_k, sizeof cu_k));
+  HIP_OK(hipMemcpy(d_cu_q, cu_q, sizeof cu_q, hipMemcpyHostToDevice));
+  HIP_OK(hipMemcpy(d_cu_k, cu_k, sizeof cu_k, hipMemcpyHostToDevice));
+  HIP_OK(hipMalloc(&dvar_o, state_elems * 2));
+  HIP_OK(hipMalloc((void**)&dvar_l, lse_elems * 4));
+  HIP_OK(hipMemset(dvar_o, 0xff, state_elems * 2));                  // NaN patterns: rows outside the segments must be zeroed
+  const int32_t vjob_begin[3] = {0, 1, 2}, vjob_chunks[2] = {0, 0}, vjob_seg[2] = {0, 1};
+  const int32_t* cu_kv_tab[2] = {d_cu_k, nullptr};                   // chunk 1 is not referenced
+  void* vouts[2] = {dvar_o, dvar_o};
+  float* vlses[2] = {dvar_l, dvar_l};
+  const int32_t one_len[2] = {Sk[0], 0};
+  DT_CHECK(dt_attn_varlen_jobs_fwd(dq, B, Sq, H, D, (int64_t)Sq * H * D, (int64_t)H * D, D, n_chunks, kp, vp, one_len, kv_sb,
+                                   (int64_t)H * D, D, 2, vjob_begin, vjob_chunks, vjob_seg, 2, d_cu_q, cu_kv_tab, 50, vouts, vlses,
+                                   0.f, 0, stream));
+  DT_CHECK(dt_zero_rows_from(dvar_o, Sq, (int64_t)H * D * 2, d_cu_q + 2, stream));
   HIP_OK(hipStreamSynchronize(stream));
 
   // ---- checks --------------------------------------------------------------------------------------------
@@ -184,6 +206,42 @@ int main() {
   for (size_t i = 0; i < want_comp.size() && i < (size_t)C; ++i) sched_bad += comp[i] != want_comp[i];
   for (size_t i = 0; i < want_reu.size() && i < (size_t)C; ++i) sched_bad += reu[i] != want_reu[i];
 
+  // the packed batch: segment s of the queries against segment s of chunk 0's keys; zero rows behind the last boundary
+  std::vector<uint16_t> vo(state_elems);
+  std::vector<float> vl(lse_elems);
+  HIP_OK(hipMemcpy(vo.data(), dvar_o, state_elems * 2, hipMemcpyDeviceToHost));
+  HIP_OK(hipMemcpy(vl.data(), dvar_l, lse_elems * 4, hipMemcpyDeviceToHost));
+  double e_var = 0, e_vlse = 0;
+  int var_bad = 0;
+  for (int h = 0; h < H; ++h)
+    for (int sq = 0; sq < Sq; ++sq) {
+      int seg = -1;
+      for (int g = 0; g < 2; ++g)
+        if (sq >= cu_q[g] && sq < cu_q[g + 1]) seg = g;
+      if (seg < 0) {
+        for (int e = 0; e < D; ++e) var_bad += vo[((size_t)sq * H + h) * D + e] != 0;
+        continue;
+      }
+      std::vector<double> sc;
+      double mx = -1e300, den = 0;
+      for (int j = cu_k[seg]; j < cu_k[seg + 1]; ++j) {
+        double d = 0;
+        for (int e = 0; e < D; ++e) d += at(q, sq, h, e) * at(k[0], j, h, e);
+        sc.push_back(d * scale);
+        mx = std::fmax(mx, d * scale);
+      }
+      std::vector<double> o(D, 0.0);
+      for (int j = cu_k[seg]; j < cu_k[seg + 1]; ++j) {
+        const double p = std::exp(sc[j - cu_k[seg]] - mx);
+        den += p;
+        for (int e = 0; e < D; ++e) o[e] += p * at(v[0], j, h, e);
+      }
+      for (int e = 0; e < D; ++e) e_var = std::fmax(e_var, std::fabs(from_bf16(vo[((size_t)sq * H + h) * D + e]) - o[e] / den));
+      e_vlse = std::fmax(e_vlse, std::fabs(vl[(size_t)h * Sq + sq] - (mx + std::log(den))));
+    }
+  std::printf("capi demo: packed batch with device-resident boundaries: out max-abs %.3e, lse max-abs %.3e, non-zero rows outside "
+              "the segments %d\n", e_var, e_vlse, var_bad);
+
   std::printf("capi demo: version %d, out max-abs %.3e, merged lse max-abs %.3e, chunk lse max-abs %.3e, "
               "slot round trip mismatches %d, schedule mismatches %d\n",
               dt_version(), e_out, e_lse, e_clse, bad, sched_bad);
@@ -191,7 +249,8 @@ int main() {
   const int rc = dt_merge_states(0, mo, ml, nullptr, nullptr, dout, DT_FP32, dlse, DT_LSE_BHS, B, Sq, H, D, stream);
   const bool err_ok = rc == DT_ERR_INVALID && std::strlen(dt_last_error()) > 0;
   if (!err_ok) std::fprintf(stderr, "expected DT_ERR_INVALID with a message for a merge of 0 states, got %d\n", rc);
-  const bool ok = e_out <= 2e-2 && e_lse <= 1e-3 && e_clse <= 1e-3 && bad == 0 && sched_bad == 0 && err_ok;
+  const bool ok = e_out <= 2e-2 && e_lse <= 1e-3 && e_clse <= 1e-3 && bad == 0 && sched_bad == 0 && err_ok &&
+                  e_var <= 2e-2 && e_vlse <= 1e-3 && var_bad == 0;
   std::printf(ok ? "capi demo ok\n" : "capi demo FAILED\n");
   return ok ? 0 : 1;
 }
