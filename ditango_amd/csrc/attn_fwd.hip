@@ -318,11 +318,16 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
       q_end = q_begin + a.job_q_len[job];
     }
   }
+  // Segment boundaries are read through the constant address space, i.e. with scalar loads: the lists were
+  // written before the launch and the address is uniform.  (As a vector load the compiler follows it with
+  // vmcnt(0), which inside the loop would also wait for every tile load in flight.)
+  typedef const int32_t __attribute__((address_space(4))) ConstI32;
+  auto boundary = [](const int32_t* list, int i) __attribute__((always_inline)) -> int { return ((ConstI32*)list)[i]; };
   if (dseg >= 0) {
     // boundaries from device memory: nothing on the host has looked at them, so they are clamped
     // to the rows that exist (a malformed list then yields wrong rows, never a stray access)
-    q_begin = min(max(__builtin_amdgcn_readfirstlane(a.cu_q[dseg]), 0), a.Sq);
-    q_end = min(max(__builtin_amdgcn_readfirstlane(a.cu_q[dseg + 1]), q_begin), a.Sq);
+    q_begin = min(max(boundary(a.cu_q, dseg), 0), a.Sq);
+    q_end = min(max(boundary(a.cu_q, dseg + 1), q_begin), a.Sq);
   }
   if (qt * kBQ >= q_end - q_begin) return;  // the grid is sized for the longest job / segment
   auto chunk_of = [&](int seg) __attribute__((always_inline)) -> int { return single >= 0 ? single : a.job_chunks[seg]; };
@@ -330,7 +335,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
   auto kv_begin_of = [&](int seg) __attribute__((always_inline)) -> int {
     if (dseg >= 0) {
       const int cid = chunk_of(seg);
-      return min(max(__builtin_amdgcn_readfirstlane(a.cu_kv[cid][dseg]), 0), a.kv_len[cid]);
+      return min(max(boundary(a.cu_kv[cid], dseg), 0), a.kv_len[cid]);
     }
     if (single < 0) return a.entry_kv_begin[seg];
     return vseg >= 0 ? a.entry_kv_begin[single * a.n_seg + vseg] : 0;
@@ -338,8 +343,8 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
   auto kv_len_of = [&](int seg) __attribute__((always_inline)) -> int {
     if (dseg >= 0) {
       const int cid = chunk_of(seg);
-      const int lo = min(max(__builtin_amdgcn_readfirstlane(a.cu_kv[cid][dseg]), 0), a.kv_len[cid]);
-      const int hi = min(max(__builtin_amdgcn_readfirstlane(a.cu_kv[cid][dseg + 1]), lo), a.kv_len[cid]);
+      const int lo = min(max(boundary(a.cu_kv[cid], dseg), 0), a.kv_len[cid]);
+      const int hi = min(max(boundary(a.cu_kv[cid], dseg + 1), lo), a.kv_len[cid]);
       return hi - lo;
     }
     if (single < 0) return a.entry_kv_len[seg];
