@@ -1,6 +1,6 @@
-"""The reference-side binding that INTEGRATION.md shows a maintainer (section B: ``flash_attn_func`` and
+"""The reference-side binding that the integration guide shows a maintainer (``flash_attn_func`` and
 ``flash_attn_varlen_func`` as ctypes stubs over the C ABI) is executed as written -- only the library's path is
-filled in -- and checked against the oracle, so the document cannot drift from the ABI."""
+filled in -- and checked against the oracle, so the guide cannot drift from the ABI."""
 import os
 import re
 
@@ -11,16 +11,17 @@ from oracle import attention_math as om
 
 pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GUIDE = os.path.join(ROOT, "INTEGRATION.md")
 
 
 def _stub_namespace(hip):
-    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    text = open(GUIDE).read()
     section = text[text.index("## B."):text.index("## C.")]
     blocks = re.findall(r"```python\n(.*?)```", section, flags=re.S)
     assert len(blocks) == 2 and "def flash_attn_func" in blocks[0] and "def flash_attn_varlen_func" in blocks[1]
     code = "\n".join(blocks).replace('ctypes.CDLL("libditango_hip.so")', f'ctypes.CDLL("{hip.LIB_PATH}")')
     ns = {}
-    exec(compile(code, "INTEGRATION.md section B", "exec"), ns)
+    exec(compile(code, "binding stubs of the integration guide", "exec"), ns)
     return ns
 
 
