@@ -719,6 +719,13 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
     // with its exact maximum.
     float mc = m_ref * c;
     float rs0 = rs_bias, rs1 = 0.f;
+    // The first tile of a work item always takes the exact path below (its reference is still -inf), so its pass
+    // through the common path is thrown away: skip it.  Results are bit-identical; +0.4-0.5 % at D = 128.  (At
+    // D = 64 the extra branch costs registers the kernel does not have: 36 spills, -18 %; it keeps the plain form.)
+    if (D == 128 && __builtin_expect(t == 0, 0)) {
+      asm volatile("" ::: "memory");   // keeps this a real branch
+      rs0 = INFINITY;
+    } else
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
