@@ -447,6 +447,13 @@ def run_workload(name, args, steps, warmup, main, reuse=None, kernels_only=False
     q_folded = (q.float() * (D ** -0.5 * math.log2(math.e))).to(torch.bfloat16)
     k1p_ms = time_kernel(lambda: k1_launch(n_typ, q_folded, True), reps)
     k1p_tflops = k1_flops(n_typ) / (k1p_ms * 1e-3) / 1e12
+    # the same typical launch on IEEE-half copies of the tensors (a model run in fp16: fp16 MFMA, fp16 states)
+    qh, ksh, vsh = q.half(), [k.half() for k in ks[:n_typ]], [v.half() for v in vs[:n_typ]]
+    table_h = _hip.ChunkTable(ksh, vsh)
+    sth = [torch.empty(B, Sq, H, D, dtype=torch.float16, device=dev) for _ in range(n_typ)]
+    k1h_ms = time_kernel(lambda: _hip.attn_jobs_fwd(qh, table_h, [[c] for c in range(n_typ)], sth, st_lses[:n_typ], workspace=k1_ws), reps)
+    k1h_tflops = k1_flops(n_typ) / (k1h_ms * 1e-3) / 1e12
+    del qh, ksh, vsh, table_h, sth
     clock = None
     mfma_probe = None
     if main and not kernels_only:
@@ -547,7 +554,8 @@ def run_workload(name, args, steps, warmup, main, reuse=None, kernels_only=False
                 "traffic": k1_traffic, "launch_ms": round(k1_ms, 4), "flop_per_launch": k1_flops(n_typ),
                 "chunks_per_launch": n_typ, "single_chunk_launch_tflops": round(k1s_tflops, 1),
                 "single_chunk_launch_ms": round(k1s_ms, 4),
-                "q_prescaled_launch_tflops": round(k1p_tflops, 1), "q_prescaled_launch_ms": round(k1p_ms, 4)}
+                "q_prescaled_launch_tflops": round(k1p_tflops, 1), "q_prescaled_launch_ms": round(k1p_ms, 4),
+                "fp16_launch_tflops": round(k1h_tflops, 1), "fp16_launch_ms": round(k1h_ms, 4)}
     if clock:
         # the part is power-limited under this kernel: what the kernel reaches of the peak AT THE CLOCK IT RUNS AT
         roofline["clock_mhz_under_load"] = clock
@@ -580,7 +588,8 @@ def run_workload(name, args, steps, warmup, main, reuse=None, kernels_only=False
                "layer_attn_tflops": round(layer_tflops, 1),
                "attn": {"frac": roofline["frac"], "tflops": roofline["achieved"], "chunks_per_launch": n_typ,
                         "launch_ms": roofline["launch_ms"], "single_chunk_frac": round(k1s_tflops / PEAK_BF16_TFLOPS, 4),
-                        "q_prescaled_frac": round(k1p_tflops / PEAK_BF16_TFLOPS, 4), "traffic": k1_traffic,
+                        "q_prescaled_frac": round(k1p_tflops / PEAK_BF16_TFLOPS, 4),
+                        "fp16_frac": round(k1h_tflops / PEAK_BF16_TFLOPS, 4), "traffic": k1_traffic,
                         "coissue_probe": coissue,
                         "frac_of_coissue_ceiling": roofline.get("frac_of_coissue_ceiling")},
                "merge": {"frac": roofline_merge["frac"], "gbs": roofline_merge["achieved"], "states": C,

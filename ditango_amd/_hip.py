@@ -15,12 +15,12 @@ import torch
 
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libditango_hip.so"
 
-DT_BF16, DT_FP32 = 0, 1
+DT_BF16, DT_FP32, DT_FP16 = 0, 1, 2
 DT_LSE_BHS, DT_LSE_BSH = 0, 1
 DT_NORM_NONE, DT_NORM_RMS, DT_NORM_LAYER = 0, 1, 2
 DT_ROPE_NONE, DT_ROPE_INTERLEAVED, DT_ROPE_HALVES = 0, 1, 2
-DT_ROUND_NORM_BF16, DT_ROUND_ROPE_BF16 = 1, 2
-DT_ATTN_Q_PRESCALED = 1
+DT_ROUND_NORM_BF16, DT_ROUND_ROPE_BF16, DT_IO_FP16 = 1, 2, 4
+DT_ATTN_Q_PRESCALED, DT_ATTN_FP16 = 1, 2
 DT_MAX_CHUNKS = 40
 DT_MAX_JOBS = 40
 DT_MAX_JOB_ENTRIES = 64
@@ -36,6 +36,8 @@ _SIGNATURES = {
     "dt_last_error": (ctypes.c_char_p, []),
     "dt_attn_chunk_fwd": (ctypes.c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_i32,
                                          c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_f32, c_vp]),
+    "dt_attn_chunk_f16_fwd": (ctypes.c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_i32,
+                                             c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_f32, c_vp]),
     "dt_attn_chunk_f32_fwd": (ctypes.c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_i32,
                                              c_i64, c_i64, c_i64, c_i64, c_i64, c_i64, c_f32, c_vp]),
     "dt_attn_jobs_fwd": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i64, c_i64, c_i64,
@@ -80,6 +82,7 @@ _SIGNATURES = {
                                        c_i32, c_i32, c_i32, c_i32, c_vp]),
     "dt_cache_store": (ctypes.c_int, [c_vp, c_i32, c_vp, c_i32, c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_vp]),
     "dt_cache_load": (ctypes.c_int, [c_vp, c_vp, c_vp, c_i32, c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp]),
+    "dt_state_copy": (ctypes.c_int, [c_vp, c_i32, c_vp, c_i32, c_vp, c_i32, c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp]),
     "dt_build_schedule": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp, c_vp]),
     "dt_build_schedule_table": (ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp, c_vp]),
     "dt_rel_l1_sums": (ctypes.c_int, [c_vp, c_vp, c_i64, c_vp, c_vp]),
@@ -132,7 +135,12 @@ def _dtype_code(t: torch.Tensor) -> int:
         return DT_BF16
     if t.dtype == torch.float32:
         return DT_FP32
-    raise DitangoHipError(f"unsupported state dtype {t.dtype} (bf16 or fp32)")
+    if t.dtype == torch.float16:
+        return DT_FP16
+    raise DitangoHipError(f"unsupported state dtype {t.dtype} (bf16, fp16 or fp32)")
+
+
+HALF_DTYPES = (torch.bfloat16, torch.float16)   # the 16-bit types the attention kernel runs in
 
 
 def _require(cond: bool, msg: str) -> None:
@@ -140,10 +148,18 @@ def _require(cond: bool, msg: str) -> None:
         raise DitangoHipError(msg)
 
 
-def _check_qkv(q: torch.Tensor, name: str = "q") -> None:
+def _check_qkv(q: torch.Tensor, name: str = "q", dtype: Optional[torch.dtype] = None) -> None:
     _require(q.is_cuda, f"{name} must live on the GPU")
-    _require(q.dtype == torch.bfloat16, f"{name} must be bf16 (got {q.dtype})")
+    if dtype is None:
+        _require(q.dtype in HALF_DTYPES, f"{name} must be bf16 or fp16 (got {q.dtype})")
+    else:
+        _require(q.dtype == dtype, f"{name} must be {dtype} like the other attention inputs (got {q.dtype})")
     _require(q.dim() == 4 and q.stride(-1) == 1, f"{name} must be [B,S,H,D] with contiguous D")
+
+
+def _attn_flags(q: torch.Tensor, q_prescaled: bool) -> int:
+    _require(not (q_prescaled and q.dtype == torch.float16), "a prescaled q is a bf16 mode")
+    return (DT_ATTN_Q_PRESCALED if q_prescaled else 0) | (DT_ATTN_FP16 if q.dtype == torch.float16 else 0)
 
 
 def lse_layout_of(lse: torch.Tensor, B: int, S: int, H: int) -> int:
@@ -172,21 +188,22 @@ def lse_layout_of(lse: torch.Tensor, B: int, S: int, H: int) -> int:
 
 def attn_chunk_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, softmax_scale: float = 0.0,
                    out: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None):
-    """(out bf16 [B,Sq,H,D], lse fp32 [B,H,Sq]) of q against one KV chunk."""
+    """(out [B,Sq,H,D] in q's dtype -- bf16 or fp16 --, lse fp32 [B,H,Sq]) of q against one KV chunk."""
     lib = load_library()
-    _check_qkv(q, "q"); _check_qkv(k, "k"); _check_qkv(v, "v")
+    _check_qkv(q, "q"); _check_qkv(k, "k", q.dtype); _check_qkv(v, "v", q.dtype)
     B, Sq, H, D = q.shape
     Sk = k.shape[1]
     _require(k.shape == v.shape and k.shape[0] == B and k.shape[2] == H and k.shape[3] == D, "k/v shape mismatch")
     _require(k.stride() == v.stride(), "k and v must share strides")
     if out is None:
-        out = torch.empty((B, Sq, H, D), dtype=torch.bfloat16, device=q.device)
+        out = torch.empty((B, Sq, H, D), dtype=q.dtype, device=q.device)
     if lse is None:
         lse = torch.empty((B, H, Sq), dtype=torch.float32, device=q.device)
-    _require(out.is_contiguous() and lse.is_contiguous(), "out/lse must be contiguous")
-    rc = lib.dt_attn_chunk_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
-                               B, Sq, Sk, H, D, q.stride(0), q.stride(1), q.stride(2),
-                               k.stride(0), k.stride(1), k.stride(2), float(softmax_scale), _stream())
+    _require(out.is_contiguous() and lse.is_contiguous() and out.dtype == q.dtype, "out/lse must be contiguous, out in q's dtype")
+    fn = lib.dt_attn_chunk_f16_fwd if q.dtype == torch.float16 else lib.dt_attn_chunk_fwd
+    rc = fn(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(),
+            B, Sq, Sk, H, D, q.stride(0), q.stride(1), q.stride(2),
+            k.stride(0), k.stride(1), k.stride(2), float(softmax_scale), _stream())
     _check(rc, "dt_attn_chunk_fwd")
     return out, lse
 
@@ -254,8 +271,9 @@ class ChunkTable:
         self._len: List[int] = []
         self._sb: List[int] = []
         ss = sh = None
+        self.dtype = k_chunks[0].dtype
         for i, (k, v) in enumerate(zip(k_chunks, v_chunks)):
-            _check_qkv(k, f"k[{i}]"); _check_qkv(v, f"v[{i}]")
+            _check_qkv(k, f"k[{i}]", self.dtype); _check_qkv(v, f"v[{i}]", self.dtype)
             _require(k.shape == v.shape and k.stride() == v.stride(), f"k[{i}] / v[{i}] mismatch")
             if k.shape[1] > 0:
                 if ss is None:
@@ -351,7 +369,8 @@ def attn_jobs_fwd(q: torch.Tensor, table: ChunkTable, jobs: Sequence[Sequence[in
     (``dt_attn_varlen_jobs_fwd``); job j is segment ``job_segments[j]`` of its state and the host reads none
     of the boundaries."""
     lib = load_library()
-    _check_qkv(q, "q")
+    _check_qkv(q, "q", table.dtype)
+    flags = _attn_flags(q, q_prescaled)
     B, Sq, H, D = q.shape
     _require((B, H, D) == (table.B, table.H, table.D), "q and KV chunks disagree on B/H/D")
     _require(not (no_alloc and workspace is not None), "no_alloc launches take no workspace")
@@ -365,7 +384,7 @@ def attn_jobs_fwd(q: torch.Tensor, table: ChunkTable, jobs: Sequence[Sequence[in
     _require(kv_ranges is None or len(kv_ranges) == nj, "one list of key ranges per job")
     for j in range(nj):
         o, l = outs[j], lses[j]
-        _require(o.dtype == torch.bfloat16 and o.is_contiguous() and tuple(o.shape) == (B, Sq, H, D), f"outs[{j}] must be contiguous bf16 [B,Sq,H,D]")
+        _require(o.dtype == q.dtype and o.is_contiguous() and tuple(o.shape) == (B, Sq, H, D), f"outs[{j}] must be contiguous [B,Sq,H,D] in q's dtype")
         _require(l.dtype == torch.float32 and l.is_contiguous() and tuple(l.shape) == (B, H, Sq), f"lses[{j}] must be contiguous fp32 [B,H,Sq]")
         _require(len(jobs[j]) <= DT_MAX_JOB_ENTRIES, f"job {j} references more than {DT_MAX_JOB_ENTRIES} chunks")
     # split into launches that fit the per-launch limits (jobs, chunk references, distinct chunks)
@@ -421,20 +440,19 @@ def attn_jobs_fwd(q: torch.Tensor, table: ChunkTable, jobs: Sequence[Sequence[in
                                              t_n, t_k, t_v, t_len, t_sb, table.ss, table.sh,
                                              n, begin, chunks, seg_ids, dev_segments.n_seg, dev_segments.cu_q.data_ptr(),
                                              cu_kv, int(dev_segments.max_seqlen_q), out_ptrs, lse_ptrs,
-                                             float(softmax_scale), DT_ATTN_Q_PRESCALED if q_prescaled else 0, _stream())
+                                             float(softmax_scale), flags, _stream())
             _check(rc, "dt_attn_varlen_jobs_fwd")
         elif no_alloc:
             rc = lib.dt_attn_seg_jobs_noalloc_fwd(q.data_ptr(), B, Sq, H, D, q.stride(0), q.stride(1), q.stride(2),
                                                   t_n, t_k, t_v, t_len, t_sb, table.ss, table.sh,
                                                   n, begin, chunks, a_kvb, a_kvl, a_qb, a_ql, out_ptrs,
-                                                  lse_ptrs, float(softmax_scale),
-                                                  DT_ATTN_Q_PRESCALED if q_prescaled else 0, _stream())
+                                                  lse_ptrs, float(softmax_scale), flags, _stream())
             _check(rc, "dt_attn_seg_jobs_noalloc_fwd")
         else:
             rc = lib.dt_attn_seg_jobs_ws_fwd(q.data_ptr(), B, Sq, H, D, q.stride(0), q.stride(1), q.stride(2),
                                              t_n, t_k, t_v, t_len, t_sb, table.ss, table.sh,
                                              n, begin, chunks, a_kvb, a_kvl, a_qb, a_ql, out_ptrs, lse_ptrs,
-                                             float(softmax_scale), DT_ATTN_Q_PRESCALED if q_prescaled else 0,
+                                             float(softmax_scale), flags,
                                              workspace.data_ptr() if workspace is not None else None,
                                              workspace.numel() * workspace.element_size() if workspace is not None else 0,
                                              _stream())
@@ -450,24 +468,25 @@ def attn_sched_fwd(q: torch.Tensor, table: ChunkTable, dev_compute_ids: torch.Te
                    workspace: Optional[torch.Tensor] = None, q_prescaled: bool = False,
                    dev_segments: Optional[DeviceSegments] = None) -> None:
     """Device-scheduled launch: chunk ids come from ``dev_compute_ids[:dev_count]`` in device memory and
-    each state lands in its slot of the arena (``slot_out [C,B,Sq,H,D]`` bf16, ``slot_lse [C,B,H,Sq]`` fp32).
+    each state lands in its slot of the arena (``slot_out [C,B,Sq,H,D]`` in q's dtype, ``slot_lse [C,B,H,Sq]`` fp32).
 
     On a packed variable-length batch, ``seg_q[s] = (begin, length)`` are the query rows of segment s and
     ``seg_kv[c][s] = (begin, length)`` its keys inside chunk c; every scheduled chunk then runs once per segment."""
     lib = load_library()
-    _check_qkv(q, "q")
+    _check_qkv(q, "q", table.dtype)
+    flags = _attn_flags(q, q_prescaled)
     B, Sq, H, D = q.shape
     _require((B, H, D) == (table.B, table.H, table.D), "q and KV chunks disagree on B/H/D")
     _require(dev_compute_ids.dtype == torch.int32 and dev_count.dtype == torch.int32 and dev_compute_ids.is_cuda and dev_count.is_cuda,
              "schedule tensors must be int32 on the GPU")
     _require(dev_compute_ids.is_contiguous() and dev_compute_ids.numel() >= max_jobs, "compute id list shorter than max_jobs")
-    _require(slot_out.dtype == torch.bfloat16 and slot_out.is_contiguous() and tuple(slot_out.shape[1:]) == (B, Sq, H, D)
-             and slot_out.shape[0] >= table.n, "slot_out must be contiguous bf16 [C,B,Sq,H,D]")
+    _require(slot_out.dtype == q.dtype and slot_out.is_contiguous() and tuple(slot_out.shape[1:]) == (B, Sq, H, D)
+             and slot_out.shape[0] >= table.n, "slot_out must be contiguous [C,B,Sq,H,D] in q's dtype")
     _require(slot_lse.dtype == torch.float32 and slot_lse.is_contiguous() and tuple(slot_lse.shape[1:]) == (B, H, Sq)
              and slot_lse.shape[0] >= table.n, "slot_lse must be contiguous fp32 [C,B,H,Sq]")
     if 0 <= diag < table.n:
         _require(diag_out is not None and diag_lse is not None, "a diag chunk needs (diag_out, diag_lse)")
-        _require(diag_out.dtype == torch.bfloat16 and diag_out.is_contiguous() and tuple(diag_out.shape) == (B, Sq, H, D), "diag_out must be contiguous bf16 [B,Sq,H,D]")
+        _require(diag_out.dtype == q.dtype and diag_out.is_contiguous() and tuple(diag_out.shape) == (B, Sq, H, D), "diag_out must be contiguous [B,Sq,H,D] in q's dtype")
         _require(diag_lse.dtype == torch.float32 and diag_lse.is_contiguous() and tuple(diag_lse.shape) == (B, H, Sq), "diag_lse must be contiguous fp32 [B,H,Sq]")
     if dev_segments is not None:
         # segment boundaries in device memory: every scheduled chunk runs once per segment, the host reads nothing
@@ -481,7 +500,7 @@ def attn_sched_fwd(q: torch.Tensor, table: ChunkTable, dev_compute_ids: torch.Te
                                           diag_lse.data_ptr() if diag_lse is not None else None,
                                           dev_segments.n_seg, dev_segments.cu_q.data_ptr(),
                                           dev_segments.kv_pointers(range(table.n)), dev_segments.max_seqlen_q,
-                                          float(softmax_scale), DT_ATTN_Q_PRESCALED if q_prescaled else 0, _stream())
+                                          float(softmax_scale), flags, _stream())
         _check(rc, "dt_attn_sched_varlen_fwd")
         return
     n_seg, a_qb, a_ql, a_kb, a_kl = 0, None, None, None, None
@@ -501,8 +520,7 @@ def attn_sched_fwd(q: torch.Tensor, table: ChunkTable, dev_compute_ids: torch.Te
                                    slot_out.data_ptr(), slot_out.stride(0), slot_lse.data_ptr(), slot_lse.stride(0),
                                    int(diag), diag_out.data_ptr() if diag_out is not None else None,
                                    diag_lse.data_ptr() if diag_lse is not None else None,
-                                   n_seg, a_qb, a_ql, a_kb, a_kl, float(softmax_scale),
-                                   DT_ATTN_Q_PRESCALED if q_prescaled else 0,
+                                   n_seg, a_qb, a_ql, a_kb, a_kl, float(softmax_scale), flags,
                                    workspace.data_ptr() if workspace is not None else None,
                                    workspace.numel() * workspace.element_size() if workspace is not None else 0, _stream())
     _check(rc, "dt_attn_sched_seg_ws_fwd")
@@ -534,7 +552,7 @@ def _merge_once(outs, lses, dst_out, dst_lse, B, Sq, H, D) -> None:
 def merge_states(outs: Sequence[torch.Tensor], lses: Sequence[torch.Tensor],
                  dst_out: Optional[torch.Tensor] = None, dst_lse: Optional[torch.Tensor] = None,
                  dst_dtype: torch.dtype = torch.float32, dst_lse_bsh: bool = False):
-    """N-way LSE merge.  outs[i] contiguous [B,Sq,H,D] (bf16 or fp32), lses[i] fp32 in
+    """N-way LSE merge.  outs[i] contiguous [B,Sq,H,D] (bf16, fp16 or fp32, in any mix), lses[i] fp32 in
     [B,H,Sq] or [B,Sq,H(,1)] storage.  Returns (dst_out, dst_lse).  Up to ``DT_MAX_MERGE`` states are one
     pass over HBM; more are folded in rounds through a running fp32 state that is updated in place (the
     merge is associative; the running state is never rounded below fp32)."""
@@ -566,10 +584,14 @@ def cache_store(src_out: torch.Tensor, src_lse: torch.Tensor, slot_out: torch.Te
     lib = load_library()
     B, Sq, H, D = src_out.shape
     _require(src_out.is_cuda and src_out.is_contiguous(), "src_out must be contiguous on the GPU")
-    _require(slot_out.dtype == torch.bfloat16 and slot_out.is_contiguous() and tuple(slot_out.shape) == (B, Sq, H, D), "slot_out must be contiguous bf16 [B,Sq,H,D]")
+    _require(slot_out.dtype in HALF_DTYPES and slot_out.is_contiguous() and tuple(slot_out.shape) == (B, Sq, H, D), "slot_out must be contiguous bf16 or fp16 [B,Sq,H,D]")
     _require(slot_lse.dtype == torch.float32 and slot_lse.is_contiguous() and tuple(slot_lse.shape) == (B, H, Sq), "slot_lse must be contiguous fp32 [B,H,Sq]")
-    rc = lib.dt_cache_store(src_out.data_ptr(), _dtype_code(src_out), src_lse.data_ptr(), lse_layout_of(src_lse, B, Sq, H),
-                            slot_out.data_ptr(), slot_lse.data_ptr(), B, Sq, H, D, _stream())
+    if slot_out.dtype == torch.bfloat16:
+        rc = lib.dt_cache_store(src_out.data_ptr(), _dtype_code(src_out), src_lse.data_ptr(), lse_layout_of(src_lse, B, Sq, H),
+                                slot_out.data_ptr(), slot_lse.data_ptr(), B, Sq, H, D, _stream())
+    else:   # fp16 slots of a model that runs in fp16
+        rc = lib.dt_state_copy(src_out.data_ptr(), _dtype_code(src_out), src_lse.data_ptr(), lse_layout_of(src_lse, B, Sq, H),
+                               slot_out.data_ptr(), DT_FP16, slot_lse.data_ptr(), DT_LSE_BHS, B, Sq, H, D, _stream())
     _check(rc, "dt_cache_store")
 
 
@@ -577,7 +599,7 @@ def cache_load(slot_out: torch.Tensor, slot_lse: torch.Tensor, dst_dtype: torch.
                dst_lse_bsh: bool = False, dst_out: Optional[torch.Tensor] = None, dst_lse: Optional[torch.Tensor] = None):
     lib = load_library()
     B, Sq, H, D = slot_out.shape
-    _require(slot_out.dtype == torch.bfloat16 and slot_out.is_contiguous(), "slot_out must be contiguous bf16")
+    _require(slot_out.dtype in HALF_DTYPES and slot_out.is_contiguous(), "slot_out must be contiguous bf16 or fp16")
     _require(slot_lse.dtype == torch.float32 and slot_lse.is_contiguous() and tuple(slot_lse.shape) == (B, H, Sq), "slot_lse must be contiguous fp32 [B,H,Sq]")
     if dst_out is None:
         dst_out = torch.empty((B, Sq, H, D), dtype=dst_dtype, device=slot_out.device)
@@ -585,8 +607,13 @@ def cache_load(slot_out: torch.Tensor, slot_lse: torch.Tensor, dst_dtype: torch.
         dst_lse = torch.empty((B, Sq, H, 1) if dst_lse_bsh else (B, H, Sq), dtype=torch.float32, device=slot_out.device)
     _require(dst_out.is_contiguous() and tuple(dst_out.shape) == (B, Sq, H, D), "dst_out must be contiguous [B,Sq,H,D]")
     dst_lse_bsh = lse_layout_of(dst_lse, B, Sq, H) == DT_LSE_BSH
-    rc = lib.dt_cache_load(slot_out.data_ptr(), slot_lse.data_ptr(), dst_out.data_ptr(), _dtype_code(dst_out),
-                           dst_lse.data_ptr(), DT_LSE_BSH if dst_lse_bsh else DT_LSE_BHS, B, Sq, H, D, _stream())
+    if slot_out.dtype == torch.bfloat16:
+        rc = lib.dt_cache_load(slot_out.data_ptr(), slot_lse.data_ptr(), dst_out.data_ptr(), _dtype_code(dst_out),
+                               dst_lse.data_ptr(), DT_LSE_BSH if dst_lse_bsh else DT_LSE_BHS, B, Sq, H, D, _stream())
+    else:
+        rc = lib.dt_state_copy(slot_out.data_ptr(), DT_FP16, slot_lse.data_ptr(), DT_LSE_BHS, dst_out.data_ptr(),
+                               _dtype_code(dst_out), dst_lse.data_ptr(), DT_LSE_BSH if dst_lse_bsh else DT_LSE_BHS,
+                               B, Sq, H, D, _stream())
     _check(rc, "dt_cache_load")
     return dst_out, dst_lse
 
@@ -648,17 +675,18 @@ def qk_norm_rope(x: torch.Tensor, *, norm: int = DT_NORM_NONE, weight: Optional[
                  cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None,
                  rope_begin: int = 0, rope_end: Optional[int] = None, sections: Sequence[int] = (),
                  rounding: int = 0, out: Optional[torch.Tensor] = None, out_scale: float = 1.0) -> torch.Tensor:
-    """x bf16 ``[B,S,H,D]`` (any strides with a contiguous last dimension) -> bf16 ``[B,S,H,D]`` contiguous,
-    normalised over D and rotated on token rows ``[rope_begin, rope_end)``.  cos/sin are fp32
+    """x bf16 or fp16 ``[B,S,H,D]`` (any strides with a contiguous last dimension) -> ``[B,S,H,D]`` contiguous in
+    the same dtype, normalised over D and rotated on token rows ``[rope_begin, rope_end)``.  cos/sin are fp32
     ``[rope_end-rope_begin, D]`` or ``[B, rope_end-rope_begin, D]``.  ``out_scale`` multiplies the result
-    before its rounding to bf16."""
+    before its rounding to the output dtype; the ``DT_ROUND_*`` bits round to x's dtype."""
     lib = load_library()
-    _require(x.is_cuda and x.dtype == torch.bfloat16 and x.dim() == 4 and x.stride(3) == 1, "x must be bf16 [B,S,H,D] on the GPU")
+    _require(x.is_cuda and x.dtype in HALF_DTYPES and x.dim() == 4 and x.stride(3) == 1, "x must be bf16 or fp16 [B,S,H,D] on the GPU")
     B, S, H, D = x.shape
     if out is None:
-        out = torch.empty((B, S, H, D), dtype=torch.bfloat16, device=x.device)
-    _require(out.is_cuda and out.dtype == torch.bfloat16 and out.is_contiguous() and tuple(out.shape) == (B, S, H, D),
-             "out must be a contiguous bf16 [B,S,H,D]")
+        out = torch.empty((B, S, H, D), dtype=x.dtype, device=x.device)
+    _require(out.is_cuda and out.dtype == x.dtype and out.is_contiguous() and tuple(out.shape) == (B, S, H, D),
+             "out must be a contiguous [B,S,H,D] in x's dtype")
+    rounding = int(rounding) | (DT_IO_FP16 if x.dtype == torch.float16 else 0)
     for name, t in (("weight", weight), ("bias", bias)):
         _require(t is None or (t.is_cuda and t.dtype == torch.float32 and t.is_contiguous() and t.numel() == D),
                  f"{name} must be fp32 [D] on the GPU")

@@ -150,13 +150,14 @@ _warned_cast = set()
 
 
 def _kernel_input(t: torch.Tensor) -> torch.Tensor:
-    """The kernels read bf16.  fp32 / fp16 inputs (flash_attn_func itself only takes fp16 / bf16; the
-    reference's CPU-runnable case is stated in fp32) are rounded to bf16 here, once, explicitly: the
-    result is then the attention of the ROUNDED inputs, which differs from fp32 attention of the
-    unrounded ones by the input rounding (2^-9 relative per element)."""
-    if t is None or t.dtype == torch.bfloat16:
+    """The kernels run in bf16 or fp16, the two dtypes flash_attn_func takes: such inputs pass as they are
+    (fp16 on the fp16 MFMA, states and cache slots in fp16).  fp32 inputs (the reference's CPU-runnable case
+    is stated in fp32) are rounded to bf16 here, once, explicitly: the result is then the attention of the
+    ROUNDED inputs, which differs from fp32 attention of the unrounded ones by the input rounding
+    (2^-9 relative per element)."""
+    if t is None or t.dtype in _hip.HALF_DTYPES:
         return t
-    if t.dtype not in (torch.float32, torch.float16):
+    if t.dtype != torch.float32:
         raise TypeError(f"attention inputs must be bf16, fp16 or fp32, got {t.dtype}")
     if t.dtype not in _warned_cast:
         _warned_cast.add(t.dtype)
@@ -218,7 +219,7 @@ class proAttention:
 
     @get_timer("oAttn")
     def attn(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor) -> Optional[torch.Tensor]:
-        """query ``[B,Sq,H,D]``, key/value ``[B,Sk,H,D]`` = this rank's shard (bf16).
+        """query ``[B,Sq,H,D]``, key/value ``[B,Sk,H,D]`` = this rank's shard (bf16 or fp16).
         Returns fp32 ``[B,Sq,H,D]`` (core/attention.py:74-237)."""
         rm = get_redundancy_map()
         self._exact_f32 = (not self.dry_run and self.fp32_inputs == "exact" and query is not None
@@ -355,7 +356,7 @@ class proAttention:
             if job.chunks in seen and job.store_slot is None:
                 states.append(seen[job.chunks])
                 continue
-            o = torch.empty((B, Sq, H, D), dtype=torch.bfloat16, device=dev)
+            o = torch.empty((B, Sq, H, D), dtype=query.dtype, device=dev)
             l = torch.empty((B, H, Sq), dtype=torch.float32, device=dev)
             if len(set(job.chunks)) > self._MAX_JOB_CHUNKS:
                 # a block of more chunks than one launch addresses (rings of 128 positions and more): its
@@ -424,7 +425,7 @@ class proAttention:
             k_c, v_c = (key, value) if use_local else self.group.kv_chunk(c)
             ks.append(_as4d(k_c, B))
             vs.append(_as4d(v_c, B))
-        if not cache.ensure_arena(C, B, Sq, H, D, query.device):
+        if not cache.ensure_arena(C, B, Sq, H, D, query.device, query.dtype):
             out = self._attn_uncached(query, ks, vs)
             rm.record_out_redundancy(timestep=t, layer_id=l, curr_out=out)
             return out
@@ -524,7 +525,7 @@ class proAttention:
             self.last_lse = torch.full((B, Sq, H, 1), float("-inf"), dtype=torch.float32, device=dev)
             return torch.zeros((B, Sq, H, D), dtype=self.out_dtype, device=dev)
         pieces = [ids[i:i + self._MAX_JOB_CHUNKS] for i in range(0, len(ids), self._MAX_JOB_CHUNKS)]
-        outs = [torch.empty((B, Sq, H, D), dtype=torch.bfloat16, device=dev) for _ in pieces]
+        outs = [torch.empty((B, Sq, H, D), dtype=query.dtype, device=dev) for _ in pieces]
         lses = [torch.empty((B, H, Sq), dtype=torch.float32, device=dev) for _ in pieces]
         q_ranges = kv_ranges = None
         jobs, d_out, d_lse = pieces, outs, lses

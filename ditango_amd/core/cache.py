@@ -155,11 +155,11 @@ class proCache:
 
     def store_block(self, block_id: int, out: torch.Tensor, lse: torch.Tensor) -> None:
         """Keep ``(out, lse)`` as block ``block_id``.  A state already in cache form
-        (contiguous bf16 ``out``, contiguous fp32 ``[B,H,S]`` ``lse`` -- what the
-        attention kernel writes) is adopted as is; anything else goes through one
-        ``dt_cache_store`` pass into fresh cache-form tensors."""
+        (contiguous bf16 or fp16 ``out``, contiguous fp32 ``[B,H,S]`` ``lse`` -- what the
+        attention kernel writes for a model that runs in that dtype) is adopted as is; anything
+        else goes through one ``dt_cache_store`` pass into fresh cache-form (bf16) tensors."""
         B, S, H, D = out.shape
-        in_cache_form = (out.dtype == torch.bfloat16 and out.is_contiguous() and lse.dtype == torch.float32
+        in_cache_form = (out.dtype in _hip.HALF_DTYPES and out.is_contiguous() and lse.dtype == torch.float32
                          and tuple(lse.shape) == (B, H, S) and lse.is_contiguous())
         if not in_cache_form:
             slot_out = torch.empty((B, S, H, D), dtype=torch.bfloat16, device=out.device)
@@ -191,14 +191,16 @@ class proCache:
         self.arena_refused = None
 
     # ---- mask-mode arena --------------------------------------------------------------------------
-    def ensure_arena(self, n_chunks: int, B: int, Sq: int, H: int, D: int, device) -> bool:
+    def ensure_arena(self, n_chunks: int, B: int, Sq: int, H: int, D: int, device,
+                     dtype: torch.dtype = torch.bfloat16) -> bool:
         """Make sure the mask-mode arena of this layer exists.  Returns False when it does not fit:
         the arena (``n_chunks + 1`` states) is only allocated if the current allocation plus its size
         stays under ``memory_constraint`` -- the same probe and budget as ``pass_memory_check``
         (cache.py:103-128) -- and a layer without arena recomputes every chunk on every call, which is
         what the reference's guard falls back to (core/attention.py:97-98: stride forced to N)."""
         shape = (n_chunks, B, Sq, H, D)
-        if self.arena_out is not None and tuple(self.arena_out.shape) == shape and self.arena_out.device == device:
+        if (self.arena_out is not None and tuple(self.arena_out.shape) == shape and self.arena_out.device == device
+                and self.arena_out.dtype == dtype):
             return True
         if self.arena_refused == shape:
             return False
@@ -211,9 +213,9 @@ class proCache:
             self.arena_refused = shape
             self.arena_valid = []
             return False
-        self.arena_out = torch.empty(shape, dtype=torch.bfloat16, device=device)
+        self.arena_out = torch.empty(shape, dtype=dtype, device=device)   # bf16, or fp16 for a model run in fp16
         self.arena_lse = torch.empty((n_chunks, B, H, Sq), dtype=torch.float32, device=device)
-        self.diag_out = torch.empty((B, Sq, H, D), dtype=torch.bfloat16, device=device)
+        self.diag_out = torch.empty((B, Sq, H, D), dtype=dtype, device=device)
         self.diag_lse = torch.empty((B, H, Sq), dtype=torch.float32, device=device)
         self.arena_valid = [False] * n_chunks
         return True

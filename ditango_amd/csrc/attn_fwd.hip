@@ -55,12 +55,43 @@
 
 namespace dt {
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// The 16-bit element type of q, K, V, P and the output states: bfloat16, or IEEE half (kHalf).  Loads, LDS
+// layout, swizzles and the transposing reads only see 16-bit elements; the type decides the MFMA and the
+// roundings of P and of the output.
+template <bool kHalf>
+struct Elem {
+  typedef __bf16 t;
+  typedef __bf16 x8 __attribute__((ext_vector_type(8)));
+  typedef __bf16 x4 __attribute__((ext_vector_type(4)));
+  typedef __bf16 x2 __attribute__((ext_vector_type(2)));
+  __device__ static __forceinline__ f32x16 mfma(x8 a, x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  // two packed elements of a 32-bit word, widened
+  __device__ static __forceinline__ f32x2 widen(uint32_t w) {
+    f32x2 f;
+    f.x = __builtin_bit_cast(float, w << 16);
+    f.y = __builtin_bit_cast(float, w & 0xffff0000u);
+    return f;
+  }
+};
+template <>
+struct Elem<true> {
+  typedef _Float16 t;
+  typedef _Float16 x8 __attribute__((ext_vector_type(8)));
+  typedef _Float16 x4 __attribute__((ext_vector_type(4)));
+  typedef _Float16 x2 __attribute__((ext_vector_type(2)));
+  __device__ static __forceinline__ f32x16 mfma(x8 a, x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  __device__ static __forceinline__ f32x2 widen(uint32_t w) {
+    return __builtin_convertvector(__builtin_bit_cast(x2, w), f32x2);
+  }
+};
 
 constexpr int kWaves = 8;
 constexpr int kThreads = kWaves * 64;
@@ -146,7 +177,10 @@ __device__ __forceinline__ void phase_barrier_after_matrix(V (&sa)[2], V (&oa)[N
 
 // A tile's per-lane sum of probabilities (32 of them) above which the tile is redone with an
 // exact row maximum.  Below it every probability is at most 2^12: harmless for the bf16
-// operand (same relative precision at any exponent) and for the fp32 accumulators.
+// operand (same relative precision at any exponent), inside the range of the fp16 operand (largest
+// finite value 65504; the reference never exceeds the row's true maximum, so a probability is at least its
+// true softmax weight and loses no more to fp16's small end than under an exact maximum) and for the fp32
+// accumulators.
 constexpr float kSumLimit = 4096.0f;
 // The same for queries that come with softmax_scale * log2(e) folded in (kPre): rows keep the
 // reference 0 while the maximum of their first tile lies in [kBandLo, kBandHi] (powers of two;
@@ -236,9 +270,15 @@ __device__ __forceinline__ void load_block_to_lds(u32x4 rsrc, uint32_t lane_off,
 #ifndef DT_D64_WAVES
 #define DT_D64_WAVES 4
 #endif
-template <int D, bool kPre>
+template <int D, bool kPre, bool kHalf>
 __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd_kernel(const AttnArgs args_by_value) {
   using T = Tile<D>;
+  using E = Elem<kHalf>;
+  typedef typename E::t elem_t;
+  typedef typename E::x8 ex8;
+  typedef typename E::x4 ex4;
+  typedef typename E::x2 ex2;
+  static_assert(!(kPre && kHalf), "the prescaled softmax keeps probabilities up to 2^40: bf16 only");
   // The arguments are read where they arrive: in the kernarg segment (constant address space, scalar loads),
   // through its base pointer -- AttnArgs is the kernel's only parameter, so it sits at offset 0.  Going through the
   // by-value parameter instead leaves it to the optimiser to prove that its private copy of the 3.6 KB struct is
@@ -276,7 +316,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
 
   int seg_begin, seg_end, single = -1;
   int q_begin = 0, q_end = a.Sq;   // query rows of this job
-  __bf16* out_ptr;
+  uint16_t* out_ptr;
   float* lse_ptr;
   int vseg = -1;  // segment of a packed variable-length batch (device-listed jobs only)
   int dseg = -1;  // segment whose boundaries are read from device memory (a.cu_q != nullptr)
@@ -360,13 +400,13 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
   const int q0 = q_begin + qt * kBQ + wave * 32;
 
   // ---- Q fragments: B operand of S^T = K Q^T, kept in registers ----------------------
-  bf16x8 qf[D / 16];
+  ex8 qf[D / 16];
   {
     int qrow = q0 + col;
     if (qrow > q_end - 1) qrow = q_end - 1;
-    const __bf16* qp = a.q + (int64_t)b * a.q_sb + (int64_t)qrow * a.q_ss + (int64_t)h * a.q_sh + 8 * hh;
+    const uint16_t* qp = a.q + (int64_t)b * a.q_sb + (int64_t)qrow * a.q_ss + (int64_t)h * a.q_sh + 8 * hh;
 #pragma unroll
-    for (int s = 0; s < D / 16; ++s) qf[s] = *reinterpret_cast<const bf16x8*>(qp + 16 * s);
+    for (int s = 0; s < D / 16; ++s) qf[s] = *reinterpret_cast<const ex8*>(qp + 16 * s);
   }
   // Route the fragments through an empty asm: they are then defined by it, not by loads.  The
   // compiler otherwise keeps "Q may still be in flight" alive round the loop and waits for ALL
@@ -532,7 +572,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
   }
 
   f32x16 s_acc[2];       // S^T of the tile whose softmax comes next
-  bf16x8 p_frag[2][2];   // P^T of the tile whose P V product comes next
+  ex8 p_frag[2][2];      // P^T of the tile whose P V product comes next
   int cp_valid = 0;      // keys that exist in the tile held in s_acc
 
   // S^T = K Q^T for tile 0 only (first matrix phase)
@@ -543,8 +583,8 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
       for (int r = 0; r < 16; ++r) s_acc[kb][r] = 0.f;
 #pragma unroll
       for (int s = 0; s < D / 16; ++s) {
-        const bf16x8 ka = *reinterpret_cast<const bf16x8*>(lds + kld[s] + kb * 32 * T::kRowBytes);
-        s_acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[s], s_acc[kb], 0, 0, 0);
+        const ex8 ka = *reinterpret_cast<const ex8*>(lds + kld[s] + kb * 32 * T::kRowBytes);
+        s_acc[kb] = E::mfma(ka, qf[s], s_acc[kb]);
       }
     }
   };
@@ -573,15 +613,15 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
   // fragments (V fragments of a tile completed at least a phase ago) are read at the END of the
   // preceding vector phase, so their LDS latency passes while the wavefront waits at the barrier
   // instead of in front of the first MFMA.
-  bf16x8 ring[kRing];
-  auto v_frag = [&](int vbuf, int i) __attribute__((always_inline)) -> bf16x8 {
+  ex8 ring[kRing];
+  auto v_frag = [&](int vbuf, int i) __attribute__((always_inline)) -> ex8 {
     // 8 consecutive keys of one d column = two transposing reads of 4 keys each
     const int db = i % (D / 32), kb = (i / (D / 32)) >> 1, half = (i / (D / 32)) & 1;
     const uint8_t* p = lds + vld[db] + vbuf * T::kBytesV + (32 * kb + 16 * half) * T::kRowBytes;
     const s16x4 lo = lds_read_tr(p);
     const s16x4 hi = lds_read_tr(p + 4 * T::kRowBytes);
     const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    return __builtin_bit_cast(bf16x8, both);
+    return __builtin_bit_cast(ex8, both);
   };
   auto ring_prefill = [&](auto u_tag) __attribute__((always_inline)) {
     constexpr int kU = decltype(u_tag)::value;
@@ -591,19 +631,19 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
   auto matrix_phase = [&](auto u_tag) __attribute__((always_inline)) {
     constexpr int kU = decltype(u_tag)::value;         // V buffer of this tile
     constexpr int kUK = (kU + 1) & (kNumBuf - 1);      // K buffer of the next tile
-    auto frag = [&](int i) -> bf16x8 {
+    auto frag = [&](int i) -> ex8 {
       if (i < kPV) return v_frag(kU, i);
       const int j = i - kPV;
       const int kb = j & 1, sidx = j >> 1;
-      return *reinterpret_cast<const bf16x8*>(lds + kld[sidx] + kUK * T::kBytesK + kb * 32 * T::kRowBytes);
+      return *reinterpret_cast<const ex8*>(lds + kld[sidx] + kUK * T::kBytesK + kb * 32 * T::kRowBytes);
     };
 #pragma unroll
     for (int i = 0; i < kFrags; ++i) {
-      const bf16x8 cur = ring[i % kRing];
+      const ex8 cur = ring[i % kRing];
       if (i + kRing < kFrags) ring[i % kRing] = frag(i + kRing);
       if (i < kPV) {
         const int db = i % (D / 32), kb = (i / (D / 32)) >> 1, half = (i / (D / 32)) & 1;
-        o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur, p_frag[kb][half], o_acc[db], 0, 0, 0);
+        o_acc[db] = E::mfma(cur, p_frag[kb][half], o_acc[db]);
       } else {
         const int j = i - kPV;
         const int kb = j & 1, sidx = j >> 1;
@@ -611,9 +651,9 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
           f32x16 zero;
 #pragma unroll
           for (int r = 0; r < 16; ++r) zero[r] = 0.f;
-          s_acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur, qf[sidx], zero, 0, 0, 0);
+          s_acc[kb] = E::mfma(cur, qf[sidx], zero);
         } else {
-          s_acc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cur, qf[sidx], s_acc[kb], 0, 0, 0);
+          s_acc[kb] = E::mfma(cur, qf[sidx], s_acc[kb]);
         }
       }
     }
@@ -745,7 +785,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
           rs0 += p.x;
           rs1 += p.y;
         }
-        const bf16x2 pb = __builtin_convertvector(p, bf16x2);
+        const ex2 pb = __builtin_convertvector(p, ex2);
         p_frag[kb][r >> 3][r & 7] = pb.x;
         p_frag[kb][r >> 3][(r & 7) + 1] = pb.y;
       }
@@ -791,7 +831,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
           p.y = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[kb][r + 1], c, -mc));
           rs0 += p.x;
           rs1 += p.y;
-          const bf16x2 pb = __builtin_convertvector(p, bf16x2);
+          const ex2 pb = __builtin_convertvector(p, ex2);
           p_frag[kb][r >> 3][r & 7] = pb.x;
           p_frag[kb][r >> 3][(r & 7) + 1] = pb.y;
         }
@@ -842,7 +882,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
     lse_ptr[((int64_t)b * a.H + h) * a.Sq + qrow] = lse;
   }
 
-  // O^T (registers, [d][query]) -> LDS [query][d] bf16 -> coalesced 16-byte stores.
+  // O^T (registers, [d][query]) -> LDS [query][d] in the element type -> coalesced 16-byte stores.
   phase_barrier();  // every wavefront is done with the tile buffers
   uint8_t* ol = lds + wave * (32 * T::kPitchO);
 #pragma unroll
@@ -854,12 +894,12 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
       lo.y = o_acc[db][4 * g + 1] * inv;
       hi.x = o_acc[db][4 * g + 2] * inv;
       hi.y = o_acc[db][4 * g + 3] * inv;
-      const bf16x2 l2 = __builtin_convertvector(lo, bf16x2);
-      const bf16x2 h2 = __builtin_convertvector(hi, bf16x2);
-      bf16x4 pk;
+      const ex2 l2 = __builtin_convertvector(lo, ex2);
+      const ex2 h2 = __builtin_convertvector(hi, ex2);
+      ex4 pk;
       pk.x = l2.x; pk.y = l2.y; pk.z = h2.x; pk.w = h2.y;
       const int d = 32 * db + 8 * g + 4 * hh;
-      *reinterpret_cast<bf16x4*>(ol + col * T::kPitchO + d * 2) = pk;
+      *reinterpret_cast<ex4*>(ol + col * T::kPitchO + d * 2) = pk;
     }
   phase_barrier();
   constexpr int kLanesPerRow = D / 8;
@@ -872,10 +912,10 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
     const int qg = q0 + row;
     const u32x4 val = *reinterpret_cast<const u32x4*>(ol + row * T::kPitchO + cc * 16);
     if (is_part) {
-      __bf16* dst = a.ws_out + (ws_slot * kBQ + wave * 32 + row) * D + cc * 8;
+      uint16_t* dst = a.ws_out + (ws_slot * kBQ + wave * 32 + row) * D + cc * 8;
       *reinterpret_cast<u32x4*>(dst) = val;
     } else if (qg < q_end) {
-      __bf16* dst = out_ptr + (((int64_t)b * a.Sq + qg) * a.H + h) * D + cc * 8;
+      uint16_t* dst = out_ptr + (((int64_t)b * a.Sq + qg) * a.H + h) * D + cc * 8;
       __builtin_nontemporal_store(val, reinterpret_cast<u32x4*>(dst));
     }
   }
@@ -883,8 +923,9 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
 
 // Folds the part_ways partial states of every tail item into the item's rows of its destination.
 // One workgroup per item and slice of 256 / (D/8) rows; a group of D/8 lanes owns a row.
-template <int D>
+template <int D, bool kHalf>
 __global__ __launch_bounds__(256) void attn_tail_fold_kernel(const AttnArgs a) {
+  using E = Elem<kHalf>;
   constexpr int kSlices = kBQ / (256 / (D / 8));
   const int slot_id = blockIdx.x / kSlices;
   const int slice = blockIdx.x - slot_id * kSlices;
@@ -898,7 +939,7 @@ __global__ __launch_bounds__(256) void attn_tail_fold_kernel(const AttnArgs a) {
   const int b = bh / a.H;
   const int h = bh - b * a.H;
   const int job = a.tail_job;
-  __bf16* out_ptr;
+  uint16_t* out_ptr;
   float* lse_ptr;
   if (a.dev_ids != nullptr) {
     if (job >= *a.dev_count) return;
@@ -931,8 +972,9 @@ __global__ __launch_bounds__(256) void attn_tail_fold_kernel(const AttnArgs a) {
         den += w;
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-          acc[2 * k] = __builtin_fmaf(w, __builtin_bit_cast(float, e[k] << 16), acc[2 * k]);
-          acc[2 * k + 1] = __builtin_fmaf(w, __builtin_bit_cast(float, e[k] & 0xffff0000u), acc[2 * k + 1]);
+          const f32x2 x = E::widen(e[k]);
+          acc[2 * k] = __builtin_fmaf(w, x.x, acc[2 * k]);
+          acc[2 * k + 1] = __builtin_fmaf(w, x.y, acc[2 * k + 1]);
         }
       }
     }
@@ -944,7 +986,7 @@ __global__ __launch_bounds__(256) void attn_tail_fold_kernel(const AttnArgs a) {
       f32x2 f;
       f.x = acc[2 * k] * inv;
       f.y = acc[2 * k + 1] * inv;
-      pk[k] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+      pk[k] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, typename E::x2));
     }
     o.x = pk[0]; o.y = pk[1]; o.z = pk[2]; o.w = pk[3];
     *reinterpret_cast<u32x4*>(out_ptr + (((int64_t)b * a.Sq + qg) * a.H + h) * D + cc * 8) = o;
@@ -955,30 +997,34 @@ __global__ __launch_bounds__(256) void attn_tail_fold_kernel(const AttnArgs a) {
 static_assert(Tile<128>::kLdsBytes == kAttnLdsBytes128 && Tile<64>::kLdsBytes == kAttnLdsBytes64,
               "dt_common.h states the LDS footprint of the attention kernel");
 
-template <int D, bool kPre>
+template <int D, bool kPre, bool kHalf>
 static int launch_one(const AttnArgs& a, dim3 grid, hipStream_t stream) {
   // more than 64 KB of dynamic LDS has to be allowed once per kernel and device
   static thread_local int allowed_dev = -1;
   int dev = 0;
   if (int rc = hip_fail(hipGetDevice(&dev), "hipGetDevice")) return rc;
   if (allowed_dev != dev) {
-    if (int rc = hip_fail(hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_fwd_kernel<D, kPre>),
+    if (int rc = hip_fail(hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_fwd_kernel<D, kPre, kHalf>),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, Tile<D>::kLdsBytes),
                           "hipFuncSetAttribute"))
       return rc;
     allowed_dev = dev;
   }
-  hipLaunchKernelGGL((attn_fwd_kernel<D, kPre>), grid, dim3(kThreads), Tile<D>::kLdsBytes, stream, a);
+  hipLaunchKernelGGL((attn_fwd_kernel<D, kPre, kHalf>), grid, dim3(kThreads), Tile<D>::kLdsBytes, stream, a);
   return hip_fail(hipGetLastError(), "attn_fwd launch");
 }
 
 static int launch_dim(const AttnArgs& a, int D, dim3 grid, hipStream_t stream) {
-  if (a.q_prescaled) {
-    if (D == 128) return launch_one<128, true>(a, grid, stream);
-    return launch_one<64, true>(a, grid, stream);
+  if (a.elem_f16) {
+    if (D == 128) return launch_one<128, false, true>(a, grid, stream);
+    return launch_one<64, false, true>(a, grid, stream);
   }
-  if (D == 128) return launch_one<128, false>(a, grid, stream);
-  return launch_one<64, false>(a, grid, stream);
+  if (a.q_prescaled) {
+    if (D == 128) return launch_one<128, true, false>(a, grid, stream);
+    return launch_one<64, true, false>(a, grid, stream);
+  }
+  if (D == 128) return launch_one<128, false, false>(a, grid, stream);
+  return launch_one<64, false, false>(a, grid, stream);
 }
 
 // Number of CUs of the current device (one workgroup of the attention kernel per CU at a time).
@@ -1032,6 +1078,10 @@ int launch_attn(const AttnArgs& a_in, int D, int n_jobs, hipStream_t stream, voi
   if (n_jobs <= 0 || a_in.total <= 0) return DT_OK;
   if (D != 128 && D != 64) {
     set_error("head dim %d not built (64 and 128 are)", D);
+    return DT_ERR_UNSUPPORTED;
+  }
+  if (a_in.elem_f16 && a_in.q_prescaled) {
+    set_error("fp16 tensors and a prescaled q do not combine (the prescaled softmax keeps probabilities beyond fp16's range)");
     return DT_ERR_UNSUPPORTED;
   }
   AttnArgs a = a_in;
@@ -1089,15 +1139,18 @@ int launch_attn(const AttnArgs& a_in, int D, int n_jobs, hipStream_t stream, voi
   a.tail_idx0 = a.per_xcd - tail / kXcds;
   a.tail_items = tail / kXcds;
   a.part_ways = ways;
-  a.ws_out = static_cast<__bf16*>(workspace);
+  a.ws_out = static_cast<uint16_t*>(workspace);
   a.ws_lse = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + (int64_t)tail * ways * kBQ * D * 2);
   // parts per XCD lane of the grid: tail / 8 items x ways parts, spread over extra planes of per_xcd entries
   const int part_planes = (a.tail_items * ways + a.per_xcd - 1) / a.per_xcd;
   if (int rc = launch_dim(a, D, dim3((unsigned)slots_per_job, (unsigned)(n_jobs + part_planes), 1), stream)) return rc;
-  if (D == 128)
-    hipLaunchKernelGGL(attn_tail_fold_kernel<128>, dim3((unsigned)tail * 16), dim3(256), 0, stream, a);
-  else
-    hipLaunchKernelGGL(attn_tail_fold_kernel<64>, dim3((unsigned)tail * 8), dim3(256), 0, stream, a);
+  if (D == 128) {
+    if (a.elem_f16) hipLaunchKernelGGL((attn_tail_fold_kernel<128, true>), dim3((unsigned)tail * 16), dim3(256), 0, stream, a);
+    else hipLaunchKernelGGL((attn_tail_fold_kernel<128, false>), dim3((unsigned)tail * 16), dim3(256), 0, stream, a);
+  } else {
+    if (a.elem_f16) hipLaunchKernelGGL((attn_tail_fold_kernel<64, true>), dim3((unsigned)tail * 8), dim3(256), 0, stream, a);
+    else hipLaunchKernelGGL((attn_tail_fold_kernel<64, false>), dim3((unsigned)tail * 8), dim3(256), 0, stream, a);
+  }
   return hip_fail(hipGetLastError(), "attn tail fold launch");
 }
 

@@ -61,7 +61,7 @@ static int fill_common(AttnArgs& a, const void* q, int32_t B, int32_t Sq, int32_
     set_error("k/v token and head strides must be multiples of 8 elements");
     return DT_ERR_INVALID;
   }
-  a.q = static_cast<const __bf16*>(q);
+  a.q = static_cast<const uint16_t*>(q);
   a.q_sb = q_sb; a.q_ss = q_ss; a.q_sh = q_sh;
   a.B = B; a.H = H; a.Sq = Sq;
   a.nqt = (Sq + 255) / 256;  // 256 queries per workgroup
@@ -87,8 +87,8 @@ static int fill_common(AttnArgs& a, const void* q, int32_t B, int32_t Sq, int32_
       set_error("chunk %d: one (batch, head) plane spans 2 GiB or more; split the chunk", i);
       return DT_ERR_INVALID;
     }
-    a.k[i] = static_cast<const __bf16*>(k_ptrs[i]);
-    a.v[i] = static_cast<const __bf16*>(v_ptrs[i]);
+    a.k[i] = static_cast<const uint16_t*>(k_ptrs[i]);
+    a.v[i] = static_cast<const uint16_t*>(v_ptrs[i]);
     a.kv_len[i] = kv_lens[i];
     a.kv_sb[i] = kv_sb[i];
   }
@@ -109,11 +109,16 @@ static int check_workspace(const void* workspace, int64_t workspace_bytes) {
 }
 
 static int apply_flags(AttnArgs& a, int32_t flags) {
-  if (flags & ~DT_ATTN_Q_PRESCALED) {
+  if (flags & ~(DT_ATTN_Q_PRESCALED | DT_ATTN_FP16)) {
     set_error("unknown attention flags 0x%x", (unsigned)flags);
     return DT_ERR_INVALID;
   }
+  if ((flags & DT_ATTN_Q_PRESCALED) && (flags & DT_ATTN_FP16)) {
+    set_error("DT_ATTN_Q_PRESCALED and DT_ATTN_FP16 do not combine (the prescaled softmax keeps probabilities beyond fp16's range)");
+    return DT_ERR_UNSUPPORTED;
+  }
   a.q_prescaled = (flags & DT_ATTN_Q_PRESCALED) ? 1 : 0;
+  a.elem_f16 = (flags & DT_ATTN_FP16) ? 1 : 0;
   return DT_OK;
 }
 
@@ -155,7 +160,7 @@ extern "C" int dt_attn_seg_jobs_ws_fwd(const void* q, int32_t B, int32_t Sq, int
       set_error("job %d: null or misaligned destination", j);
       return DT_ERR_INVALID;
     }
-    a.job_out[j] = static_cast<__bf16*>(out_ptrs[j]);
+    a.job_out[j] = static_cast<uint16_t*>(out_ptrs[j]);
     a.job_lse[j] = lse_ptrs[j];
     a.job_begin[j] = job_begin[j];
     const int32_t qb = job_q_begin ? job_q_begin[j] : 0;
@@ -262,7 +267,7 @@ extern "C" int dt_attn_varlen_jobs_fwd(const void* q, int32_t B, int32_t Sq, int
       set_error("job %d: segment %d outside 0..%d", j, job_segment[j], n_seg - 1);
       return DT_ERR_INVALID;
     }
-    a.job_out[j] = static_cast<__bf16*>(out_ptrs[j]);
+    a.job_out[j] = static_cast<uint16_t*>(out_ptrs[j]);
     a.job_lse[j] = lse_ptrs[j];
     a.job_begin[j] = job_begin[j];
     a.job_q_begin[j] = job_segment[j];   // with device boundaries this field names the segment
@@ -334,9 +339,9 @@ extern "C" int dt_attn_jobs_fwd(const void* q, int32_t B, int32_t Sq, int32_t H,
                               softmax_scale, stream);
 }
 
-extern "C" int dt_attn_chunk_fwd(const void* q, const void* k, const void* v, void* out, float* lse, int32_t B,
-                                 int32_t Sq, int32_t Sk, int32_t H, int32_t D, int64_t q_sb, int64_t q_ss, int64_t q_sh,
-                                 int64_t kv_sb, int64_t kv_ss, int64_t kv_sh, float softmax_scale, void* stream) {
+static int chunk_fwd(const void* q, const void* k, const void* v, void* out, float* lse, int32_t B, int32_t Sq, int32_t Sk,
+                     int32_t H, int32_t D, int64_t q_sb, int64_t q_ss, int64_t q_sh, int64_t kv_sb, int64_t kv_ss,
+                     int64_t kv_sh, float softmax_scale, int32_t flags, void* stream) {
   const void* kp[1] = {k};
   const void* vp[1] = {v};
   const int32_t lens[1] = {Sk};
@@ -345,8 +350,22 @@ extern "C" int dt_attn_chunk_fwd(const void* q, const void* k, const void* v, vo
   const int32_t chunks[1] = {0};
   void* outs[1] = {out};
   float* lses[1] = {lse};
-  return dt_attn_jobs_fwd(q, B, Sq, H, D, q_sb, q_ss, q_sh, 1, kp, vp, lens, sbs, kv_ss, kv_sh, 1, begin, chunks, outs,
-                          lses, softmax_scale, stream);
+  return dt_attn_seg_jobs_ws_fwd(q, B, Sq, H, D, q_sb, q_ss, q_sh, 1, kp, vp, lens, sbs, kv_ss, kv_sh, 1, begin, chunks,
+                                 nullptr, nullptr, nullptr, nullptr, outs, lses, softmax_scale, flags, nullptr, 0, stream);
+}
+
+extern "C" int dt_attn_chunk_fwd(const void* q, const void* k, const void* v, void* out, float* lse, int32_t B,
+                                 int32_t Sq, int32_t Sk, int32_t H, int32_t D, int64_t q_sb, int64_t q_ss, int64_t q_sh,
+                                 int64_t kv_sb, int64_t kv_ss, int64_t kv_sh, float softmax_scale, void* stream) {
+  return chunk_fwd(q, k, v, out, lse, B, Sq, Sk, H, D, q_sb, q_ss, q_sh, kv_sb, kv_ss, kv_sh, softmax_scale, 0, stream);
+}
+
+extern "C" int dt_attn_chunk_f16_fwd(const void* q, const void* k, const void* v, void* out, float* lse, int32_t B,
+                                     int32_t Sq, int32_t Sk, int32_t H, int32_t D, int64_t q_sb, int64_t q_ss,
+                                     int64_t q_sh, int64_t kv_sb, int64_t kv_ss, int64_t kv_sh, float softmax_scale,
+                                     void* stream) {
+  return chunk_fwd(q, k, v, out, lse, B, Sq, Sk, H, D, q_sb, q_ss, q_sh, kv_sb, kv_ss, kv_sh, softmax_scale, DT_ATTN_FP16,
+                   stream);
 }
 
 // Checks and fields every device-scheduled launch shares.
@@ -374,12 +393,12 @@ static int fill_sched(AttnArgs& a, int32_t n_chunks, const void* const* k_ptrs, 
   }
   a.dev_ids = dev_compute_ids;
   a.dev_count = dev_count;
-  a.slot_out = static_cast<__bf16*>(slot_out);
+  a.slot_out = static_cast<uint16_t*>(slot_out);
   a.slot_lse = slot_lse;
   a.slot_out_stride = slot_out_stride;
   a.slot_lse_stride = slot_lse_stride;
   a.diag = diag;
-  a.diag_out = static_cast<__bf16*>(diag_out);
+  a.diag_out = static_cast<uint16_t*>(diag_out);
   a.diag_lse = diag_lse;
   return DT_OK;
 }

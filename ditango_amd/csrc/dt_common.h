@@ -13,7 +13,8 @@ int hip_fail(hipError_t e, const char* what);
 // chunk and job tables travel in the kernarg segment: no device-side table,
 // no host-to-device copy per call.
 struct AttnArgs {
-  const __bf16* q;
+  // q, K, V and the output states are 16-bit elements: bfloat16, or IEEE half when elem_f16 is set
+  const uint16_t* q;
   int64_t q_sb, q_ss, q_sh;
   int32_t B, H, Sq;
   int32_t nqt;        // query tiles per (batch, head)
@@ -21,15 +22,16 @@ struct AttnArgs {
   int32_t per_xcd;    // work items handed to each of the 8 XCDs
   float scale_log2;   // softmax scale * log2(e)
   int32_t q_prescaled;  // the caller folded scale_log2 into q: scores are already in log2 units
+  int32_t elem_f16;     // the 16-bit tensors are IEEE half instead of bfloat16
   // chunk table
   int32_t n_chunks;
-  const __bf16* k[DT_MAX_CHUNKS];
-  const __bf16* v[DT_MAX_CHUNKS];
+  const uint16_t* k[DT_MAX_CHUNKS];
+  const uint16_t* v[DT_MAX_CHUNKS];
   int64_t kv_sb[DT_MAX_CHUNKS];
   int32_t kv_len[DT_MAX_CHUNKS];
   int64_t kv_ss, kv_sh;
   // host-listed jobs
-  __bf16* job_out[DT_MAX_JOBS];
+  uint16_t* job_out[DT_MAX_JOBS];
   float* job_lse[DT_MAX_JOBS];
   int32_t job_begin[DT_MAX_JOBS + 1];
   int32_t job_chunks[DT_MAX_JOB_ENTRIES];
@@ -42,11 +44,11 @@ struct AttnArgs {
   // device-listed jobs (dev_ids != nullptr): job j computes chunk dev_ids[j] if j < *dev_count
   const int32_t* dev_ids;
   const int32_t* dev_count;
-  __bf16* slot_out;
+  uint16_t* slot_out;
   float* slot_lse;
   int64_t slot_out_stride, slot_lse_stride;
   int32_t diag;
-  __bf16* diag_out;
+  uint16_t* diag_out;
   float* diag_lse;
   // device-listed jobs on a packed variable-length batch (n_seg > 0): launch job j is segment
   // j % n_seg of the chunk listed at j / n_seg; the keys of segment s inside chunk c are
@@ -73,7 +75,7 @@ struct AttnArgs {
   int32_t tail_idx0;
   int32_t tail_items;  // tail items per XCD lane of the grid (= tail workgroup slots / 8)
   int32_t part_ways;
-  __bf16* ws_out;   // [slot][256 queries][D]
+  uint16_t* ws_out;   // [slot][256 queries][D]
   float* ws_lse;    // [slot][256]
 };
 

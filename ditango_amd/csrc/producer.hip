@@ -1,5 +1,5 @@
 // Producer side of an attention call: per-head QK normalisation and rotary position
-// embedding in one pass over HBM, written as the bf16 [B,S,H,D] tensor the attention
+// embedding in one pass over HBM, written as the bf16 (or fp16) [B,S,H,D] tensor the attention
 // kernel reads.  Replaces the chains of eager ops in front of the attention call at
 // executor/cogvideox/attention_processor.py:55-71 (LayerNorm over D, interleaved RoPE on the
 // video tokens only), executor/hunyuanvideo/hunyuan_transformer.py:177-191 (RMSNorm over D,
@@ -17,20 +17,21 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kThreads = 256;
 constexpr int kHeads = 8;  // heads of one token handled by a lane group with one set of table loads
 
 struct PrepArgs {
-  const __bf16* x;
-  __bf16* y;
+  const uint16_t* x;   // bfloat16, or IEEE half (DT_IO_FP16)
+  uint16_t* y;
   int64_t xs_b, xs_s, xs_h;
   int32_t B, S, H;
   int32_t norm, rope, rounding;
   const float* w;
   const float* bias;
   float eps;
-  float out_scale;  // multiplies the result before its rounding to bf16
+  float out_scale;  // multiplies the result before its rounding to the output type
   const float* cos;
   const float* sin;
   int64_t tab_sb;
@@ -38,22 +39,36 @@ struct PrepArgs {
   int32_t sec_end[3];  // rotate-half sections [0,e0) [e0,e1) [e1,D); unused ones end at D
 };
 
-__device__ __forceinline__ float bf16r(float v) { return (float)(__bf16)v; }
+// kHalf: the 16-bit type is IEEE half, else bfloat16
+template <bool kHalf>
+__device__ __forceinline__ float round16(float v) {
+  if constexpr (kHalf) return (float)(_Float16)v;
+  else return (float)(__bf16)v;
+}
 
+template <bool kHalf>
 __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
   f32x2 f;
   f.x = lo;
   f.y = hi;
-  const bf16x2 b = __builtin_convertvector(f, bf16x2);  // round to nearest even
-  return __builtin_bit_cast(uint32_t, b);
+  // round to nearest even
+  if constexpr (kHalf) return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, f16x2));
+  else return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
 }
 
+template <bool kHalf>
 __device__ __forceinline__ void unpack8(const u32x4 r, float (&v)[8]) {
   const uint32_t u[4] = {r.x, r.y, r.z, r.w};
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    v[2 * i] = __builtin_bit_cast(float, u[i] << 16);
-    v[2 * i + 1] = __builtin_bit_cast(float, u[i] & 0xffff0000u);
+    if constexpr (kHalf) {
+      const f32x2 f = __builtin_convertvector(__builtin_bit_cast(f16x2, u[i]), f32x2);
+      v[2 * i] = f.x;
+      v[2 * i + 1] = f.y;
+    } else {
+      v[2 * i] = __builtin_bit_cast(float, u[i] << 16);
+      v[2 * i + 1] = __builtin_bit_cast(float, u[i] & 0xffff0000u);
+    }
   }
 }
 
@@ -66,7 +81,7 @@ __device__ __forceinline__ float group_sum(float v) {
 
 // One lane group of D/8 lanes handles up to kHeads heads of one token; a lane owns the
 // 8 consecutive elements [8c, 8c+8) of each of those rows.
-template <int D>
+template <int D, bool kHalf>
 __global__ __launch_bounds__(kThreads) void qk_norm_rope_kernel(const PrepArgs a) {
   constexpr int G = D / 8;
   const int c = threadIdx.x % G;
@@ -82,7 +97,7 @@ __global__ __launch_bounds__(kThreads) void qk_norm_rope_kernel(const PrepArgs a
   const int nh = (a.H - h0 < kHeads) ? a.H - h0 : kHeads;
   const int d0 = 8 * c;
 
-  const __bf16* xp = a.x + (int64_t)b * a.xs_b + (int64_t)s * a.xs_s + (int64_t)h0 * a.xs_h + d0;
+  const uint16_t* xp = a.x + (int64_t)b * a.xs_b + (int64_t)s * a.xs_s + (int64_t)h0 * a.xs_h + d0;
   u32x4 raw[kHeads];
 #pragma unroll
   for (int r = 0; r < kHeads; ++r)
@@ -136,12 +151,12 @@ __global__ __launch_bounds__(kThreads) void qk_norm_rope_kernel(const PrepArgs a
   const bool round_norm = (a.rounding & DT_ROUND_NORM_BF16) != 0;
   const bool round_rope = (a.rounding & DT_ROUND_ROPE_BF16) != 0;
 
-  __bf16* yp = a.y + (((int64_t)b * a.S + s) * a.H + h0) * D + d0;
+  uint16_t* yp = a.y + (((int64_t)b * a.S + s) * a.H + h0) * D + d0;
 #pragma unroll
   for (int r = 0; r < kHeads; ++r) {
     if (r >= nh) break;
     float v[8];
-    unpack8(raw[r], v);
+    unpack8<kHalf>(raw[r], v);
     if (a.norm == DT_NORM_RMS) {
       float ss = 0.0f;
 #pragma unroll
@@ -151,9 +166,9 @@ __global__ __launch_bounds__(kThreads) void qk_norm_rope_kernel(const PrepArgs a
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         float t = v[i] * rs;
-        if (round_norm) t = bf16r(t);
+        if (round_norm) t = round16<kHalf>(t);
         t *= w[i];
-        if (round_norm) t = bf16r(t);
+        if (round_norm) t = round16<kHalf>(t);
         v[i] = t;
       }
     } else if (a.norm == DT_NORM_LAYER) {
@@ -172,7 +187,7 @@ __global__ __launch_bounds__(kThreads) void qk_norm_rope_kernel(const PrepArgs a
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         float t = v[i] * rs * w[i] + bias[i];
-        if (round_norm) t = bf16r(t);
+        if (round_norm) t = round16<kHalf>(t);
         v[i] = t;
       }
     }
@@ -192,7 +207,7 @@ __global__ __launch_bounds__(kThreads) void qk_norm_rope_kernel(const PrepArgs a
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
           if (round_rope)
-            v[i] = bf16r(v[i] * cs[i]) + bf16r(rot[i] * sn[i]);
+            v[i] = round16<kHalf>(v[i] * cs[i]) + round16<kHalf>(rot[i] * sn[i]);
           else
             v[i] = v[i] * cs[i] + rot[i] * sn[i];
         }
@@ -203,10 +218,10 @@ __global__ __launch_bounds__(kThreads) void qk_norm_rope_kernel(const PrepArgs a
       for (int i = 0; i < 8; ++i) v[i] *= a.out_scale;
     }
     u32x4 o;
-    o.x = pack2(v[0], v[1]);
-    o.y = pack2(v[2], v[3]);
-    o.z = pack2(v[4], v[5]);
-    o.w = pack2(v[6], v[7]);
+    o.x = pack2<kHalf>(v[0], v[1]);
+    o.y = pack2<kHalf>(v[2], v[3]);
+    o.z = pack2<kHalf>(v[4], v[5]);
+    o.w = pack2<kHalf>(v[6], v[7]);
     __builtin_nontemporal_store(o, reinterpret_cast<u32x4*>(yp + (int64_t)r * D));
   }
 }
@@ -237,7 +252,7 @@ extern "C" int dt_qk_norm_rope(const void* x, int64_t x_stride_b, int64_t x_stri
     return DT_ERR_INVALID;
   }
   if (norm < DT_NORM_NONE || norm > DT_NORM_LAYER || rope < DT_ROPE_NONE || rope > DT_ROPE_HALVES ||
-      (rounding & ~(DT_ROUND_NORM_BF16 | DT_ROUND_ROPE_BF16))) {
+      (rounding & ~(DT_ROUND_NORM_BF16 | DT_ROUND_ROPE_BF16 | DT_IO_FP16))) {
     set_error("bad norm / rope / rounding code (%d, %d, %d)", norm, rope, rounding);
     return DT_ERR_INVALID;
   }
@@ -250,11 +265,12 @@ extern "C" int dt_qk_norm_rope(const void* x, int64_t x_stride_b, int64_t x_stri
     return DT_ERR_INVALID;
   }
   PrepArgs a{};
-  a.x = static_cast<const __bf16*>(x);
-  a.y = static_cast<__bf16*>(y);
+  a.x = static_cast<const uint16_t*>(x);
+  a.y = static_cast<uint16_t*>(y);
   a.xs_b = x_stride_b; a.xs_s = x_stride_s; a.xs_h = x_stride_h;
   a.B = B; a.S = S; a.H = H;
-  a.norm = norm; a.rope = rope; a.rounding = rounding;
+  a.norm = norm; a.rope = rope; a.rounding = rounding & (DT_ROUND_NORM_BF16 | DT_ROUND_ROPE_BF16);
+  const bool half = (rounding & DT_IO_FP16) != 0;
   a.w = weight; a.bias = bias; a.eps = eps;
   a.out_scale = out_scale;
   a.sec_end[0] = a.sec_end[1] = a.sec_end[2] = D;
@@ -297,9 +313,13 @@ extern "C" int dt_qk_norm_rope(const void* x, int64_t x_stride_b, int64_t x_stri
     set_error("too many rows (%lld workgroups)", (long long)wgs);
     return DT_ERR_INVALID;
   }
-  if (D == 128)
-    hipLaunchKernelGGL(qk_norm_rope_kernel<128>, dim3((unsigned)wgs), dim3(kThreads), 0, (hipStream_t)stream, a);
-  else
-    hipLaunchKernelGGL(qk_norm_rope_kernel<64>, dim3((unsigned)wgs), dim3(kThreads), 0, (hipStream_t)stream, a);
+  const dim3 grid((unsigned)wgs), block(kThreads);
+  if (D == 128) {
+    if (half) hipLaunchKernelGGL((qk_norm_rope_kernel<128, true>), grid, block, 0, (hipStream_t)stream, a);
+    else hipLaunchKernelGGL((qk_norm_rope_kernel<128, false>), grid, block, 0, (hipStream_t)stream, a);
+  } else {
+    if (half) hipLaunchKernelGGL((qk_norm_rope_kernel<64, true>), grid, block, 0, (hipStream_t)stream, a);
+    else hipLaunchKernelGGL((qk_norm_rope_kernel<64, false>), grid, block, 0, (hipStream_t)stream, a);
+  }
   return hip_fail(hipGetLastError(), "qk_norm_rope launch");
 }

@@ -25,13 +25,28 @@ struct MergeArgs {
   int32_t B, Sq, H;
   const void* out[DT_MAX_MERGE];
   const float* lse[DT_MAX_MERGE];
-  uint64_t fp32_mask;   // bit i: out[i] is fp32 (else bf16)
+  uint64_t fp32_mask;   // bit i: out[i] is fp32 (else a 16-bit type)
+  uint64_t f16_mask;    // bit i: out[i] is IEEE half (neither bit: bfloat16)
   uint64_t bsh_mask;    // bit i: lse[i] is [B,Sq,H] (else [B,H,Sq])
   void* dst_out;
   float* dst_lse;
-  int32_t dst_fp32;
+  int32_t dst_dtype;    // DT_BF16 / DT_FP32 / DT_FP16
   int32_t dst_bsh;
 };
+
+// The two 16-bit elements of a word, widened (f16: IEEE half, else bfloat16), and back (round to nearest even).
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void widen16x2(uint32_t w, bool f16, float& lo, float& hi) {
+  if (f16) {
+    const f32x2 f = __builtin_convertvector(__builtin_bit_cast(f16x2, w), f32x2);
+    lo = f.x;
+    hi = f.y;
+  } else {
+    lo = __uint_as_float(w << 16);
+    hi = __uint_as_float(w & 0xffff0000u);
+  }
+}
 
 __device__ __forceinline__ int64_t lse_index(bool bsh, int b, int h, int s, int H, int Sq) {
   return bsh ? ((int64_t)b * Sq + s) * H + h : ((int64_t)b * H + h) * Sq + s;
@@ -39,12 +54,12 @@ __device__ __forceinline__ int64_t lse_index(bool bsh, int b, int h, int s, int 
 
 // A lane owns 8 elements of its row: [4c, 4c+4) and [D/2 + 4c, D/2 + 4c + 4), c = lane index
 // within the row's lane group.  Every load/store instruction is then contiguous across the
-// group (8 bytes per lane for bf16, 16 bytes per lane for fp32), for either dtype on either
+// group (8 bytes per lane for the 16-bit types, 16 bytes per lane for fp32), for any dtype on either
 // side; a lane owning 8 consecutive elements would write fp32 as two interleaved half-sector
 // streams.
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 struct Row8 {
-  u32x4 lo, hi;  // bf16: lo.xy = first group, lo.zw = second group; fp32: lo / hi = the two groups
+  u32x4 lo, hi;  // 16-bit types: lo.xy = first group, lo.zw = second group; fp32: lo / hi = the two groups
 };
 
 template <int D>
@@ -64,8 +79,8 @@ __device__ __forceinline__ Row8 load_row8(const void* base, bool fp32, int64_t r
   return r;
 }
 
-__device__ __forceinline__ void unpack_row8(const Row8& r, bool fp32, float (&x)[8]) {
-  if (fp32) {
+__device__ __forceinline__ void unpack_row8(const Row8& r, int dtype, float (&x)[8]) {
+  if (dtype == DT_FP32) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       x[i] = __uint_as_float(r.lo[i]);
@@ -73,15 +88,11 @@ __device__ __forceinline__ void unpack_row8(const Row8& r, bool fp32, float (&x)
     }
   } else {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      x[2 * i] = __uint_as_float(r.lo[i] << 16);
-      x[2 * i + 1] = __uint_as_float(r.lo[i] & 0xffff0000u);
-    }
+    for (int i = 0; i < 4; ++i) widen16x2(r.lo[i], dtype == DT_FP16, x[2 * i], x[2 * i + 1]);
   }
 }
 
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  typedef float f32x2 __attribute__((ext_vector_type(2)));
   typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
   f32x2 f;
   f.x = lo;
@@ -89,10 +100,17 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   const bf16x2 b = __builtin_convertvector(f, bf16x2);  // round to nearest even
   return __builtin_bit_cast(uint32_t, b);
 }
+__device__ __forceinline__ uint32_t pack16x2(float lo, float hi, bool f16) {
+  if (!f16) return pack_bf16x2(lo, hi);
+  f32x2 f;
+  f.x = lo;
+  f.y = hi;
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, f16x2));  // round to nearest even
+}
 
 template <int D>
-__device__ __forceinline__ void store_row8(void* base, bool fp32, int64_t row_elem, int c, const float (&x)[8]) {
-  if (fp32) {
+__device__ __forceinline__ void store_row8(void* base, int dtype, int64_t row_elem, int c, const float (&x)[8]) {
+  if (dtype == DT_FP32) {
     float* p = reinterpret_cast<float*>(base) + row_elem + 4 * c;
     u32x4 a, b;
 #pragma unroll
@@ -104,11 +122,12 @@ __device__ __forceinline__ void store_row8(void* base, bool fp32, int64_t row_el
     __builtin_nontemporal_store(b, reinterpret_cast<u32x4*>(p + D / 2));
   } else {
     uint16_t* p = reinterpret_cast<uint16_t*>(base) + row_elem + 4 * c;
+    const bool f16 = dtype == DT_FP16;
     u32x2 g0, g1;
-    g0.x = pack_bf16x2(x[0], x[1]);
-    g0.y = pack_bf16x2(x[2], x[3]);
-    g1.x = pack_bf16x2(x[4], x[5]);
-    g1.y = pack_bf16x2(x[6], x[7]);
+    g0.x = pack16x2(x[0], x[1], f16);
+    g0.y = pack16x2(x[2], x[3], f16);
+    g1.x = pack16x2(x[4], x[5], f16);
+    g1.y = pack16x2(x[6], x[7], f16);
     __builtin_nontemporal_store(g0, reinterpret_cast<u32x2*>(p));
     __builtin_nontemporal_store(g1, reinterpret_cast<u32x2*>(p + D / 2));
   }
@@ -167,11 +186,11 @@ struct UnitAcc {
 template <int R, int NB, int P>
 struct UnitRegs {
   float l[P][R][NB];
-  u32x4 rb[P][NB];   // all states bf16
+  u32x4 rb[P][NB];   // all states of one 16-bit type
   Row8 r[P][NB];     // mixed dtypes
 };
 
-template <int R, int NB, bool ALL_BF16, int P>
+template <int R, int NB, int FAST, int P>
 __device__ __forceinline__ void unit_load(const MergeArgs& a, int i0, const UnitPos<R> (&u)[P], int cc,
                                           UnitRegs<R, NB, P>& g) {
 #pragma unroll
@@ -187,7 +206,7 @@ __device__ __forceinline__ void unit_load(const MergeArgs& a, int i0, const Unit
       for (int r = 0; r < R; ++r)
         g.l[p][r][j] = u[p].live[r] ? lp[lse_index(bsh, u[p].b[r], u[p].h[r], u[p].s[r], a.H, a.Sq)] : -INFINITY;
       const bool live_lo = u[p].live[0], live_hi = u[p].live[R - 1];
-      if (ALL_BF16) {
+      if (FAST == 1 || FAST == 2) {
         const uint16_t* q = reinterpret_cast<const uint16_t*>(op) + u[p].elem + 4 * cc;
         u32x2 g0 = u32x2{0u, 0u}, g1 = u32x2{0u, 0u};
         if (live_lo) g0 = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(q));
@@ -214,7 +233,7 @@ __device__ __forceinline__ void unit_load(const MergeArgs& a, int i0, const Unit
   }
 }
 
-template <int R, int NB, bool ALL_BF16, int P>
+template <int R, int NB, int FAST, int P>
 __device__ __forceinline__ void unit_fold(const MergeArgs& a, int i0, const UnitRegs<R, NB, P>& g,
                                           UnitAcc<R> (&ua)[P]) {
   constexpr int kPer = 8 / R;   // elements of a lane that belong to one row
@@ -234,14 +253,13 @@ __device__ __forceinline__ void unit_fold(const MergeArgs& a, int i0, const Unit
         for (int j = 0; j < NB; ++j) {
           const float w = __expf(g.l[p][r][j] - m_new);
           float x[8];
-          if (ALL_BF16) {
+          if (FAST == 1 || FAST == 2) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              x[2 * q] = __uint_as_float(g.rb[p][j][q] << 16);
-              x[2 * q + 1] = __uint_as_float(g.rb[p][j][q] & 0xffff0000u);
-            }
+            for (int q = 0; q < 4; ++q) widen16x2(g.rb[p][j][q], FAST == 2, x[2 * q], x[2 * q + 1]);
           } else {
-            unpack_row8(g.r[p][j], (a.fp32_mask >> (i0 + j)) & 1, x);
+            const int i = i0 + j;
+            const int other = (FAST == 0 && ((a.f16_mask >> i) & 1)) ? DT_FP16 : DT_BF16;
+            unpack_row8(g.r[p][j], ((a.fp32_mask >> i) & 1) ? DT_FP32 : other, x);
           }
           ua[p].den[r] += w;
 #pragma unroll
@@ -254,20 +272,20 @@ __device__ __forceinline__ void unit_fold(const MergeArgs& a, int i0, const Unit
   }
 }
 
-template <int R, int NB, bool ALL_BF16, int P>
+template <int R, int NB, int FAST, int P>
 __device__ __forceinline__ void unit_batch(const MergeArgs& a, int i0, const UnitPos<R> (&u)[P], int cc,
                                            UnitAcc<R> (&ua)[P]) {
   UnitRegs<R, NB, P> g;
-  unit_load<R, NB, ALL_BF16, P>(a, i0, u, cc, g);
-  unit_fold<R, NB, ALL_BF16, P>(a, i0, g, ua);
+  unit_load<R, NB, FAST, P>(a, i0, u, cc, g);
+  unit_fold<R, NB, FAST, P>(a, i0, g, ua);
 }
 
-template <int R, bool ALL_BF16, int NB, int P>
+template <int R, int FAST, int NB, int P>
 __device__ __forceinline__ void unit_rest(const MergeArgs& a, int i0, int rest, const UnitPos<R> (&u)[P],
                                           int cc, UnitAcc<R> (&ua)[P]) {
   if constexpr (NB >= 1) {
-    if (rest == NB) unit_batch<R, NB, ALL_BF16, P>(a, i0, u, cc, ua);
-    else unit_rest<R, ALL_BF16, NB - 1, P>(a, i0, rest, u, cc, ua);
+    if (rest == NB) unit_batch<R, NB, FAST, P>(a, i0, u, cc, ua);
+    else unit_rest<R, FAST, NB - 1, P>(a, i0, rest, u, cc, ua);
   }
 }
 
@@ -355,7 +373,9 @@ static int64_t unit_grid(int B, int Sq, int H, int D, bool tiled, int passes) {
 }
 static bool unit_tiles_fit(int H, int D) { return H % ((128 / D) * kTileHeadUnits) == 0; }
 
-template <int D, bool ALL_BF16, int MAP, int P>
+// FAST: 1 = every state bfloat16, 2 = every state IEEE half (one decode, no per-state dtype); mixed dtypes:
+// 3 = bfloat16 and fp32 only, 0 = any of the three.
+template <int D, int FAST, int MAP, int P>
 __global__ __launch_bounds__(kThreads) void merge_states_kernel(const MergeArgs a) {
   constexpr int R = 128 / D;
   const int cc = threadIdx.x % kUnitLanes;
@@ -373,8 +393,8 @@ __global__ __launch_bounds__(kThreads) void merge_states_kernel(const MergeArgs 
     for (int k = 0; k < 8; ++k) ua[p].acc[k] = 0.f;
   }
   int i0 = 0;
-  for (; i0 + kBatch <= a.n; i0 += kBatch) unit_batch<R, kBatch, ALL_BF16, P>(a, i0, u, cc, ua);
-  unit_rest<R, ALL_BF16, kBatch - 1, P>(a, i0, a.n - i0, u, cc, ua);
+  for (; i0 + kBatch <= a.n; i0 += kBatch) unit_batch<R, kBatch, FAST, P>(a, i0, u, cc, ua);
+  unit_rest<R, FAST, kBatch - 1, P>(a, i0, a.n - i0, u, cc, ua);
   constexpr int kPer = 8 / R;
 #pragma unroll
   for (int p = 0; p < P; ++p) {
@@ -386,7 +406,7 @@ __global__ __launch_bounds__(kThreads) void merge_states_kernel(const MergeArgs 
       for (int k = 0; k < kPer; ++k) o[r * kPer + k] = ua[p].acc[r * kPer + k] * inv;
     }
     const bool live_lo = u[p].live[0], live_hi = u[p].live[R - 1];
-    if (a.dst_fp32) {
+    if (a.dst_dtype == DT_FP32) {
       float* q = reinterpret_cast<float*>(a.dst_out) + u[p].elem + 4 * cc;
       u32x4 v0, v1;
 #pragma unroll
@@ -398,11 +418,12 @@ __global__ __launch_bounds__(kThreads) void merge_states_kernel(const MergeArgs 
       if (live_hi) __builtin_nontemporal_store(v1, reinterpret_cast<u32x4*>(q + 64));
     } else {
       uint16_t* q = reinterpret_cast<uint16_t*>(a.dst_out) + u[p].elem + 4 * cc;
+      const bool f16 = a.dst_dtype == DT_FP16;
       u32x2 g0, g1;
-      g0.x = pack_bf16x2(o[0], o[1]);
-      g0.y = pack_bf16x2(o[2], o[3]);
-      g1.x = pack_bf16x2(o[4], o[5]);
-      g1.y = pack_bf16x2(o[6], o[7]);
+      g0.x = pack16x2(o[0], o[1], f16);
+      g0.y = pack16x2(o[2], o[3], f16);
+      g1.x = pack16x2(o[4], o[5], f16);
+      g1.y = pack16x2(o[6], o[7], f16);
       if (live_lo) __builtin_nontemporal_store(g0, reinterpret_cast<u32x2*>(q));
       if (live_hi) __builtin_nontemporal_store(g1, reinterpret_cast<u32x2*>(q + 64));
     }
@@ -422,13 +443,14 @@ struct CopyArgs {
   void* dst_out;
   float* dst_lse;
   int32_t B, Sq, H;
-  int32_t src_fp32, src_bsh, dst_fp32, dst_bsh;
+  int32_t src_dtype, src_bsh, dst_dtype, dst_bsh;   // DT_BF16 / DT_FP32 / DT_FP16
 };
 
 
 constexpr int kCopyRows = 1;  // rows per lane group (2 and 4 measured: -6 % and -12 %)
 
-template <int D>
+// SRC / DST: the DT_* codes of the two sides, fixed at compile time (the launcher picks the instantiation).
+template <int D, int SRC, int DST>
 __global__ __launch_bounds__(kThreads) void state_copy_kernel(const CopyArgs a) {
   constexpr int kLanesPerRow = D / 8;
   constexpr int kRowsPerPass = kThreads / kLanesPerRow;
@@ -445,7 +467,7 @@ __global__ __launch_bounds__(kThreads) void state_copy_kernel(const CopyArgs a) 
     const int s = st * kRowsPerWg + p * kRowsPerPass + rr;
     if (s < a.Sq) {
       const int64_t elem = (((int64_t)b * a.Sq + s) * a.H + h) * D;
-      r[p] = load_row8<D>(a.src_out, a.src_fp32 != 0, elem, cc);
+      r[p] = load_row8<D>(a.src_out, SRC == DT_FP32, elem, cc);
       if (copy_lse) l[p] = a.src_lse[lse_index(a.src_bsh != 0, b, h, s, a.H, a.Sq)];
     }
   }
@@ -455,8 +477,8 @@ __global__ __launch_bounds__(kThreads) void state_copy_kernel(const CopyArgs a) 
     if (s < a.Sq) {
       const int64_t elem = (((int64_t)b * a.Sq + s) * a.H + h) * D;
       float x[8];
-      unpack_row8(r[p], a.src_fp32 != 0, x);
-      store_row8<D>(a.dst_out, a.dst_fp32 != 0, elem, cc, x);
+      unpack_row8(r[p], SRC, x);
+      store_row8<D>(a.dst_out, DST, elem, cc, x);
       if (copy_lse) a.dst_lse[lse_index(a.dst_bsh != 0, b, h, s, a.H, a.Sq)] = l[p];
     }
   }
@@ -465,7 +487,7 @@ __global__ __launch_bounds__(kThreads) void state_copy_kernel(const CopyArgs a) 
 // The same copy on 256-byte units (see the merge): at D = 64 a lane group then moves two neighbouring
 // rows and every load / store instruction covers whole 128-byte lines, where the row-mapped kernel above
 // touches half of each line per instruction.
-template <int D, int MAP>
+template <int D, int MAP, int SRC, int DST>
 __global__ __launch_bounds__(kThreads) void state_copy_units_kernel(const CopyArgs a) {
   constexpr int R = 128 / D;
   const int cc = threadIdx.x % kUnitLanes;
@@ -482,7 +504,7 @@ __global__ __launch_bounds__(kThreads) void state_copy_units_kernel(const CopyAr
       l = a.src_lse[lse_index(a.src_bsh != 0, u[0].b[r], u[0].h[r], u[0].s[r], a.H, a.Sq)];
     }
   float x[8];
-  if (a.src_fp32) {
+  if (SRC == DT_FP32) {
     const float* q = reinterpret_cast<const float*>(a.src_out) + u[0].elem + 4 * cc;
     u32x4 v0 = u32x4{0u, 0u, 0u, 0u}, v1 = v0;
     if (live_lo) v0 = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(q));
@@ -497,12 +519,13 @@ __global__ __launch_bounds__(kThreads) void state_copy_units_kernel(const CopyAr
     u32x2 g0 = u32x2{0u, 0u}, g1 = g0;
     if (live_lo) g0 = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(q));
     if (live_hi) g1 = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(q + 64));
-    x[0] = __uint_as_float(g0.x << 16); x[1] = __uint_as_float(g0.x & 0xffff0000u);
-    x[2] = __uint_as_float(g0.y << 16); x[3] = __uint_as_float(g0.y & 0xffff0000u);
-    x[4] = __uint_as_float(g1.x << 16); x[5] = __uint_as_float(g1.x & 0xffff0000u);
-    x[6] = __uint_as_float(g1.y << 16); x[7] = __uint_as_float(g1.y & 0xffff0000u);
+    const bool f16 = SRC == DT_FP16;
+    widen16x2(g0.x, f16, x[0], x[1]);
+    widen16x2(g0.y, f16, x[2], x[3]);
+    widen16x2(g1.x, f16, x[4], x[5]);
+    widen16x2(g1.y, f16, x[6], x[7]);
   }
-  if (a.dst_fp32) {
+  if (DST == DT_FP32) {
     float* q = reinterpret_cast<float*>(a.dst_out) + u[0].elem + 4 * cc;
     u32x4 v0, v1;
 #pragma unroll
@@ -514,11 +537,12 @@ __global__ __launch_bounds__(kThreads) void state_copy_units_kernel(const CopyAr
     if (live_hi) __builtin_nontemporal_store(v1, reinterpret_cast<u32x4*>(q + 64));
   } else {
     uint16_t* q = reinterpret_cast<uint16_t*>(a.dst_out) + u[0].elem + 4 * cc;
+    const bool f16 = DST == DT_FP16;
     u32x2 g0, g1;
-    g0.x = pack_bf16x2(x[0], x[1]);
-    g0.y = pack_bf16x2(x[2], x[3]);
-    g1.x = pack_bf16x2(x[4], x[5]);
-    g1.y = pack_bf16x2(x[6], x[7]);
+    g0.x = pack16x2(x[0], x[1], f16);
+    g0.y = pack16x2(x[2], x[3], f16);
+    g1.x = pack16x2(x[4], x[5], f16);
+    g1.y = pack16x2(x[6], x[7], f16);
     if (live_lo) __builtin_nontemporal_store(g0, reinterpret_cast<u32x2*>(q));
     if (live_hi) __builtin_nontemporal_store(g1, reinterpret_cast<u32x2*>(q + 64));
   }
@@ -528,7 +552,7 @@ __global__ __launch_bounds__(kThreads) void state_copy_units_kernel(const CopyAr
       a.dst_lse[lse_index(a.dst_bsh != 0, u[0].b[r], u[0].h[r], u[0].s[r], a.H, a.Sq)] = l;
 }
 
-// bf16 state -> fp32 state (a cache load): `out` is an elementwise widening in the same element order,
+// bf16 or fp16 state -> fp32 state (a cache load): `out` is an elementwise widening in the same element order,
 // so it runs as a flat pass -- a lane takes 4 consecutive elements (8 bytes in, 16 bytes out), one
 // load and one store, both non-temporal (+5 % over the row-mapped kernel above in this direction; in
 // the narrowing direction the row-mapped kernel is the faster one by 5-13 %, so it keeps that).  The
@@ -545,11 +569,13 @@ __global__ __launch_bounds__(kConvThreads) void state_widen_kernel(const CopyArg
     const int64_t g = (int64_t)(blockIdx.x - wgs_lse) * kConvThreads + threadIdx.x;   // 4 elements
     if (g >= groups) return;
     const u32x2 v = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(a.src_out) + g);
+    const bool f16 = a.src_dtype == DT_FP16;
+    float x[4];
+    widen16x2(v.x, f16, x[0], x[1]);
+    widen16x2(v.y, f16, x[2], x[3]);
     u32x4 o;
-    o.x = v.x << 16;
-    o.y = v.x & 0xffff0000u;
-    o.z = v.y << 16;
-    o.w = v.y & 0xffff0000u;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = __float_as_uint(x[i]);
     __builtin_nontemporal_store(o, reinterpret_cast<u32x4*>(a.dst_out) + g);
     return;
   }
@@ -723,8 +749,11 @@ constexpr int64_t kTwoPassUnits = 1 << 20;
 
 template <int D, int MAP, int P>
 static void launch_merge_k(const MergeArgs& a, unsigned wgs, hipStream_t stream) {
-  if (a.fp32_mask == 0) hipLaunchKernelGGL((merge_states_kernel<D, true, MAP, P>), dim3(wgs), dim3(kThreads), 0, stream, a);
-  else hipLaunchKernelGGL((merge_states_kernel<D, false, MAP, P>), dim3(wgs), dim3(kThreads), 0, stream, a);
+  const uint64_t all = a.n >= 64 ? ~0ull : ((1ull << a.n) - 1);
+  if (a.fp32_mask == 0 && a.f16_mask == 0) hipLaunchKernelGGL((merge_states_kernel<D, 1, MAP, P>), dim3(wgs), dim3(kThreads), 0, stream, a);
+  else if (a.f16_mask == all) hipLaunchKernelGGL((merge_states_kernel<D, 2, MAP, P>), dim3(wgs), dim3(kThreads), 0, stream, a);
+  else if (a.f16_mask == 0) hipLaunchKernelGGL((merge_states_kernel<D, 3, MAP, P>), dim3(wgs), dim3(kThreads), 0, stream, a);
+  else hipLaunchKernelGGL((merge_states_kernel<D, 0, MAP, P>), dim3(wgs), dim3(kThreads), 0, stream, a);
 }
 
 template <int D>
@@ -760,14 +789,43 @@ int launch_merge(const MergeArgs& a, int D, hipStream_t stream) {
   return hip_fail(hipGetLastError(), "merge_states launch");
 }
 
+// Picks the instantiation of a copy kernel for the (source, destination) dtypes of `a`.
+template <template <int, int> class Launch>
+static void dispatch_copy_dtypes(const CopyArgs& a, unsigned wgs, hipStream_t stream) {
+#define DT_COPY_CASE(S, T) \
+  if (a.src_dtype == S && a.dst_dtype == T) return Launch<S, T>::run(a, wgs, stream);
+  DT_COPY_CASE(DT_BF16, DT_BF16) DT_COPY_CASE(DT_BF16, DT_FP32) DT_COPY_CASE(DT_BF16, DT_FP16)
+  DT_COPY_CASE(DT_FP32, DT_BF16) DT_COPY_CASE(DT_FP32, DT_FP32) DT_COPY_CASE(DT_FP32, DT_FP16)
+  DT_COPY_CASE(DT_FP16, DT_BF16) DT_COPY_CASE(DT_FP16, DT_FP32) DT_COPY_CASE(DT_FP16, DT_FP16)
+#undef DT_COPY_CASE
+}
+template <int SRC, int DST>
+struct LaunchCopyUnits64 {
+  static void run(const CopyArgs& a, unsigned wgs, hipStream_t stream) {
+    hipLaunchKernelGGL((state_copy_units_kernel<64, MAP_TILED, SRC, DST>), dim3(wgs), dim3(kThreads), 0, stream, a);
+  }
+};
+template <int SRC, int DST>
+struct LaunchCopyRows128 {
+  static void run(const CopyArgs& a, unsigned wgs, hipStream_t stream) {
+    hipLaunchKernelGGL((state_copy_kernel<128, SRC, DST>), dim3(wgs), dim3(kThreads), 0, stream, a);
+  }
+};
+template <int SRC, int DST>
+struct LaunchCopyRows64 {
+  static void run(const CopyArgs& a, unsigned wgs, hipStream_t stream) {
+    hipLaunchKernelGGL((state_copy_kernel<64, SRC, DST>), dim3(wgs), dim3(kThreads), 0, stream, a);
+  }
+};
+
 int launch_copy(const CopyArgs& a, int D, hipStream_t stream) {
   const bool with_lse = a.dst_lse != nullptr && a.src_lse != nullptr;
-  if (a.src_fp32 == a.dst_fp32 && (!with_lse || a.src_bsh == a.dst_bsh) && (D == 64 || D == 128)) {
+  if (a.src_dtype == a.dst_dtype && (!with_lse || a.src_bsh == a.dst_bsh) && (D == 64 || D == 128)) {
     const int64_t rows = (int64_t)a.B * a.Sq * a.H;
     FlatCopyArgs f{};
     f.src[0] = static_cast<const uint8_t*>(a.src_out);
     f.dst[0] = static_cast<uint8_t*>(a.dst_out);
-    f.bytes[0] = rows * D * (a.src_fp32 ? 4 : 2);
+    f.bytes[0] = rows * D * (a.src_dtype == DT_FP32 ? 4 : 2);
     f.src[1] = reinterpret_cast<const uint8_t*>(a.src_lse);
     f.dst[1] = reinterpret_cast<uint8_t*>(a.dst_lse);
     f.bytes[1] = with_lse ? rows * 4 : 0;
@@ -784,7 +842,7 @@ int launch_copy(const CopyArgs& a, int D, hipStream_t stream) {
     set_error("head dim %d not built (64 and 128 are)", D);
     return DT_ERR_UNSUPPORTED;
   }
-  if (!a.src_fp32 && a.dst_fp32) {
+  if (a.src_dtype != DT_FP32 && a.dst_dtype == DT_FP32) {
     const int64_t rows = (int64_t)a.B * a.Sq * a.H;
     const int64_t groups = rows * D / 4;
     const int64_t w_out = (groups + kConvThreads - 1) / kConvThreads;
@@ -813,7 +871,7 @@ int launch_copy(const CopyArgs& a, int D, hipStream_t stream) {
       set_error("copy grid too large");
       return DT_ERR_INVALID;
     }
-    hipLaunchKernelGGL((state_copy_units_kernel<64, MAP_TILED>), dim3((unsigned)wgs), dim3(kThreads), 0, stream, a);
+    dispatch_copy_dtypes<LaunchCopyUnits64>(a, (unsigned)wgs, stream);
     return hip_fail(hipGetLastError(), "state_copy_units launch");
   }
   const int rows_per_wg = kThreads / (D / 8) * kCopyRows;
@@ -824,8 +882,8 @@ int launch_copy(const CopyArgs& a, int D, hipStream_t stream) {
     set_error("copy grid too large");
     return DT_ERR_INVALID;
   }
-  if (D == 128) hipLaunchKernelGGL(state_copy_kernel<128>, dim3((unsigned)wgs), dim3(kThreads), 0, stream, a);
-  else hipLaunchKernelGGL(state_copy_kernel<64>, dim3((unsigned)wgs), dim3(kThreads), 0, stream, a);
+  if (D == 128) dispatch_copy_dtypes<LaunchCopyRows128>(a, (unsigned)wgs, stream);
+  else dispatch_copy_dtypes<LaunchCopyRows64>(a, (unsigned)wgs, stream);
   return hip_fail(hipGetLastError(), "state_copy launch");
 }
 
@@ -834,6 +892,7 @@ int launch_copy(const CopyArgs& a, int D, hipStream_t stream) {
 using namespace dt;
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+static bool known_dtype(int32_t d) { return d == DT_BF16 || d == DT_FP32 || d == DT_FP16; }
 
 static int check_dims(int32_t B, int32_t Sq, int32_t H, int32_t D) {
   if (B <= 0 || Sq <= 0 || H <= 0) {
@@ -872,21 +931,21 @@ extern "C" int dt_merge_states(int32_t n, const void* const* outs, const float* 
     a.lse[i] = lses[i];
     const int dtp = src_dtype ? src_dtype[i] : DT_BF16;
     const int lay = src_lse_layout ? src_lse_layout[i] : DT_LSE_BHS;
-    if ((dtp != DT_BF16 && dtp != DT_FP32) || (lay != DT_LSE_BHS && lay != DT_LSE_BSH)) {
+    if (!known_dtype(dtp) || (lay != DT_LSE_BHS && lay != DT_LSE_BSH)) {
       set_error("state %d: bad dtype/layout code", i);
       return DT_ERR_INVALID;
     }
     if (dtp == DT_FP32) a.fp32_mask |= (1ull << i);
+    if (dtp == DT_FP16) a.f16_mask |= (1ull << i);
     if (lay == DT_LSE_BSH) a.bsh_mask |= (1ull << i);
   }
-  if (!aligned16(dst_out) || (dst_dtype != DT_BF16 && dst_dtype != DT_FP32) ||
-      (dst_lse_layout != DT_LSE_BHS && dst_lse_layout != DT_LSE_BSH)) {
+  if (!aligned16(dst_out) || !known_dtype(dst_dtype) || (dst_lse_layout != DT_LSE_BHS && dst_lse_layout != DT_LSE_BSH)) {
     set_error("bad destination pointer/dtype/layout");
     return DT_ERR_INVALID;
   }
   a.dst_out = dst_out;
   a.dst_lse = dst_lse;
-  a.dst_fp32 = dst_dtype == DT_FP32;
+  a.dst_dtype = dst_dtype;
   a.dst_bsh = dst_lse_layout == DT_LSE_BSH;
   return launch_merge(a, D, (hipStream_t)stream);
 }
@@ -899,7 +958,7 @@ static int state_copy(const void* src_out, int32_t src_dtype, const float* src_l
     set_error("null or misaligned state pointer");
     return DT_ERR_INVALID;
   }
-  if ((src_dtype != DT_BF16 && src_dtype != DT_FP32) || (dst_dtype != DT_BF16 && dst_dtype != DT_FP32) ||
+  if (!known_dtype(src_dtype) || !known_dtype(dst_dtype) ||
       (src_layout != DT_LSE_BHS && src_layout != DT_LSE_BSH) || (dst_layout != DT_LSE_BHS && dst_layout != DT_LSE_BSH)) {
     set_error("bad dtype/layout code");
     return DT_ERR_INVALID;
@@ -907,8 +966,8 @@ static int state_copy(const void* src_out, int32_t src_dtype, const float* src_l
   CopyArgs a{};
   a.src_out = src_out; a.src_lse = src_lse; a.dst_out = dst_out; a.dst_lse = dst_lse;
   a.B = B; a.Sq = Sq; a.H = H;
-  a.src_fp32 = src_dtype == DT_FP32; a.src_bsh = src_layout == DT_LSE_BSH;
-  a.dst_fp32 = dst_dtype == DT_FP32; a.dst_bsh = dst_layout == DT_LSE_BSH;
+  a.src_dtype = src_dtype; a.src_bsh = src_layout == DT_LSE_BSH;
+  a.dst_dtype = dst_dtype; a.dst_bsh = dst_layout == DT_LSE_BSH;
   return launch_copy(a, D, (hipStream_t)stream);
 }
 
@@ -923,6 +982,13 @@ extern "C" int dt_cache_load(const void* slot_out, const float* slot_lse, void* 
                              float* dst_lse, int32_t dst_lse_layout, int32_t B, int32_t Sq, int32_t H, int32_t D,
                              void* stream) {
   return state_copy(slot_out, DT_BF16, slot_lse, DT_LSE_BHS, dst_out, dst_dtype, dst_lse, dst_lse_layout, B, Sq, H, D,
+                    stream);
+}
+
+extern "C" int dt_state_copy(const void* src_out, int32_t src_dtype, const float* src_lse, int32_t src_lse_layout,
+                             void* dst_out, int32_t dst_dtype, float* dst_lse, int32_t dst_lse_layout, int32_t B,
+                             int32_t Sq, int32_t H, int32_t D, void* stream) {
+  return state_copy(src_out, src_dtype, src_lse, src_lse_layout, dst_out, dst_dtype, dst_lse, dst_lse_layout, B, Sq, H, D,
                     stream);
 }
 

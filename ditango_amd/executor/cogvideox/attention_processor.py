@@ -40,14 +40,14 @@ class CVX_oCacheAttnProcessor:
 
     def project_qkv(self, attn, hidden_states: torch.Tensor, encoder_hidden_states: torch.Tensor,
                     image_rotary_emb: Optional[Tuple[torch.Tensor, torch.Tensor]] = None):
-        """(query, key, value) of this rank's token shard, text tokens first, as bf16 ``[B,S,H,D]`` in the layout
+        """(query, key, value) of this rank's token shard, text tokens first, as ``[B,S,H,D]`` (bf16 or fp16, the model's dtype) in the layout
         the attention reads (:39-71 of the reference, without its transposes).  Also what a test or a ring
         stand-in calls to produce the K/V another rank would send."""
         text_seqlen = encoder_hidden_states.size(1)
         batch_size = hidden_states.shape[0]
         x = torch.cat([encoder_hidden_states, hidden_states], dim=1)
-        if x.dtype != torch.bfloat16:
-            raise TypeError(f"the adapter runs bf16 activations (the model's dtype), got {x.dtype}")
+        if x.dtype not in (torch.bfloat16, torch.float16):
+            raise TypeError(f"the adapter runs bf16 or fp16 activations (the model's dtype), got {x.dtype}")
         query, key, value = attn.to_q(x), attn.to_k(x), attn.to_v(x)
         head_num = attn.heads
         head_dim = key.shape[-1] // head_num
@@ -56,7 +56,7 @@ class CVX_oCacheAttnProcessor:
         value = value.view(batch_size, -1, head_num, head_dim)
         rope = dict(rope="interleaved", freqs_cis=image_rotary_emb, rope_begin=text_seqlen) if image_rotary_emb is not None else {}
         k_rope = rope if not getattr(attn, "is_cross_attention", False) else {}
-        # rounded where the reference's bf16 modules round: after the norm, after the rotation
+        # rounded where the reference's modules round in the model's dtype: after the norm, after the rotation
         query = prepare_qk(query, **self._norm_args(getattr(attn, "norm_q", None)), match_eager_rounding=True, **rope)
         key = prepare_qk(key, **self._norm_args(getattr(attn, "norm_k", None)), match_eager_rounding=True, **k_rope)
         return query, key, value.contiguous()

@@ -35,6 +35,6 @@ class Attention(nn.Module):
         writes that dtype itself; the reference's ``.to(q.dtype)`` pass disappears."""
         rm = get_redundancy_map()
         profiling = rm is not None and rm.auto_setting      # the profiled metric is defined on the fp32 result
-        self.oAttn.out_dtype = q.dtype if (q.dtype == torch.bfloat16 and not profiling) else torch.float32
+        self.oAttn.out_dtype = q.dtype if (q.dtype in (torch.bfloat16, torch.float16) and not profiling) else torch.float32
         x = self.oAttn.attn(q, k, v)
         return x.to(q.dtype)

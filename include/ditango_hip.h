@@ -12,8 +12,8 @@
  * message for the calling thread.
  *
  * Tensor layouts (element strides, innermost dimension contiguous):
- *   q / out state   bf16  [B, Sq, H, D]
- *   k, v chunk      bf16  [B, Sk, H, D]
+ *   q / out state   bf16  [B, Sq, H, D]   (IEEE half instead where an entry point or a flag says so:
+ *   k, v chunk      bf16  [B, Sk, H, D]    dt_attn_chunk_f16_fwd, DT_ATTN_FP16, DT_FP16, DT_IO_FP16)
  *   lse state       fp32  [B, H, Sq]     (DT_LSE_BHS, flash-attn's layout)
  *                   fp32  [B, Sq, H]     (DT_LSE_BSH, the running layout
  *                                         [B,S,H,1] of utils.py:49)
@@ -36,6 +36,7 @@ extern "C" {
 
 #define DT_BF16 0
 #define DT_FP32 1
+#define DT_FP16 2 /* IEEE binary16 */
 
 #define DT_LSE_BHS 0
 #define DT_LSE_BSH 1
@@ -50,6 +51,7 @@ extern "C" {
 
 #define DT_ROUND_NORM_BF16 1 /* round to bf16 where the callers' bf16 norm modules do */
 #define DT_ROUND_ROPE_BF16 2 /* RoPE products and their sum each rounded to bf16 */
+#define DT_IO_FP16 4         /* x and y are fp16; the two bits above then round to fp16 */
 
 #define DT_MAX_CHUNKS 40       /* KV chunks one launch can address */
 #define DT_MAX_JOBS 40         /* attention states one launch can produce */
@@ -73,6 +75,19 @@ int dt_attn_chunk_fwd(const void* q, const void* k, const void* v, void* out, fl
                       int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
                       int64_t kv_stride_b, int64_t kv_stride_s, int64_t kv_stride_h,
                       float softmax_scale, void* stream);
+
+/*
+ * The same call for IEEE half tensors (flash_attn_func takes fp16 or bf16; the reference passes whatever
+ * dtype the model runs in, core/attention.py:137-143, and executor/hunyuanvideo offers --precision fp16):
+ * q, k, v and out are fp16, the products run on the fp16 MFMA, P is rounded to fp16 where the bf16 path
+ * rounds it to bf16.  Everything else as above.  The launches that take `flags` do the same under
+ * DT_ATTN_FP16.
+ */
+int dt_attn_chunk_f16_fwd(const void* q, const void* k, const void* v, void* out, float* lse,
+                          int32_t B, int32_t Sq, int32_t Sk, int32_t H, int32_t D,
+                          int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
+                          int64_t kv_stride_b, int64_t kv_stride_s, int64_t kv_stride_h,
+                          float softmax_scale, void* stream);
 
 /*
  * The same call site (core/attention.py:185-191) for fp32 tensors, computed in fp32 throughout (vector
@@ -241,8 +256,12 @@ int dt_zero_rows_from(void* dst, int64_t n_rows, int64_t row_bytes, const int32_
  * q k^T are then exponents of 2 as they stand, softmax_scale is ignored, and the softmax needs a
  * quarter fewer vector instructions (4 % faster at D = 128, 10 % at D = 64).  out and lse are those
  * of softmax(q k^T * ln 2).  The reference has no such mode (flash_attn_func scales inside).
+ * DT_ATTN_FP16 says that q, k, v, the output states (and the partial states in the workspace) are IEEE
+ * half instead of bfloat16, as in dt_attn_chunk_f16_fwd; it does not combine with DT_ATTN_Q_PRESCALED
+ * (DT_ERR_UNSUPPORTED).
  */
 #define DT_ATTN_Q_PRESCALED 1
+#define DT_ATTN_FP16 2
 int64_t dt_attn_workspace_bytes(void);
 int dt_attn_seg_jobs_ws_fwd(const void* q, int32_t B, int32_t Sq, int32_t H, int32_t D,
                             int64_t q_stride_b, int64_t q_stride_s, int64_t q_stride_h,
@@ -302,7 +321,7 @@ int dt_attn_seg_jobs_noalloc_fwd(const void* q, int32_t B, int32_t Sq, int32_t H
  * Replaces the chain of update_out_and_lse / _update_out_and_lse calls
  * (utils.py:24-84; called at core/attention.py:116,144,194,196,213 and
  * core/cache.py:42) with one pass over HBM.  outs[i] is [B,Sq,H,D] contiguous
- * in src_dtype[i]; lses[i] is fp32 in src_lse_layout[i].  A state whose lse is
+ * in src_dtype[i] (DT_BF16, DT_FP16 or DT_FP32, in any mix); lses[i] is fp32 in src_lse_layout[i].  A state whose lse is
  * -inf contributes nothing.  dst may alias one of the inputs of the same dtype
  * and layout (in-place cache coarsening, core/cache.py:28-46).  A pointer may
  * appear more than once (the reference can merge the local chunk twice,
@@ -318,12 +337,17 @@ int dt_merge_states(int32_t n, const void* const* outs, const float* const* lses
  * State cache store / load: one streaming copy of (out, lse) between a caller
  * tensor and a cache slot (out bf16 [B,Sq,H,D], lse fp32 [B,H,Sq]).  Replaces
  * proCache.store_block / get_block (core/cache.py:75-84), which in the
- * reference keep Python references to fp32 tensors.
+ * reference keep Python references to fp32 tensors.  dt_state_copy is the same
+ * copy between any two state formats (out in DT_BF16 / DT_FP16 / DT_FP32, lse in
+ * either layout), e.g. for the fp16 slots of a model that runs in fp16.
  */
 int dt_cache_store(const void* src_out, int32_t src_dtype, const float* src_lse, int32_t src_lse_layout,
                    void* slot_out, float* slot_lse,
                    int32_t B, int32_t Sq, int32_t H, int32_t D, void* stream);
 int dt_cache_load(const void* slot_out, const float* slot_lse,
+                  void* dst_out, int32_t dst_dtype, float* dst_lse, int32_t dst_lse_layout,
+                  int32_t B, int32_t Sq, int32_t H, int32_t D, void* stream);
+int dt_state_copy(const void* src_out, int32_t src_dtype, const float* src_lse, int32_t src_lse_layout,
                   void* dst_out, int32_t dst_dtype, float* dst_lse, int32_t dst_lse_layout,
                   int32_t B, int32_t Sq, int32_t H, int32_t D, void* stream);
 
@@ -379,7 +403,8 @@ int dt_rel_l1_sums(const float* a, const float* b, int64_t n, double* sums, void
  *     half, x[d - (hi-lo)/2] in the second.  sections (HOST array, n_sections <= 3, each a
  *     multiple of 16, summing to D; n_sections = 0 means one section of D).
  * rounding = 0 computes in fp32 and rounds once on the way out; the DT_ROUND_* bits reproduce
- * the intermediate bf16 roundings of the callers' eager modules.
+ * the intermediate bf16 roundings of the callers' eager modules.  With DT_IO_FP16 in `rounding`, x and y
+ * are IEEE half (a model run in fp16) and those intermediate roundings are to fp16.
  * out_scale (> 0; 1 for none) multiplies the result before that last rounding: with
  * softmax_scale * log2(e) here for q, the attention may run with DT_ATTN_Q_PRESCALED.
  */

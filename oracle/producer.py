@@ -32,25 +32,32 @@ ROPE_NONE, ROPE_INTERLEAVED, ROPE_HALVES = 0, 1, 2
 ROUND_NORM_BF16, ROUND_ROPE_BF16 = 1, 2
 
 
-def _r(x: torch.Tensor) -> torch.Tensor:
-    return x.to(torch.bfloat16).to(torch.float32)
+def _r(x: torch.Tensor, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    return x.to(dtype).to(torch.float32)
 
 
-def rms_norm(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, round_bf16: bool) -> torch.Tensor:
-    """``x.float() * rsqrt(mean(x^2, -1) + eps)`` [cast to bf16] ``* weight`` [cast to bf16]; fp32 result."""
+def _model_dtype(x: torch.Tensor) -> torch.dtype:
+    """The dtype the callers' eager modules round to: the activations' own (fp16 for a model run in fp16), bf16
+    for anything else."""
+    return torch.float16 if x.dtype == torch.float16 else torch.bfloat16
+
+
+def rms_norm(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, round_bf16: bool,
+             round_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """``x.float() * rsqrt(mean(x^2, -1) + eps)`` [cast to the model dtype] ``* weight`` [cast again]; fp32 result."""
     xf = x.to(torch.float32)
     y = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
     if round_bf16:
-        y = _r(y)
+        y = _r(y, round_dtype)
     if weight is not None:
         y = y * weight.to(torch.float32)
         if round_bf16:
-            y = _r(y)
+            y = _r(y, round_dtype)
     return y
 
 
 def layer_norm(x: torch.Tensor, weight: Optional[torch.Tensor], bias: Optional[torch.Tensor], eps: float,
-               round_bf16: bool) -> torch.Tensor:
+               round_bf16: bool, round_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
     """LayerNorm over the last dimension (biased variance); fp32 math, one rounding at the end if asked."""
     xf = x.to(torch.float32)
     mu = xf.mean(-1, keepdim=True)
@@ -60,7 +67,7 @@ def layer_norm(x: torch.Tensor, weight: Optional[torch.Tensor], bias: Optional[t
         y = y * weight.to(torch.float32)
     if bias is not None:
         y = y + bias.to(torch.float32)
-    return _r(y) if round_bf16 else y
+    return _r(y, round_dtype) if round_bf16 else y
 
 
 def rotate_interleaved(x: torch.Tensor) -> torch.Tensor:
@@ -76,12 +83,12 @@ def rotate_half(x: torch.Tensor) -> torch.Tensor:
 
 
 def rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, kind: int, sections: Sequence[int] = (),
-         bf16_math: bool = False) -> torch.Tensor:
+         bf16_math: bool = False, round_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
     """x fp32 ``[B,S,H,D]``; cos/sin ``[S,D]`` or ``[B,S,D]``.  fp32 result.
 
     ``bf16_math`` follows executor/step/rope.py:30-35, where the whole expression
     ``tokens * cos + rotate_half(tokens) * sin`` runs in the tokens' dtype: both products and the
-    sum are rounded to bf16 (the sum's rounding is the caller's final cast here)."""
+    sum are rounded to that dtype (the sum's rounding is the caller's final cast here)."""
     if cos.dim() == 2:
         cos, sin = cos[None], sin[None]
     cos, sin = cos[:, :, None, :].to(torch.float32), sin[:, :, None, :].to(torch.float32)
@@ -93,7 +100,7 @@ def rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, kind: int, secti
         rot = torch.cat([rotate_half(p) for p in torch.split(x, secs, dim=-1)], dim=-1)  # rope.py:79-88
     a, b = x * cos, rot * sin
     if bf16_math:
-        a, b = _r(a), _r(b)
+        a, b = _r(a, round_dtype), _r(b, round_dtype)
     return a + b
 
 
@@ -102,14 +109,16 @@ def qk_norm_rope(x: torch.Tensor, norm: int = NORM_NONE, weight: Optional[torch.
                  cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None, rope_begin: int = 0,
                  rope_end: Optional[int] = None, sections: Sequence[int] = (), rounding: int = 0,
                  out_scale: float = 1.0) -> torch.Tensor:
-    """The whole producer step on x bf16 ``[B,S,H,D]``; returns the fp32 value BEFORE the final
-    rounding to bf16 (the caller rounds, so a test can bound the distance to the exact value).
+    """The whole producer step on x ``[B,S,H,D]`` (bf16, or fp16 for a model run in fp16); returns the fp32
+    value BEFORE the final rounding to x's dtype (the caller rounds, so a test can bound the distance to the
+    exact value).  The intermediate roundings ``rounding`` asks for are to x's dtype.
     ``out_scale`` multiplies the result (fp32) last: a caller's way of folding the softmax scale into q."""
     rn = bool(rounding & ROUND_NORM_BF16)
+    rd = _model_dtype(x)
     if norm == NORM_RMS:
-        y = rms_norm(x, weight, eps, rn)
+        y = rms_norm(x, weight, eps, rn, rd)
     elif norm == NORM_LAYER:
-        y = layer_norm(x, weight, bias, eps, rn)
+        y = layer_norm(x, weight, bias, eps, rn, rd)
     else:
         y = x.to(torch.float32)
     if rope_kind != ROPE_NONE:
@@ -118,7 +127,7 @@ def qk_norm_rope(x: torch.Tensor, norm: int = NORM_NONE, weight: Optional[torch.
         if rope_end > rope_begin:
             y = y.clone()
             y[:, rope_begin:rope_end] = rope(y[:, rope_begin:rope_end], cos, sin, rope_kind, sections,
-                                             bool(rounding & ROUND_ROPE_BF16))
+                                             bool(rounding & ROUND_ROPE_BF16), rd)
     if out_scale != 1.0:
         y = y * torch.tensor(out_scale, dtype=torch.float32)
     return y

@@ -534,12 +534,10 @@ def test_mask_mode_memory_guard_recomputes_without_arena(env):
     assert tight.cache.arena_out is None and roomy.cache.arena_out is not None
 
 
-def test_fp16_inputs_are_rounded_to_bf16_once(env):
-    """flash_attn_func takes fp16 as well as bf16; the kernels here read bf16, so fp16 tensors are rounded to bf16
-    at the kernel boundary (3 mantissa bits fewer than an fp16 flash-attn run would carry; parity with that run is
-    unpinned -- the wheel is absent and the reference holds no fp16 vectors).  What is checked: the result is the
-    attention of the ROUNDED inputs to the usual bar, and its distance to fp32 attention of the fp16 inputs stays
-    within the price of that rounding (2^-9 relative per element; the test allows 5e-3 / 5e-3)."""
+def test_fp16_inputs_run_as_fp16(env):
+    """flash_attn_func takes fp16 as well as bf16: fp16 tensors run on the fp16 MFMA with fp16 states, they are
+    not rounded to bf16 at the boundary.  The result is fp32 attention of the fp16 inputs to an fp16 pipeline's
+    accuracy (1e-3 / 2e-4 here; rounding the inputs to bf16 first would cost 5e-3).  More in test_fp16_gpu.py."""
     from ditango_amd.core.attention import proAttention
     from ditango_amd.core.parallel_state import get_usp_group
     B, H, D, S, N = 1, 2, 128, 200, 2
@@ -554,11 +552,9 @@ def test_fp16_inputs_are_rounded_to_bf16_once(env):
     out = attn.attn(q.cuda(), ks[0].cuda(), vs[0].cuda())
     torch.cuda.synchronize()
     assert out.dtype == torch.float32
-    r_out, r_lse = om.full_attention(q.bfloat16(), [k.bfloat16() for k in ks], [v.bfloat16() for v in vs])
-    _cmp(out, attn.last_lse, r_out, r_lse, "fp16 inputs vs attention of their bf16 roundings")
     f_out, f_lse = om.full_attention(q.float(), [k.float() for k in ks], [v.float() for v in vs])
     lse = attn.last_lse.cpu().squeeze(-1).transpose(1, 2)
-    assert (out.cpu() - f_out).abs().max() <= 5e-3 and (lse - f_lse).abs().max() <= 5e-3
+    assert (out.cpu() - f_out).abs().max() <= 1e-3 and (lse - f_lse).abs().max() <= 2e-4
 
 
 def test_update_out_and_lse_dropin(hip):

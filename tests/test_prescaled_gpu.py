@@ -176,7 +176,7 @@ def test_unknown_flags_and_bad_out_scale_are_rejected(hip):
                                            1, begin, chunks, None, None, None, None, outs, lses, ctypes.c_float(0.0),
                                            flags, None, 0, None)
 
-    assert call(2) == -1 and b"flags" in lib.dt_last_error()
+    assert call(4) == -1 and b"flags" in lib.dt_last_error()       # 1 and 2 are DT_ATTN_Q_PRESCALED and DT_ATTN_FP16
     torch.cuda.synchronize()
     assert (out.float() == 7.0).all()
     assert call(hip.DT_ATTN_Q_PRESCALED) == 0
