@@ -74,20 +74,20 @@ def _reference_cvx_qkv(attn, hidden_states, encoder_hidden_states, image_rotary_
     return query.transpose(1, 2).contiguous(), key.transpose(1, 2).contiguous(), value.transpose(1, 2).contiguous()
 
 
-@pytest.mark.parametrize("D,H", [(64, 6), (128, 3)])
-def test_cogvideox_processor_matches_the_reference_adapter(env, D, H):
+@pytest.mark.parametrize("D,H,dtype", [(64, 6, torch.bfloat16), (128, 3, torch.bfloat16), (64, 6, torch.float16)])
+def test_cogvideox_processor_matches_the_reference_adapter(env, D, H, dtype):
     from ditango.executor.cogvideox.attention_processor import CVX_oCacheAttnProcessor      # the reference's import path
     from ditango_amd.utils import update_timestep
     N, rank, B, C, n_text, n_video = 2, 0, 1, 192, 26, 170
     group = env(N, rank)
     torch.manual_seed(3)
-    attn = _DiffusersLikeAttention(C, H, D).cuda().bfloat16()
+    attn = _DiffusersLikeAttention(C, H, D).cuda().to(dtype)      # the model's dtype: bf16, or fp16
     with torch.no_grad():
         for ln in (attn.norm_q, attn.norm_k):            # a trained affine, not the identity
             ln.weight.add_(0.1 * torch.randn_like(ln.weight))
             ln.bias.add_(0.1 * torch.randn_like(ln.bias))
     g = torch.Generator().manual_seed(5)
-    shards = [(torch.randn(B, n_video, C, generator=g).bfloat16().cuda(), torch.randn(B, n_text, C, generator=g).bfloat16().cuda())
+    shards = [(torch.randn(B, n_video, C, generator=g).to(dtype).cuda(), torch.randn(B, n_text, C, generator=g).to(dtype).cuda())
               for _ in range(N)]
     ang = torch.rand(n_video, D // 2, generator=g) * 6.28
     rope = (ang.cos().repeat_interleave(2, -1).contiguous().cuda(), ang.sin().repeat_interleave(2, -1).contiguous().cuda())
@@ -99,8 +99,8 @@ def test_cogvideox_processor_matches_the_reference_adapter(env, D, H):
         update_timestep(0)
         hidden, enc = proc(attn, *shards[0], attention_mask=None, image_rotary_emb=rope)
         torch.cuda.synchronize()
-        assert hidden.dtype == torch.bfloat16 and tuple(hidden.shape) == (B, n_video, C) and tuple(enc.shape) == (B, n_text, C)
-        # 1. the producer: q / k / v against the reference's eager chain, to one bf16 rounding
+        assert hidden.dtype == dtype and tuple(hidden.shape) == (B, n_video, C) and tuple(enc.shape) == (B, n_text, C)
+        # 1. the producer: q / k / v against the reference's eager chain, to one rounding of the model's dtype
         q_a, k_a, v_a = proc.project_qkv(attn, *shards[0], rope)
         q_r, k_r, v_r = _reference_cvx_qkv(attn, *shards[0], rope)
         _, k1_r, v1_r = _reference_cvx_qkv(attn, *shards[1], rope)
@@ -113,7 +113,7 @@ def test_cogvideox_processor_matches_the_reference_adapter(env, D, H):
         ref_o, ref_l = om.full_attention(q_r.cpu(), [k_r.cpu(), k1_r.cpu()], [v_r.cpu(), v1_r.cpu()])
         lse = proc.oAttn.last_lse.cpu().squeeze(-1).transpose(1, 2)
         assert (lse - ref_l).abs().max() <= 5e-3          # q / k differ from the eager ones by up to one rounding
-        ref_h = ref_o.to(torch.bfloat16).cuda().reshape(B, -1, H * D)
+        ref_h = ref_o.to(dtype).cuda().reshape(B, -1, H * D)
         ref_h = attn.to_out[1](attn.to_out[0](ref_h))
         ref_enc, ref_hidden = ref_h.split([n_text, n_video], dim=1)
         for a, r, what in ((hidden, ref_hidden, "hidden_states"), (enc, ref_enc, "encoder_hidden_states")):
@@ -149,21 +149,22 @@ def test_hunyuan_processor_matches_the_varlen_oracle(env):
     assert err <= OUT_TOL and lerr <= LSE_TOL
 
 
-def test_step_attention_o_attn_func_matches_the_oracle(env):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_step_attention_o_attn_func_matches_the_oracle(env, dtype):
     from ditango.executor.step.attentions import Attention
     from ditango_amd.utils import update_timestep
     N, rank, B, H, D, S = 2, 0, 1, 4, 128, 210
     group = env(N, rank)
     g = torch.Generator().manual_seed(13)
-    q = torch.randn(B, S, H, D, generator=g).bfloat16()
-    ks = [torch.randn(B, S, H, D, generator=g).bfloat16() for _ in range(N)]
-    vs = [torch.randn(B, S, H, D, generator=g).bfloat16() for _ in range(N)]
+    q = torch.randn(B, S, H, D, generator=g).to(dtype)
+    ks = [torch.randn(B, S, H, D, generator=g).to(dtype) for _ in range(N)]
+    vs = [torch.randn(B, S, H, D, generator=g).to(dtype) for _ in range(N)]
     group.set_kv_chunks([k.cuda() for k in ks], [v.cuda() for v in vs])
     module = Attention(layer_id=0)
     update_timestep(0)
     x = module.attn_processor("oattn")(q.cuda(), ks[rank].cuda(), vs[rank].cuda())
     torch.cuda.synchronize()
-    assert x.dtype == torch.bfloat16 and tuple(x.shape) == (B, S, H, D)          # ``x.to(q.dtype)`` of :98
+    assert x.dtype == dtype and tuple(x.shape) == (B, S, H, D)                   # ``x.to(q.dtype)`` of :98
     ref_o, ref_l = om.full_attention(q, ks, vs)
     err = (x.float().cpu() - ref_o).abs().max().item()
     lerr = (module.oAttn.last_lse.cpu().squeeze(-1).transpose(1, 2) - ref_l).abs().max().item()
