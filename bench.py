@@ -503,6 +503,18 @@ def run_workload(name, args, steps, warmup, main, reuse=None, kernels_only=False
     k2_ms = time_kernel(Rotation(merge_layer, L_run * dst_n), reps)
     k2_bytes = rows * (C * (2 * D + 4) + (4 * D + 4))
     k2_gbs = k2_bytes / (k2_ms * 1e-3) / 1e9
+
+    # the reference's own use of the merge: a running fp32 (out, lse [B,S,H,1]) updated in place with one bf16 block
+    # state (utils.py:24-84 as called at core/attention.py:116,144,194,196,213), rotating over states and slots
+    def update_running(i):
+        cache = layers[i % L_run].cache
+        c = (i // L_run) % C
+        blk = (cache.arena_out[c], cache.arena_lse[c]) if c != diag else (cache.diag_out, cache.diag_lse)
+        _hip.merge_states([dst_os[i % dst_n], blk[0]], [dst_ls[i % dst_n], blk[1]], dst_out=dst_os[i % dst_n], dst_lse=dst_ls[i % dst_n])
+
+    k2u_ms = time_kernel(Rotation(update_running, L_run * C * dst_n), reps)
+    k2u_bytes = rows * ((2 * D + 4) + 2 * (4 * D + 4))
+    k2u_gbs = k2u_bytes / (k2u_ms * 1e-3) / 1e9
     k2_ws_mb = (L_run * C * state_bytes + dst_n * rows * (4 * D + 4)) / 1e6
 
     # cache store / load, over a rotation of cache slots of distinct layers and of source / destination tensors
@@ -571,7 +583,10 @@ def run_workload(name, args, steps, warmup, main, reuse=None, kernels_only=False
                       "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(k2_gbs / PEAK_HBM_GBS, 4),
                       "traffic": k2_traffic, "launch_us": round(k2_ms * 1e3, 2), "bytes_per_launch": k2_bytes,
                       "states": C, "working_set_mb": round(k2_ws_mb, 0),
-                      "read_probe_gbs": round(kr_gbs, 1), "frac_of_read_probe": round(k2_gbs / kr_gbs, 4)}
+                      "read_probe_gbs": round(kr_gbs, 1), "frac_of_read_probe": round(k2_gbs / kr_gbs, 4),
+                      "running_update": {"what": "fp32 running state updated in place with one bf16 block (update_out_and_lse as the reference calls it)",
+                                         "gbs": round(k2u_gbs, 1), "frac": round(k2u_gbs / PEAK_HBM_GBS, 4),
+                                         "launch_us": round(k2u_ms * 1e3, 2), "bytes_per_launch": k2u_bytes}}
     cache_gbs = {"store_fp32_to_slot": round(k3s_gbs, 1), "store_bf16_to_slot": round(k3c_gbs, 1),
                  "load_slot_to_fp32": round(k3l_gbs, 1), "peak": PEAK_HBM_GBS,
                  "frac_store_bf16": round(k3c_gbs / PEAK_HBM_GBS, 4), "frac_load": round(k3l_gbs / PEAK_HBM_GBS, 4),

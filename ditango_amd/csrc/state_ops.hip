@@ -18,7 +18,8 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kThreads = 256;
-constexpr int kBatch = 8;  // states whose loads are in flight together
+constexpr int kBatch = 8;       // states whose loads are in flight together (all states in one 16-bit type)
+constexpr int kBatchMixed = 4;  // ... when the launch mixes fp32 with 16-bit states
 
 struct MergeArgs {
   int32_t n;
@@ -375,7 +376,11 @@ static bool unit_tiles_fit(int H, int D) { return H % ((128 / D) * kTileHeadUnit
 
 // FAST: 1 = every state bfloat16, 2 = every state IEEE half (one decode, no per-state dtype); mixed dtypes:
 // 3 = bfloat16 and fp32 only, 0 = any of the three.
-template <int D, int FAST, int MAP, int P>
+// KB: states per batch.  A mixed-dtype batch holds twice the bytes per state and pass of a 16-bit one; in batches of
+// 8 that is 106 registers and 4 resident wavefronts per SIMD (against 70 and 7), in batches of 4 again 70 and 7 --
+// and 5.8 instead of 4.3 TB/s on an fp32 running state merged with four bf16 blocks at the HunyuanVideo share (the
+// running-state update of utils.py:24-40 as the reference calls it, two states: 5.7 instead of 4.9 TB/s).
+template <int D, int FAST, int MAP, int P, int KB>
 __global__ __launch_bounds__(kThreads) void merge_states_kernel(const MergeArgs a) {
   constexpr int R = 128 / D;
   const int cc = threadIdx.x % kUnitLanes;
@@ -393,8 +398,8 @@ __global__ __launch_bounds__(kThreads) void merge_states_kernel(const MergeArgs 
     for (int k = 0; k < 8; ++k) ua[p].acc[k] = 0.f;
   }
   int i0 = 0;
-  for (; i0 + kBatch <= a.n; i0 += kBatch) unit_batch<R, kBatch, FAST, P>(a, i0, u, cc, ua);
-  unit_rest<R, FAST, kBatch - 1, P>(a, i0, a.n - i0, u, cc, ua);
+  for (; i0 + KB <= a.n; i0 += KB) unit_batch<R, KB, FAST, P>(a, i0, u, cc, ua);
+  unit_rest<R, FAST, KB - 1, P>(a, i0, a.n - i0, u, cc, ua);
   constexpr int kPer = 8 / R;
 #pragma unroll
   for (int p = 0; p < P; ++p) {
@@ -750,10 +755,11 @@ constexpr int64_t kTwoPassUnits = 1 << 20;
 template <int D, int MAP, int P>
 static void launch_merge_k(const MergeArgs& a, unsigned wgs, hipStream_t stream) {
   const uint64_t all = a.n >= 64 ? ~0ull : ((1ull << a.n) - 1);
-  if (a.fp32_mask == 0 && a.f16_mask == 0) hipLaunchKernelGGL((merge_states_kernel<D, 1, MAP, P>), dim3(wgs), dim3(kThreads), 0, stream, a);
-  else if (a.f16_mask == all) hipLaunchKernelGGL((merge_states_kernel<D, 2, MAP, P>), dim3(wgs), dim3(kThreads), 0, stream, a);
-  else if (a.f16_mask == 0) hipLaunchKernelGGL((merge_states_kernel<D, 3, MAP, P>), dim3(wgs), dim3(kThreads), 0, stream, a);
-  else hipLaunchKernelGGL((merge_states_kernel<D, 0, MAP, P>), dim3(wgs), dim3(kThreads), 0, stream, a);
+  const dim3 grid(wgs), block(kThreads);
+  if (a.fp32_mask == 0 && a.f16_mask == 0) hipLaunchKernelGGL((merge_states_kernel<D, 1, MAP, P, kBatch>), grid, block, 0, stream, a);
+  else if (a.f16_mask == all) hipLaunchKernelGGL((merge_states_kernel<D, 2, MAP, P, kBatch>), grid, block, 0, stream, a);
+  else if (a.f16_mask == 0) hipLaunchKernelGGL((merge_states_kernel<D, 3, MAP, P, kBatchMixed>), grid, block, 0, stream, a);
+  else hipLaunchKernelGGL((merge_states_kernel<D, 0, MAP, P, kBatchMixed>), grid, block, 0, stream, a);
 }
 
 template <int D>
