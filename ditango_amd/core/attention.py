@@ -2,7 +2,7 @@
 
 API of the reference's ``proAttention`` (core/attention.py:20-419):
 ``proAttention(layer_id, isp_group).attn(query, key, value)`` with inputs
-``[B, S, H, D]`` bf16 and an fp32 result of the same shape.
+``[B, S, H, D]`` bf16 (or fp16) and an fp32 result of the same shape.
 
 One GPU plays one sequence-parallel rank.  Where the reference interleaves ring
 hops, one ``flash_attn_func`` call per chunk and one eager merge chain per state,

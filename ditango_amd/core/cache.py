@@ -1,7 +1,7 @@
 """HBM-resident cache of attention states, one per transformer layer.
 
 API of the reference's ``proCache`` (core/cache.py:9-128).  A cached state is
-``(out bf16 [B,Sq,H,D], lse fp32 [B,H,Sq])`` in device memory -- half the bytes
+``(out bf16 [B,Sq,H,D] -- fp16 for a model run in fp16 --, lse fp32 [B,H,Sq])`` in device memory -- half the bytes
 of the fp32 states the reference keeps -- written by the attention kernel itself
 and read exactly once per reuse by the fused merge kernel.
 

@@ -9,7 +9,7 @@ The reference's executors run these as chains of eager torch ops right before
 * Step-Video  ``executor/step/blocks.py:66-75`` + ``executor/step/rope.py:13-90``  RMSNorm, rotate-half RoPE
   on the sections ``[64, 32, 32]`` of D.
 
-``prepare_qk`` does the whole chain in one launch of ``dt_qk_norm_rope`` and writes the bf16
+``prepare_qk`` does the whole chain in one launch of ``dt_qk_norm_rope`` and writes the bf16 (or fp16)
 ``[B,S,H,D]`` tensor the attention kernels read.  There is no non-HIP fallback.
 """
 from __future__ import annotations
@@ -39,8 +39,9 @@ def prepare_qk(x: torch.Tensor, *, norm: Optional[str] = None, weight: Optional[
                rope_end: Optional[int] = None, sections: Sequence[int] = (), match_eager_rounding: bool = False,
                bf16_rope_math: bool = False, out: Optional[torch.Tensor] = None,
                fold_softmax_scale: Optional[float] = None) -> torch.Tensor:
-    """x: bf16 ``[B,S,H,D]`` view (e.g. a slice of a fused QKV projection; only the last dimension
-    must be contiguous).  Returns bf16 ``[B,S,H,D]`` contiguous.
+    """x: bf16 (or fp16: a model run in fp16) ``[B,S,H,D]`` view (e.g. a slice of a fused QKV projection; only
+    the last dimension must be contiguous).  Returns ``[B,S,H,D]`` contiguous in x's dtype; where "bf16" is said
+    below, an fp16 x reads "fp16".
 
     norm: ``"rms"`` | ``"layer_norm"`` | None, with ``weight`` / ``bias`` of shape ``[D]`` (any float dtype).
     rope: ``"interleaved"`` (pairs ``(2i, 2i+1)``; CogVideoX, HunyuanVideo) | ``"rotate_half"`` (Step-Video,
