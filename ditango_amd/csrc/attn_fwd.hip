@@ -100,9 +100,7 @@ constexpr int kBK = 64;           // keys per tile
 constexpr int kXcds = 8;
 constexpr int kNumBuf = DT_SCHED_NUM_BUF;  // LDS buffers per operand; a tile uses buffer (tile & 3)
 static_assert(kNumBuf == 4, "buffer indices are computed with & 3 and the loop is unrolled by four");
-#ifndef DT_RING
-#define DT_RING 4
-#endif
+constexpr int kRingDepth = 4;     // operand fragments the LDS reads of a matrix phase run ahead of its MFMAs (2 and 6 measured: no gain)
 // Row permutation of the K operand: MFMA row i -> key (within a 32-key half tile).
 __device__ __forceinline__ int key_of_row(int i) {
   return (i & 19) | ((i & 4) << 1) | ((i & 8) >> 1);
@@ -267,11 +265,9 @@ __device__ __forceinline__ void load_block_to_lds(u32x4 rsrc, uint32_t lane_off,
 // tiles fill the CU).  D = 64: four, i.e. TWO workgroups per CU (64 KB of LDS and at most 128
 // registers each): the second workgroup's wavefronts issue into the barrier waits, the start-up and
 // the epilogue of the first, which at 35 key tiles per work item are a tenth of its time (+10 %).
-#ifndef DT_D64_WAVES
-#define DT_D64_WAVES 4
-#endif
+constexpr int kWavesPerSimdD64 = 4;
 template <int D, bool kPre, bool kHalf>
-__global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd_kernel(const AttnArgs args_by_value) {
+__global__ __launch_bounds__(kThreads, D == 64 ? kWavesPerSimdD64 : 2) void attn_fwd_kernel(const AttnArgs args_by_value) {
   using T = Tile<D>;
   using E = Elem<kHalf>;
   typedef typename E::t elem_t;
@@ -597,7 +593,7 @@ __global__ __launch_bounds__(kThreads, D == 64 ? DT_D64_WAVES : 2) void attn_fwd
   constexpr int kPV = D / 32 * 4;       // fragments of the P V product
   constexpr int kQK = 2 * (D / 16);     // fragments of the score product
   constexpr int kFrags = kPV + kQK;
-  constexpr int kRing = DT_RING;
+  constexpr int kRing = kRingDepth;
   // Where a wavefront issues its tile loads: at the start of its vector phase, or behind the
   // MFMAs of its matrix phase (one phase later, and then awaited one call earlier).  At D = 64
   // the vector phase is the longer one (half the MFMAs per softmax element) and the matrix
