@@ -142,7 +142,7 @@ def test_jobs_with_tail_split_and_fold_in_fp16(hip, D, lens):
 
 
 @pytest.mark.parametrize("D", [64, 128])
-@pytest.mark.parametrize("n,kinds", [(3, "hhh"), (9, "hhhhhhhhh"), (5, "hbfhb"), (2, "fh")])
+@pytest.mark.parametrize("n,kinds", [(3, "hhh"), (6, "hhhhhh"), (9, "hhhhhhhhh"), (5, "hbfhb"), (2, "fh")])
 @pytest.mark.parametrize("dst", [torch.float32, torch.float16])
 def test_merge_of_fp16_states_matches_closed_form(hip, D, n, kinds, dst):
     """All-fp16 launches (their own decode path), and fp16 mixed with bf16 and fp32 states; fp32 and fp16 results."""

@@ -142,7 +142,7 @@ def test_multi_chunk_job_equals_merge_of_chunks(hip):
 
 
 @pytest.mark.parametrize("D,n,src_fp32", [(128, 1, False), (128, 5, False), (64, 8, False), (128, 3, True), (64, 33, False),
-                                          (128, 6, False), (128, 7, True), (64, 9, True)])
+                                          (128, 6, False), (128, 7, True), (64, 9, True), (64, 4, False), (64, 7, False), (128, 8, False)])
 def test_merge_states_matches_closed_form(hip, D, n, src_fp32):
     B, Sq, H = 2, 150, 3
     g = torch.Generator().manual_seed(n * 7 + D)
