@@ -744,12 +744,12 @@ __global__ __launch_bounds__(kThreads) void zero_rows_from_kernel(u32x4* dst, in
 // ---- host-side launchers ---------------------------------------------------------------
 
 // Which mapping and how many passes a launch gets (A/B on one box, states rotating through HBM; TB/s):
-//   * D = 128, up to 5 states: linear, one pass (2 states 6.3 against 6.2 tiled; two passes 5.2-5.6);
-//   * D = 128, 6 states and more: tiled, two passes (8 states 6.52-6.56 against 6.43 linear; 32 states of
-//     743 MB 5.88 against 5.74 with one pass);
-//   * D = 64: tiled; one pass while the launch is small (8 states of 14 MB: 5.6 against 5.2 with two
+//   * tiled wherever the tiles fit the head count (D = 128: 3 states 6.28 against 6.10 linear, 5 states 6.41
+//     against 6.24, 8 states 6.52-6.56 against 6.43);
+//   * D = 128: two passes from a full batch of states on (8 states 6.46 against 6.41 with one pass, 32 states
+//     of 743 MB 5.88 against 5.74), one pass below (3 states 6.28 against 5.84 with two);
+//   * D = 64: one pass while the launch is small (8 states of 14 MB: 5.6 against 5.2 with two
 //     passes -- finer workgroups fill the last round of the chip better), two passes on large ones.
-constexpr int kTiledFrom = 6;
 constexpr int64_t kTwoPassUnits = 1 << 20;
 
 template <int D, int MAP, int P>
@@ -789,10 +789,10 @@ int launch_merge(const MergeArgs& a, int D, hipStream_t stream) {
   }
   const int R = 128 / D;   // rows per unit
   const int64_t units = ((int64_t)a.B * a.Sq * a.H + R - 1) / R;
-  const bool tiled = (D == 64 || a.n >= kTiledFrom) && unit_tiles_fit(a.H, D);
+  const bool tiled = unit_tiles_fit(a.H, D);
   int passes;
   if (D == 64) passes = units >= kTwoPassUnits ? 2 : 1;
-  else passes = a.n >= kTiledFrom ? 2 : 1;
+  else passes = a.n >= kBatch ? 2 : 1;
   const int64_t wgs = unit_grid(a.B, a.Sq, a.H, D, tiled, passes);
   if (wgs <= 0) return DT_OK;
   if (wgs > 0x7fffffffLL) {
