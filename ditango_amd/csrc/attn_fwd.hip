@@ -260,6 +260,21 @@ __device__ __forceinline__ void load_block_to_lds(u32x4 rsrc, uint32_t lane_off,
                  "s"(__builtin_amdgcn_readfirstlane(lds_addr))
                : "memory", "m0");
 }
+// The wavefront's next 1 KB block of the same tile: same M0, the instruction's immediate offset moves both the LDS
+// address and the global address on by 1 KB (lane_off is reduced by as much where the global side should not move).
+// Rewriting M0 between two such loads costs about 17 cycles each time: the write waits until the load before it
+// has read the register.
+__device__ __forceinline__ void load_next_block_to_lds(u32x4 rsrc, uint32_t lane_off, uint32_t uniform_off) {
+  u32x4 r;
+  r.x = __builtin_amdgcn_readfirstlane(rsrc.x);
+  r.y = __builtin_amdgcn_readfirstlane(rsrc.y);
+  r.z = __builtin_amdgcn_readfirstlane(rsrc.z);
+  r.w = __builtin_amdgcn_readfirstlane(rsrc.w);
+  asm volatile("buffer_load_dwordx4 %0, %1, %2 offen offset:1024 lds"
+               :
+               : "v"(lane_off), "s"(r), "s"(__builtin_amdgcn_readfirstlane(uniform_off))
+               : "memory");
+}
 
 // Wavefronts per SIMD the register budget is set for.  D = 128: two (one workgroup per CU: its LDS
 // tiles fill the CU).  D = 64: four, i.e. TWO workgroups per CU (64 KB of LDS and at most 128
@@ -482,8 +497,9 @@ __global__ __launch_bounds__(kThreads, D == 64 ? kWavesPerSimdD64 : 2) void attn
   }
 
   // ---- tile loads: global memory -> LDS without passing through registers ---------------
-  // A wavefront brings in kLoads 1 KB blocks of every K tile and of every V tile (block
-  // wave + 8 i = rows kRowsPerBlock * (wave + 8 i) ...).  Lane L of a load lands at LDS bytes
+  // A wavefront brings in kLoads consecutive 1 KB blocks of every K tile and of every V tile (blocks
+  // kLoads * wave + i = rows kRowsPerBlock * (kLoads * wave + i) ...; consecutive, so that one M0 value serves
+  // all of them).  Lane L of a load lands at LDS bytes
   // 16 L .. 16 L + 15 of the block, i.e. at row L / kChunks, chunk position L % kChunks; it
   // therefore fetches the chunk of global memory that the swizzle assigns to that position.
   // Raw buffer loads: the descriptor (base of the chunk's first key for this batch and head,
@@ -491,17 +507,19 @@ __global__ __launch_bounds__(kThreads, D == 64 ? kWavesPerSimdD64 : 2) void attn
   // load's scalar offset (which the range check includes), and rows past the end of the chunk fail
   // the hardware bounds check and arrive as zeros (their scores are masked to -inf; zero V rows
   // add nothing).
-  uint32_t k_goff, v_goff;  // this lane's byte offset from the tile's first key, loop invariant
-  {
-    const int lrow = T::kRowsPerBlock * wave + lane / T::kChunks;  // + 8 * kRowsPerBlock * i
+  // this lane's byte offset from the tile's first key for its i-th block, loop invariant; less the 1 KB per block
+  // that the immediate offset of load_next_block_to_lds adds back (a block's rows start at least that far in)
+  uint32_t k_goff[T::kLoads], v_goff[T::kLoads];
+#pragma unroll
+  for (int i = 0; i < T::kLoads; ++i) {
+    const int lrow = T::kRowsPerBlock * (T::kLoads * wave + i) + lane / T::kChunks;
     const int pos = lane % T::kChunks;
-    k_goff = (uint32_t)lrow * row_bytes + 16u * (uint32_t)(pos ^ T::swz_k(lrow));
-    v_goff = (uint32_t)lrow * row_bytes + 16u * (uint32_t)((((pos >> 2) ^ T::swz_v(lrow)) << 2) | (pos & 3));
+    k_goff[i] = (uint32_t)lrow * row_bytes + 16u * (uint32_t)(pos ^ T::swz_k(lrow)) - 1024u * i;
+    v_goff[i] = (uint32_t)lrow * row_bytes + 16u * (uint32_t)((((pos >> 2) ^ T::swz_v(lrow)) << 2) | (pos & 3)) - 1024u * i;
   }
-  static_assert((8 * T::kRowsPerBlock) % 16 == 0, "the swizzle must not depend on the load index");
+  static_assert(T::kLoads <= 2 && T::kRowsPerBlock * T::kRowBytes == 1024, "one immediate offset of 1 KB, whole rows per block");
   typedef __attribute__((address_space(3))) uint8_t* lds_ptr_t;
   const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
-  const uint32_t block_step = (uint32_t)(8 * T::kRowsPerBlock) * row_bytes;   // from a wavefront's block to its next one
   // Issues this wavefront's loads of V of the tile before the one under the load cursor and of
   // K of the tile under it (tile X, into K buffer X & 3; V is needed two phases later than K, so
   // its loads run one tile behind), and moves the cursor on.  Past the last tile the loads are still
@@ -514,19 +532,20 @@ __global__ __launch_bounds__(kThreads, D == 64 ? kWavesPerSimdD64 : 2) void attn
   bool v_lags = true;
   auto load_tile = [&](int kbuf) __attribute__((always_inline)) {
     const int vbuf = (kbuf + kNumBuf - 1) & (kNumBuf - 1);
-    const uint32_t kdst = lds_base + kbuf * T::kBytesK + wave * 1024;
-    const uint32_t vdst = lds_base + T::kOffV + vbuf * T::kBytesV + wave * 1024;
+    const uint32_t kdst = lds_base + kbuf * T::kBytesK + wave * (1024 * T::kLoads);
+    const uint32_t vdst = lds_base + T::kOffV + vbuf * T::kBytesV + wave * (1024 * T::kLoads);
+    auto load_blocks = [&](const u32x4& rsrc, const uint32_t (&goff)[T::kLoads], uint32_t off, uint32_t dst) __attribute__((always_inline)) {
+      load_block_to_lds(rsrc, goff[0], off, dst);
+      if constexpr (T::kLoads == 2) load_next_block_to_lds(rsrc, goff[1], off);
+    };
     // V first: the barrier waits let the K half of a call stay in flight one vector phase longer
     if (__builtin_expect(v_lags, 0)) {
-#pragma unroll
-      for (int i = 0; i < T::kLoads; ++i) load_block_to_lds(rv_old, v_goff, v_off + i * block_step, vdst + i * 8192);
+      load_blocks(rv_old, v_goff, v_off, vdst);
       v_lags = false;
     } else {
-#pragma unroll
-      for (int i = 0; i < T::kLoads; ++i) load_block_to_lds(rv, v_goff, v_off + i * block_step, vdst + i * 8192);
+      load_blocks(rv, v_goff, v_off, vdst);
     }
-#pragma unroll
-    for (int i = 0; i < T::kLoads; ++i) load_block_to_lds(rk, k_goff, k_off + i * block_step, kdst + i * 8192);
+    load_blocks(rk, k_goff, k_off, kdst);
     v_off = k_off;
     k_off += tile_bytes;
     ld_left -= kBK;
