@@ -111,16 +111,34 @@ class Rotation:
         self.k += 1
 
 
-def sample_clock_mhz(fn, seconds=2.0):
-    """Shader clock (MHz) read with ``rocm-smi`` while ``fn`` keeps the GPU busy; None if it cannot be read."""
-    samples, stop = [], [False]
+def _hwmon_watts(name):
+    """The first readable ``power1_<name>`` of a GPU's hwmon node, in W (the files hold microwatts), or None."""
+    import glob
+    for path in sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_" + name)):
+        try:
+            with open(path) as f:
+                return int(f.read().strip()) / 1e6
+        except (OSError, ValueError):
+            continue
+    return None
+
+
+def sample_clock_and_power(fn, seconds=2.0):
+    """(shader clock in MHz from ``rocm-smi``, package power in W from the GPU's hwmon node) while ``fn`` keeps the
+    GPU busy; None for what cannot be read."""
+    clocks, watts, stop = [], [], [False]
 
     def sampler():
         while not stop[0]:
             try:
+                w = _hwmon_watts("input")
+                if w is None:
+                    w = _hwmon_watts("average")
+                if w is not None:
+                    watts.append((time.perf_counter(), w))
                 r = subprocess.run(["rocm-smi", "--showclocks", "--json"], capture_output=True, text=True, timeout=10)
-                card = list(json.loads(r.stdout).values())[0]
-                samples.append((time.perf_counter(), float(card["sclk clock speed:"].strip("()Mhz"))))
+                card = list(json.loads(r.stdout[r.stdout.index("{"):]).values())[0]
+                clocks.append((time.perf_counter(), float(card["sclk clock speed:"].strip("()Mhz"))))
             except Exception:
                 pass
             time.sleep(0.1)
@@ -135,8 +153,20 @@ def sample_clock_mhz(fn, seconds=2.0):
         torch.cuda.synchronize()
     stop[0] = True
     th.join(timeout=15)
-    vals = [v for ts, v in samples if ts - t0 > 0.5]   # after the ramp
-    return round(sum(vals) / len(vals), 0) if vals else None
+
+    def mean(samples):
+        vals = [v for ts, v in samples if ts - t0 > 0.5]   # after the ramp
+        return round(sum(vals) / len(vals), 0) if vals else None
+    return mean(clocks), mean(watts)
+
+
+def sample_clock_mhz(fn, seconds=2.0):
+    return sample_clock_and_power(fn, seconds)[0]
+
+
+def power_cap_w():
+    """The package power limit of the GPU's hwmon node in W, or None."""
+    return _hwmon_watts("cap")
 
 
 def stratified_order(counts):
@@ -454,10 +484,10 @@ def run_workload(name, args, steps, warmup, main, reuse=None, kernels_only=False
     k1h_ms = time_kernel(lambda: _hip.attn_jobs_fwd(qh, table_h, [[c] for c in range(n_typ)], sth, st_lses[:n_typ], workspace=k1_ws), reps)
     k1h_tflops = k1_flops(n_typ) / (k1h_ms * 1e-3) / 1e12
     del qh, ksh, vsh, table_h, sth
-    clock = None
+    clock = watts = None
     mfma_probe = None
     if main and not kernels_only:
-        clock = sample_clock_mhz(lambda: k1_launch(n_typ))
+        clock, watts = sample_clock_and_power(lambda: k1_launch(n_typ))
         # the yardstick: back-to-back MFMAs on registers in the same launch shape, sized to last about as long
         # as the typical launch -- what the power limit leaves of the nominal peak when only the matrix pipes work
         probe_sink = torch.zeros(1, dtype=torch.float32, device=dev)
@@ -468,8 +498,9 @@ def run_workload(name, args, steps, warmup, main, reuse=None, kernels_only=False
             probe_flops[0] = bench_probes.mfma_probe(probe_wgs, probe_iters, probe_sink)
 
         kp_ms = time_kernel(probe_launch, reps)
+        probe_clock, probe_watts = sample_clock_and_power(probe_launch, seconds=1.5)
         mfma_probe = {"tflops": round(probe_flops[0] / (kp_ms * 1e-3) / 1e12, 1), "launch_ms": round(kp_ms, 4),
-                      "clock_mhz_under_load": sample_clock_mhz(probe_launch, seconds=1.5)}
+                      "clock_mhz_under_load": probe_clock, "power_w_under_load": probe_watts}
     del q_folded
     # the co-issue yardstick: one wavefront of each SIMD issues MFMAs, the other the softmax's vector instructions
     # per MFMA at this head dimension; the MFMA rate with the softmax against the rate without is the ceiling of the
@@ -572,9 +603,14 @@ def run_workload(name, args, steps, warmup, main, reuse=None, kernels_only=False
         # the part is power-limited under this kernel: what the kernel reaches of the peak AT THE CLOCK IT RUNS AT
         roofline["clock_mhz_under_load"] = clock
         roofline["frac_at_clock"] = round(frac * NOMINAL_CLOCK_MHZ / clock, 4)
+    if watts:
+        roofline["power_w_under_load"] = watts
+        roofline["power_cap_w"] = power_cap_w()
     if mfma_probe:
         roofline["mfma_probe_tflops"] = mfma_probe["tflops"]
         roofline["mfma_probe_clock_mhz"] = mfma_probe["clock_mhz_under_load"]
+        if mfma_probe["power_w_under_load"]:
+            roofline["mfma_probe_power_w"] = mfma_probe["power_w_under_load"]
         roofline["frac_of_mfma_probe"] = round(k1_tflops / mfma_probe["tflops"], 4)
     if coissue:
         roofline["coissue_probe"] = coissue
