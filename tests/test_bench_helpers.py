@@ -55,3 +55,20 @@ def test_rotation_cycles_through_its_argument_sets():
     for _ in range(7):
         r()
     assert seen == [0, 1, 2, 0, 1, 2, 0]
+
+
+def test_power_readings_come_from_the_hwmon_files_in_watts(tmp_path, monkeypatch):
+    """bench.py reads the package power and its cap from the GPU's hwmon node (microwatts); a box without the
+    files yields None, never an exception."""
+    bench = _bench()
+    import glob as glob_module
+    node = tmp_path / "card0" / "device" / "hwmon" / "hwmon3"
+    node.mkdir(parents=True)
+    (node / "power1_input").write_text("1357000000\n")
+    (node / "power1_cap").write_text("1400000000\n")
+    real_glob = glob_module.glob
+    monkeypatch.setattr(glob_module, "glob", lambda pat: real_glob(pat.replace("/sys/class/drm", str(tmp_path))))
+    assert bench._hwmon_watts("input") == 1357.0 and bench.power_cap_w() == 1400.0
+    assert bench._hwmon_watts("average") is None
+    (node / "power1_input").write_text("not a number\n")
+    assert bench._hwmon_watts("input") is None
